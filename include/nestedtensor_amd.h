@@ -1,0 +1,157 @@
+/*
+ * nestedtensor_amd -- C ABI of the MI355X (gfx950) ragged hot path.
+ *
+ * The reference (pytorch/nestedtensor) has no C ABI: its device code is reached
+ * through C++ templates `*_kernelLauncher<T>(ptrs, int metadata..., cudaStream_t)`
+ * (nestedtensor/csrc/cuda/padding.h:12-45, cuda/attention.h:25-51) called from
+ * the operator layer (nestedtensor/csrc/masking.cpp, csrc/cuda/mha.cpp).  The
+ * entry points below are the plain-C surface those call sites would bind
+ * instead.  Each one cites the reference interface it replaces.
+ *
+ * Conventions
+ *  - all pointers are device pointers unless a parameter is named `*_host`;
+ *  - a nested tensor of nested_dim 1 is (packed buffer, sizes[B, D] int64,
+ *    offsets[B + 1] int64); offsets are ELEMENT offsets into the packed buffer;
+ *  - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *  - functions enqueue work on `stream` and return; they never allocate device
+ *    memory, never synchronise and never throw.  Scratch memory, where needed,
+ *    is passed in as `workspace` with the size the matching `*_workspace_bytes`
+ *    function reports;
+ *  - return value: NT_OK or an NT_ERR_* code; nt_last_error() gives the text
+ *    for the calling thread.
+ */
+#ifndef NESTEDTENSOR_AMD_H
+#define NESTEDTENSOR_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NT_ABI_VERSION 1
+
+enum {
+  NT_OK = 0,
+  NT_ERR_INVALID_ARGUMENT = 1,
+  NT_ERR_UNSUPPORTED = 2,
+  NT_ERR_HIP = 3,
+  NT_ERR_WORKSPACE = 4
+};
+
+/* element types of the attention path */
+enum { NT_F32 = 0, NT_F16 = 1, NT_BF16 = 2 };
+
+/* No reference counterpart: ABI handshake and error text. */
+int nt_abi_version(void);
+const char* nt_last_error(void);
+
+/* ---- metadata: device prefix scan ------------------------------------- */
+
+/* offsets[0] = 0, offsets[b + 1] = offsets[b] + prod_k sizes[b, k] for b < B.
+ * Replaces the host loop batch_offsets_from_efficient_size
+ * (nestedtensor/csrc/masking.cpp:110-125) and the unused int32 Blelloch scan
+ * exclusiveScan_kernelLauncher (nestedtensor/csrc/cuda/cuda_kernels.cu:271-517).
+ * D == 0 gives prod = 1 (0-d constituents). */
+size_t nt_offsets_workspace_bytes(int64_t B);
+int nt_offsets_from_sizes(const int64_t* sizes, int64_t B, int64_t D,
+                          int64_t* offsets, void* workspace, size_t workspace_bytes,
+                          void* stream);
+
+/* ---- packed <-> padded ------------------------------------------------- */
+
+/* padded[b, i_1..i_D] = inside(sizes[b]) ? packed[offsets[b] + lin(i)] : pad
+ * with padded of shape [B, padded_sizes_host[0..D)] (the batch maxima).
+ * `n_ragged` (1..3) leading constituent dims may differ between constituents;
+ * the trailing D - n_ragged dims must equal padded_sizes_host[k] for every b.
+ * `elem_bytes` in {1, 2, 4, 8}; `pad_bits` is the padding value already
+ * converted to the element type, in the low elem_bytes bytes.
+ * Replaces add_padding_kernelLauncher<T> (nestedtensor/csrc/cuda/padding.h:12-23,
+ * kernels padding.cu:10-193) as called by to_padded_tensor
+ * (nestedtensor/csrc/masking.cpp:558-625). */
+int nt_add_padding(const void* packed, void* padded, const int64_t* offsets,
+                   const int64_t* sizes, int64_t B, int64_t D, int64_t n_ragged,
+                   const int64_t* padded_sizes_host, int elem_bytes, uint64_t pad_bits,
+                   void* stream);
+
+/* packed[offsets[b] + lin(i)] = padded[b, i] for i inside sizes[b]: the
+ * length-based inverse of nt_add_padding.  Replaces
+ * remove_padding_kernelLauncher<T> (nestedtensor/csrc/cuda/padding.h:36-45,
+ * kernels padding.cu:286-394) as called by from_padded_tensor
+ * (nestedtensor/csrc/masking.cpp:459-509). */
+int nt_remove_padding(const void* padded, void* packed, const int64_t* offsets,
+                      const int64_t* sizes, int64_t B, int64_t D, int64_t n_ragged,
+                      const int64_t* padded_sizes_host, int elem_bytes, void* stream);
+
+/* mask[b, i_1..i_K] = all_k(i_k < sizes[b, k]) as bytes 0/1, shape
+ * [B, mask_sizes_host[0..K)], K <= D, K in 1..3.  Together with nt_add_padding
+ * (pad 0) this is to_tensor_mask; alone it is to_mask.  Replaces
+ * add_padding_mask_kernelLauncher<T> (nestedtensor/csrc/cuda/padding.h:25-34,
+ * kernel padding.cu:217-262: one thread per batch entry) and the host fill
+ * loops of to_mask (nestedtensor/csrc/masking.cpp:436-451, 353-406). */
+int nt_build_mask(uint8_t* mask, const int64_t* sizes, int64_t B, int64_t D, int64_t K,
+                  const int64_t* mask_sizes_host, void* stream);
+
+/* Gather B contiguous device tensors into one packed buffer:
+ * packed[offsets[b] .. offsets[b+1]) = *srcs[b].  `srcs` is a device array of
+ * B device pointers.  Replaces the per-constituent copy_ loop of impl::pack
+ * (nestedtensor/csrc/storage/Packed.h:75-98). */
+int nt_pack(const void* const* srcs, void* packed, const int64_t* offsets, int64_t B,
+            int elem_bytes, void* stream);
+
+/* ---- mask -> nested size, compaction ----------------------------------- */
+
+/* Row statistics of a byte mask viewed as [R, M] (nonzero = true):
+ * counts[r] = number of true entries in row r (int32).  One wavefront per row
+ * with ballot + popcount.  The reference has no device counterpart: it reads
+ * every mask element with .item<bool>() on the host
+ * (nestedtensor/csrc/masking.cpp:190-201). */
+int nt_mask_row_counts(const uint8_t* mask, int64_t R, int64_t M, int32_t* counts,
+                       void* stream);
+
+/* Compaction of the rows of `data` viewed as [R, M, chunk_bytes]: the kept
+ * chunks of row r (mask[r, m] != 0) are written, in order, starting at byte
+ * out + row_offsets[r] * chunk_bytes, where row_offsets is the exclusive scan
+ * of counts (nt_exclusive_scan_i32).  Replaces the recursive host walk of
+ * nt_from_tensor_mask (nestedtensor/csrc/masking.cpp:181-249). */
+int nt_compact_rows(const void* data, const uint8_t* mask, const int64_t* row_offsets,
+                    int64_t R, int64_t M, int64_t chunk_bytes, void* out, void* stream);
+
+/* out[0] = 0, out[i + 1] = out[i] + in[i] (int32 in, int64 out, n + 1 outputs). */
+size_t nt_scan_workspace_bytes(int64_t n);
+int nt_exclusive_scan_i32(const int32_t* in, int64_t n, int64_t* out, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
+/* ---- nested multi-head attention --------------------------------------- */
+
+/* C[M, N] = A[M, K] * W[N, K]^T + bias[N] (bias may be NULL); row-major, A with
+ * row stride lda, C with row stride ldc (elements).  fp32 accumulation.
+ * This is the packed projection of the reference: NestedTensor_matmul's
+ * single GEMM on buffer.reshape(-1, E) (nestedtensor/csrc/matmul.cpp:13-41)
+ * plus the packed bias add (nestedtensor/csrc/BinaryOps.cpp:97-107); call sites
+ * nestedtensor/csrc/mha.cpp:42-54,66-67 and csrc/cuda/mha.cpp:57,106. */
+int nt_linear(const void* A, int64_t lda, const void* W, const void* bias, void* C,
+              int64_t ldc, int64_t M, int64_t N, int64_t K, int dtype, void* stream);
+
+/* Self/cross attention on packed projections, one softmax per (sequence, head)
+ * over that sequence's own keys only:
+ *   out[q_off[b] + i, h*hd + d] = sum_j softmax_j(scale * q_i . k_j) v_j[d]
+ * q rows are q[(q_off[b] + i) * ldq + h*hd ...], k/v likewise with kv_off.
+ * head_dim must be 64 for f16/bf16.  Replaces the padded chain of bt_min_mha
+ * (nestedtensor/csrc/cuda/mha.cpp:59-105: to_padded_tensor, batched QK^T,
+ * softmax_kernel_kernelLauncher of cuda/attention.h:25-33, PV,
+ * from_padded_tensor) and the unwired add_QKV_bias_padding /
+ * transpose_rm_padding kernels (nestedtensor/csrc/cuda/attention.cu:107-174,
+ * 488-538); semantics are those of the per-sequence loop of min_mha
+ * (nestedtensor/csrc/mha.cpp:58-65). */
+int nt_varlen_attention(const void* q, int64_t ldq, const void* k, int64_t ldk,
+                        const void* v, int64_t ldv, void* out, int64_t ldo,
+                        const int64_t* q_offsets, const int64_t* kv_offsets, int64_t B,
+                        int64_t num_heads, int64_t head_dim, int64_t max_q_len,
+                        float scale, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NESTEDTENSOR_AMD_H */

@@ -1,0 +1,51 @@
+// Shared helpers of the nestedtensor_amd HIP library (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/nestedtensor_amd.h"
+
+namespace nt {
+
+constexpr int kWave = 64;
+
+// Error text of the calling thread, returned by nt_last_error().
+char* error_buffer();
+
+inline int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(error_buffer(), 512, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    return fail(NT_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+  }
+  return NT_OK;
+}
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// 16-byte load from an address of any alignment (gfx950 runs with unaligned
+// access mode; the compiler emits one global_load_dwordx4).
+__device__ __forceinline__ u32x4 load16_unaligned(const char* p) {
+  u32x4 v;
+  __builtin_memcpy(&v, p, 16);
+  return v;
+}
+
+__device__ __forceinline__ void store16(char* p, u32x4 v) {
+  *reinterpret_cast<u32x4*>(p) = v;
+}
+
+__device__ __forceinline__ void store16_stream(char* p, u32x4 v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+}
+
+}  // namespace nt

@@ -1,0 +1,132 @@
+"""Packed storage of a nested tensor: buffer + nested size + device offsets.
+
+Counterpart of the reference's NestedTensorImpl / EfficientSizeNode
+(nestedtensor/csrc/nested_tensor_impl.h:46-173,
+nestedtensor/csrc/storage/EfficientSizeNode.h:53-138): one contiguous 1-D
+buffer, a host int64 table ``sizes[B, D]`` and the per-dimension "regular or
+not" summary ``opt_sizes``.  What is new here is the device side of the
+metadata: ``sizes`` mirrored in HBM and int64 element ``offsets[B + 1]`` built
+by the device prefix scan (nt_offsets_from_sizes), both cached on the impl and
+created on first use on the buffer's stream.  Only nested_dim 1 and the
+contiguous layout exist (EfficientSizeNode.h:86-88).
+"""
+
+import torch
+
+from . import _C
+
+
+class NestedTensorImpl:
+    __slots__ = ("buffer", "sizes", "_opt_sizes", "_sizes_dev", "_offsets_dev",
+                 "_row_offsets_dev", "_max_sizes")
+
+    def __init__(self, buffer, sizes):
+        """buffer: 1-D contiguous tensor; sizes: CPU int64 [B, D], or 0-d for an
+        empty nested tensor (EfficientSizeNode.h:8-12)."""
+        if buffer.dim() != 1:
+            raise RuntimeError("Given buffer must be vector, i.e. dim 1 Tensor.")
+        if not buffer.is_contiguous():
+            raise RuntimeError("Given buffer must be contiguous.")
+        assert sizes.dtype == torch.int64 and sizes.device.type == "cpu"
+        self.buffer = buffer
+        self.sizes = sizes
+        self._opt_sizes = None
+        self._sizes_dev = None
+        self._offsets_dev = None
+        self._row_offsets_dev = None
+        self._max_sizes = None
+
+    # ---- host metadata ----------------------------------------------------
+    @property
+    def B(self):
+        return self.sizes.size(0) if self.sizes.dim() > 0 else 0
+
+    @property
+    def D(self):
+        return self.sizes.size(1) if self.sizes.dim() > 0 else 0
+
+    def dim(self):
+        # EfficientSizeNode::dim (EfficientSizeNode.h:94-96)
+        return 1 + self.sizes.size(1) if self.sizes.dim() > 0 else 1
+
+    def nested_dim(self):
+        return 1
+
+    def numel(self):
+        # EfficientSizeNode::numel (EfficientSizeNode.h:113-131)
+        if self.sizes.dim() == 0 or self.sizes.numel() == 0:
+            return 0
+        return int(self.sizes.prod(1).sum())
+
+    def opt_sizes(self):
+        # construct_efficient_size (EfficientSizeNode.h:27-49)
+        if self._opt_sizes is None:
+            res = [self.B]
+            if self.sizes.dim() > 0 and self.B > 0:
+                first = self.sizes[0]
+                same = (self.sizes == first).all(0)
+                for j in range(self.D):
+                    res.append(int(first[j]) if bool(same[j]) else None)
+            self._opt_sizes = res
+        return list(self._opt_sizes)
+
+    def max_sizes(self):
+        # get_max_size_from_efficient_size (masking.cpp:83-103)
+        if self._max_sizes is None:
+            if self.B > 0 and self.D > 0:
+                self._max_sizes = [int(v) for v in self.sizes.max(0).values]
+            else:
+                self._max_sizes = []
+        return list(self._max_sizes)
+
+    def has_empty_constituent(self):
+        return self.B > 0 and self.D > 0 and bool((self.sizes == 0).any())
+
+    def shapes(self):
+        return [tuple(int(v) for v in row) for row in self.sizes] if self.sizes.dim() > 0 else []
+
+    # ---- device metadata ---------------------------------------------------
+    def sizes_dev(self):
+        if self._sizes_dev is None:
+            _C.require_device(self.buffer, "device metadata")
+            self._sizes_dev = self.sizes.contiguous().to(self.buffer.device)
+        return self._sizes_dev
+
+    def offsets_dev(self):
+        """int64 [B + 1] element offsets, built on the device by the prefix scan."""
+        if self._offsets_dev is None:
+            self._offsets_dev = device_offsets(self.sizes_dev(), self.B, self.D)
+        return self._offsets_dev
+
+    def row_offsets_dev(self):
+        """int64 [B + 1] offsets counted in rows of the first constituent dim
+        (token offsets for a [B, L_i, E] nested tensor)."""
+        if self._row_offsets_dev is None:
+            first = self.sizes_dev()[:, :1].contiguous()
+            self._row_offsets_dev = device_offsets(first, self.B, 1)
+        return self._row_offsets_dev
+
+    def with_buffer(self, buffer):
+        """Same nested size over another buffer; shares the cached metadata when
+        the device matches."""
+        out = NestedTensorImpl(buffer, self.sizes)
+        out._opt_sizes = self._opt_sizes
+        out._max_sizes = self._max_sizes
+        if buffer.device == self.buffer.device:
+            out._sizes_dev = self._sizes_dev
+            out._offsets_dev = self._offsets_dev
+            out._row_offsets_dev = self._row_offsets_dev
+        return out
+
+
+def device_offsets(sizes_dev, B, D):
+    """offsets[b] = sum_{c<b} prod_k sizes[c, k] on the device (nt_offsets_from_sizes)."""
+    dev = sizes_dev.device
+    offsets = torch.empty(B + 1, dtype=torch.int64, device=dev)
+    ws_bytes = _C.lib.nt_offsets_workspace_bytes(B)
+    ws = torch.empty(max(ws_bytes, 8), dtype=torch.uint8, device=dev) if ws_bytes else None
+    with torch.cuda.device(dev):
+        _C.check(_C.lib.nt_offsets_from_sizes(
+            _C.ptr(sizes_dev), B, D, _C.ptr(offsets), _C.ptr(ws), ws_bytes,
+            _C.current_stream(dev)))
+    return offsets

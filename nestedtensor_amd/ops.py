@@ -1,0 +1,403 @@
+"""Operator layer: the reference's ``torch.ops.nestedtensor.*`` surface for the
+ragged hot path, lowered to the C ABI.
+
+The reference registers these ops on ``DispatchKey::NestedTensor`` with a custom
+TensorImpl (nestedtensor/csrc/masking.cpp:652-675, csrc/mha.cpp:71-74,
+csrc/cuda/mha.cpp:109-113, csrc/py_init.cpp:132-216).  That dispatch key belongs
+to torch core now, so here the ``Tensor nt`` argument is the Python
+``NestedTensor`` wrapper: ``NestedTensor.__torch_function__`` intercepts the op
+call and routes it to the functions below, which work on
+``(buffer, sizes, offsets)``.  Schemas (names, argument order) are the
+reference's.  Host code in this file only validates, sizes outputs from the
+host copy of the nested size and launches; all data movement and arithmetic is
+in the HIP library.
+"""
+
+import torch
+
+from . import _C
+from .impl import NestedTensorImpl
+
+# ---------------------------------------------------------------------------
+# schemas (same names and argument order as the reference)
+
+_lib = torch.library.Library("nestedtensor", "DEF")
+_SCHEMAS = [
+    # nestedtensor/csrc/masking.cpp:652-675
+    "to_padded_tensor(Tensor nt, float padding) -> Tensor",
+    "to_tensor_mask(Tensor nt, int? mask_dim) -> (Tensor, Tensor)",
+    "to_mask(Tensor nt, int? mask_dim) -> Tensor",
+    "nt_from_tensor_mask(Tensor tensor, Tensor mask, int nested_dim) -> (Tensor, Tensor)",
+    "get_max_size(Tensor nt) -> int[]",
+    # nestedtensor/csrc/mha.cpp:72, nestedtensor/csrc/cuda/mha.cpp:110-111
+    "min_mha(int num_heads, int head_dim, float dropout_p, bool training, Tensor query, "
+    "Tensor key, Tensor value, Tensor in_proje_weight, Tensor? in_proj_bias, float scaling, "
+    "Tensor out_proj_weight, Tensor out_proj_bias) -> Tensor",
+    "bt_min_mha(int num_heads, int head_dim, float dropout_p, bool training, Tensor query, "
+    "Tensor key, Tensor value, Tensor attr_kernel, Tensor attr_bias, float scaling, "
+    "Tensor out_proj_weight, Tensor out_proj_bias) -> Tensor",
+    # nestedtensor/csrc/py_init.cpp:132-216
+    "is_nested_tensor_impl(Tensor tensor) -> bool",
+    "nested_dim(Tensor tensor) -> int",
+    "sizes(Tensor tensor) -> int?[]",
+    "len(Tensor self) -> int",
+    "get_dim(Tensor self) -> int",
+    "get_numel(Tensor self) -> int",
+    "get_is_contiguous(Tensor self, MemoryFormat memory_format) -> bool",
+    "make_contiguous(Tensor self) -> Tensor",
+    "to_tensor_list(Tensor tensor) -> Tensor[]",
+]
+for _s in _SCHEMAS:
+    _lib.define(_s)
+
+
+def _elem_bytes(dtype):
+    n = torch.empty((), dtype=dtype).element_size()
+    if n not in (1, 2, 4, 8):
+        # masking.cpp:622 returns an uninitialised tensor for other dtypes; raise instead.
+        raise RuntimeError("Input datatype %s is not supported." % dtype)
+    return n
+
+
+def _pad_bits(padding, dtype):
+    """The padding value converted the way the reference converts it,
+    ``(T)(double)`` (masking.cpp:594,610), as raw bits."""
+    t = torch.tensor(padding, dtype=dtype)
+    view = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()]
+    return int(t.view(view).item()) & ((1 << (8 * t.element_size())) - 1)
+
+
+def _n_ragged(impl):
+    """Number of leading constituent dims the row decode must walk: up to and
+    including the last irregular dim.  Trailing regular dims are one contiguous
+    run (the generalisation of _collapse_two_dims_3, masking.cpp:535-556)."""
+    opt = impl.opt_sizes()[1:]
+    n = 1
+    for k, v in enumerate(opt):
+        if v is None:
+            n = k + 1
+    return n
+
+
+def _check_no_empty(impl):
+    if impl.has_empty_constituent():
+        # masking.cpp:140-142, 640-642
+        raise RuntimeError("Empty tensors are not yet supported.")
+
+
+# ---------------------------------------------------------------------------
+# packed -> padded
+
+
+def add_padding(impl, padding):
+    """Launch nt_add_padding: [B, max_1..max_D] from the packed buffer."""
+    _C.require_device(impl.buffer, "to_padded_tensor")
+    B, D = impl.B, impl.D
+    max_size = impl.max_sizes()
+    nrag = _n_ragged(impl)
+    if nrag > 3:
+        raise RuntimeError("to_padded_tensor supports at most 3 irregular dimensions.")
+    out = torch.empty([B] + max_size, dtype=impl.buffer.dtype, device=impl.buffer.device)
+    eb = _elem_bytes(impl.buffer.dtype)
+    dev = impl.buffer.device
+    with torch.cuda.device(dev):
+        _C.check(_C.lib.nt_add_padding(
+            _C.ptr(impl.buffer), _C.ptr(out), _C.ptr(impl.offsets_dev()), _C.ptr(impl.sizes_dev()),
+            B, D, nrag, _C.i64_array(max_size), eb, _pad_bits(padding, impl.buffer.dtype),
+            _C.current_stream(dev)))
+    return out
+
+
+def to_padded_tensor(impl, padding):
+    """to_padded_tensor (masking.cpp:558-650)."""
+    opt = impl.opt_sizes()
+    if len(opt) == 1 and opt[0] == 1:
+        return impl.buffer                       # masking.cpp:628-631 (alias)
+    if impl.B == 0:
+        return torch.tensor([float(padding)])     # masking.cpp:634-636
+    if impl.D == 0:
+        # B scalars: the stack of the constituents.  (The reference pushes every
+        # 0-d constituent twice, masking.cpp:644-647; not followed.)
+        return impl.buffer.clone()
+    _check_no_empty(impl)
+    return add_padding(impl, padding)
+
+
+# ---------------------------------------------------------------------------
+# masks
+
+
+def _collapsed_mask_dims(impl, mask_dim):
+    """Closed form of merge_tensor_mask (masking.cpp:12-43) on the mask of a
+    nested tensor without empty constituents: starting from [B, max_1..max_D],
+    the last dim collapses iff it is regular; if every dim is regular the batch
+    dim collapses too and the mask is the scalar True.  Collapsing stops at
+    mask_dim.  Returns the number of mask dims kept (0 = scalar)."""
+    opt = impl.opt_sizes()
+    cur = impl.dim()
+    while True:
+        if mask_dim is not None and cur == mask_dim:
+            return cur
+        if cur == 0:
+            return 0
+        # last mask dim is index cur-1 of opt_sizes; the batch dim (index 0)
+        # collapses when everything after it did.
+        if cur == 1 or opt[cur - 1] is not None:
+            cur -= 1
+            continue
+        if mask_dim is not None and mask_dim != cur:
+            raise RuntimeError("Mask dimension is too small to represent data tensor.")
+        return cur
+
+
+def build_mask(impl, kept_dims):
+    """Bool mask over [B, max_1..max_{kept_dims-1}] (nt_build_mask)."""
+    dev = impl.buffer.device
+    if kept_dims == 0:
+        return torch.tensor(True, device=dev)
+    if kept_dims == 1:
+        return torch.ones(impl.B, dtype=torch.bool, device=dev)
+    _C.require_device(impl.buffer, "to_tensor_mask")
+    K = kept_dims - 1
+    if K > 3:
+        raise RuntimeError("masks over more than 3 constituent dimensions are not supported.")
+    ext = impl.max_sizes()[:K]
+    mask = torch.empty([impl.B] + ext, dtype=torch.bool, device=dev)
+    with torch.cuda.device(dev):
+        _C.check(_C.lib.nt_build_mask(
+            _C.ptr(mask), _C.ptr(impl.sizes_dev()), impl.B, impl.D, K, _C.i64_array(ext),
+            _C.current_stream(dev)))
+    return mask
+
+
+def _check_mask_dim(impl, mask_dim):
+    if mask_dim is not None and mask_dim > impl.dim():
+        raise RuntimeError(
+            "Requested mask dimension %d is bigger than dimension %d of given NestedTensor."
+            % (mask_dim, impl.dim()))
+
+
+def to_tensor_mask(impl, mask_dim=None):
+    """to_tensor_mask (masking.cpp:251-320).  The mask is always bool (the
+    reference's device path returns bool, its host path uint8 when nothing
+    collapsed)."""
+    _check_mask_dim(impl, mask_dim)
+    opt = impl.opt_sizes()
+    dev = impl.buffer.device
+    if len(opt) == 1 and opt[0] == 1:
+        # masking.cpp:305-313
+        mask = torch.tensor(True, device=dev) if (mask_dim is None or mask_dim == 0) \
+            else torch.tensor([True], device=dev)
+        return impl.buffer.reshape(-1), mask
+    if impl.B == 0:
+        # masking.cpp:164-167 then merge_tensor_mask
+        if mask_dim == 1:
+            return torch.tensor([0]), torch.tensor([False])
+        return torch.tensor([0]), torch.tensor(False)
+    if impl.D == 0:
+        # masking.cpp:91
+        raise RuntimeError("Internal error: Expected sizes_size_1 to be greater than 0.")
+    _check_no_empty(impl)
+    kept = _collapsed_mask_dims(impl, mask_dim)
+    data = add_padding(impl, 0)
+    return data, build_mask(impl, kept)
+
+
+def to_mask(impl, mask_dim=None):
+    """to_mask (masking.cpp:408-457)."""
+    _check_mask_dim(impl, mask_dim)
+    opt = impl.opt_sizes()
+    dev = impl.buffer.device
+    if len(opt) == 1 and opt[0] == 1:
+        return torch.tensor(True, device=dev) if (mask_dim is None or mask_dim == 0) \
+            else torch.tensor([True], device=dev)
+    if impl.B == 0:
+        raise RuntimeError("to_mask of an empty NestedTensor is not defined.")
+    if impl.dim() > 1 and mask_dim is not None and mask_dim > 1:
+        # masking.cpp:428-453: the first mask_dim - 1 constituent dims, no merge
+        K = mask_dim - 1
+        if bool((impl.sizes[:, :K] == 0).any()):
+            raise RuntimeError("Empty tensors are not yet supported.")
+        return build_mask(impl, mask_dim)
+    if impl.D == 0:
+        raise RuntimeError("Internal error: Expected sizes_size_1 to be greater than 0.")
+    _check_no_empty(impl)
+    return build_mask(impl, _collapsed_mask_dims(impl, mask_dim))
+
+
+# ---------------------------------------------------------------------------
+# padded -> packed (length based)
+
+
+def from_padded_tensor(padded, target):
+    """from_padded_tensor (masking.cpp:459-533): gather the entries inside
+    ``target``'s nested size out of ``padded``.  ``target`` is a NestedTensorImpl
+    whose nested size the result takes."""
+    if padded.dim() != target.dim():
+        raise RuntimeError("Target size has different dimension as input padded Tensor.")
+    _C.require_device(padded, "from_padded_tensor")
+    padded = padded.contiguous()
+    B, D = target.B, target.D
+    if padded.size(0) != B:
+        raise RuntimeError("Target size has a different batch size than the padded Tensor.")
+    ext = list(padded.shape[1:])
+    mx = target.max_sizes()
+    for k in range(D):
+        if mx[k] > ext[k]:
+            raise RuntimeError("Target size exceeds the padded Tensor in dimension %d." % (k + 1))
+    nrag = _n_ragged(target)
+    # a dim that is regular in `target` but shorter than the padded extent must
+    # be walked as ragged
+    opt = target.opt_sizes()[1:]
+    for k in range(D):
+        if opt[k] is not None and opt[k] != ext[k]:
+            nrag = max(nrag, k + 1)
+    if nrag > 3:
+        raise RuntimeError("from_padded_tensor supports at most 3 irregular dimensions.")
+    dev = padded.device
+    out = torch.empty(target.numel(), dtype=padded.dtype, device=dev)
+    res = target.with_buffer(out)
+    eb = _elem_bytes(padded.dtype)
+    with torch.cuda.device(dev):
+        _C.check(_C.lib.nt_remove_padding(
+            _C.ptr(padded), _C.ptr(out), _C.ptr(res.offsets_dev()), _C.ptr(res.sizes_dev()),
+            B, D, nrag, _C.i64_array(ext), eb, _C.current_stream(dev)))
+    return res
+
+
+# ---------------------------------------------------------------------------
+# list of tensors -> packed
+
+
+def pack_device(tensors, offsets_dev, total, dtype, device):
+    """impl::pack (Packed.h:75-98) for constituents that already live on the
+    device: one gather launch (nt_pack) instead of B copy_ calls."""
+    keep = [t.contiguous() for t in tensors]
+    out = torch.empty(total, dtype=dtype, device=device)
+    ptrs = torch.tensor([t.data_ptr() for t in keep], dtype=torch.int64).to(device)
+    with torch.cuda.device(device):
+        _C.check(_C.lib.nt_pack(
+            _C.ptr(ptrs), _C.ptr(out), _C.ptr(offsets_dev), len(keep),
+            _elem_bytes(dtype), _C.current_stream(device)))
+    # `keep` must outlive the launch on this stream; torch's caching allocator
+    # only reuses the blocks for later work on the same stream.
+    return out
+
+
+# ---------------------------------------------------------------------------
+# nested multi-head attention
+
+
+def linear(x, weight, bias):
+    """y = x @ weight.T + bias on a 2-D row-major view (nt_linear).  This is the
+    packed fast path of NestedTensor_matmul (matmul.cpp:13-41) with the packed
+    bias add (BinaryOps.cpp:97-107) fused into the GEMM epilogue."""
+    _C.require_device(x, "linear")
+    assert x.dim() == 2 and weight.dim() == 2 and x.stride(1) == 1
+    M, K = x.shape
+    N = weight.size(0)
+    if weight.size(1) != K:
+        raise RuntimeError("linear: weight of shape %s does not match input feature size %d"
+                           % (tuple(weight.shape), K))
+    weight = weight.contiguous()
+    if weight.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
+        raise RuntimeError("linear: input, weight and bias must have the same dtype")
+    if bias is not None:
+        bias = bias.contiguous()
+    out = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _C.check(_C.lib.nt_linear(
+            _C.ptr(x), x.stride(0), _C.ptr(weight), _C.ptr(bias), _C.ptr(out), N, M, N, K,
+            _C.dtype_code(x.dtype), _C.current_stream(x.device)))
+    return out
+
+
+def _check_mha_inputs(query, key, value):
+    if query.dim() != 3:
+        raise RuntimeError("query needs to be 3 dim.")
+    if key.dim() != 3:
+        raise RuntimeError("key needs to be 3 dim.")
+    if value.dim() != 3:
+        raise RuntimeError("value needs to be 3 dim.")
+
+
+def _offset_ptr(t, col):
+    import ctypes
+    return ctypes.c_void_p(t.data_ptr() + col * t.element_size())
+
+
+def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_bias, scaling,
+               out_proj_weight, out_proj_bias):
+    """Nested multi-head attention on packed buffers.  Semantics of min_mha
+    (mha.cpp:18-69): per sequence, softmax over that sequence's own keys only.
+    query/key/value are NestedTensorImpl of dim 3 with regular last dim."""
+    _check_mha_inputs(query, key, value)
+    opt = query.opt_sizes()
+    if opt[2] is None:
+        raise RuntimeError("query's third dimension must be regular.")
+    E = num_heads * head_dim
+    if opt[2] != E:
+        raise RuntimeError("query's embedding dimension %d does not match num_heads * head_dim = %d"
+                           % (opt[2], E))
+    if key.opt_sizes()[2] != E or value.opt_sizes()[2] != E:
+        raise RuntimeError("key and value must have the embedding dimension of query.")
+    if key.B != query.B or value.B != query.B:
+        raise RuntimeError("query, key and value must hold the same number of sequences.")
+    if not torch.equal(key.sizes, value.sizes):
+        raise RuntimeError("key and value must have the same nested size.")
+    _C.require_device(query.buffer, "multi-head attention")
+    dev = query.buffer.device
+    dtype = query.buffer.dtype
+    W = in_proj_weight.contiguous()
+    if tuple(W.shape) != (3 * E, E):
+        raise RuntimeError("in_proj_weight must have shape [3 * embed_dim, embed_dim].")
+    xq = query.buffer.reshape(-1, E)
+    same = (key is query or key.buffer.data_ptr() == query.buffer.data_ptr()) and \
+        (value is query or value.buffer.data_ptr() == query.buffer.data_ptr()) and \
+        torch.equal(key.sizes, query.sizes)
+    if same:
+        qkv = linear(xq, W, in_proj_bias)                       # [T, 3E]
+        q_t, k_t, v_t = qkv, qkv, qkv
+        qc, kc, vc = 0, E, 2 * E
+        ld = 3 * E
+        ldq = ldk = ldv = ld
+    else:
+        b = in_proj_bias
+        q_t = linear(xq, W[0:E], None if b is None else b[0:E])
+        k_t = linear(key.buffer.reshape(-1, E), W[E:2 * E], None if b is None else b[E:2 * E])
+        v_t = linear(value.buffer.reshape(-1, E), W[2 * E:], None if b is None else b[2 * E:])
+        qc = kc = vc = 0
+        ldq = ldk = ldv = E
+    attn = torch.empty((xq.size(0), E), dtype=dtype, device=dev)
+    max_q = int(query.sizes[:, 0].max()) if query.B > 0 else 0
+    with torch.cuda.device(dev):
+        _C.check(_C.lib.nt_varlen_attention(
+            _offset_ptr(q_t, qc), ldq, _offset_ptr(k_t, kc), ldk, _offset_ptr(v_t, vc), ldv,
+            _C.ptr(attn), E, _C.ptr(query.row_offsets_dev()), _C.ptr(key.row_offsets_dev()),
+            query.B, num_heads, head_dim, max_q, float(scaling), _C.dtype_code(dtype),
+            _C.current_stream(dev)))
+    out = linear(attn, out_proj_weight, out_proj_bias)
+    return query.with_buffer(out.reshape(-1))
+
+
+def min_mha(num_heads, head_dim, dropout_p, training, query, key, value, in_proj_weight,
+            in_proj_bias, scaling, out_proj_weight, out_proj_bias):
+    """min_mha (mha.cpp:18-69)."""
+    _check_mha_inputs(query, key, value)
+    if in_proj_bias is None:
+        raise RuntimeError("Input projection bias needs to be defined.")
+    if training and dropout_p > 0:
+        raise RuntimeError("nested multi-head attention is inference only (no dropout).")
+    return mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_bias,
+                      scaling, out_proj_weight, out_proj_bias)
+
+
+def bt_min_mha(num_heads, head_dim, dropout_p, training, query, key, value, attr_kernel,
+               attr_bias, scaling, out_proj_weight, out_proj_bias):
+    """bt_min_mha (cuda/mha.cpp:22-107).  As in the reference, key and value
+    are taken to be query, and out_proj_bias is not added (cuda/mha.cpp:106).
+    The softmax is the exact one over each sequence's own keys, which the
+    reference's -10000 additive mask and +1e-6 denominator approximate."""
+    _check_mha_inputs(query, key, value)
+    return mha_packed(num_heads, head_dim, query, query, query, attr_kernel, attr_bias, scaling,
+                      out_proj_weight, None)

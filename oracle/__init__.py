@@ -1,0 +1,61 @@
+"""CPU oracle for the nestedtensor ragged hot path.  TEST INFRASTRUCTURE ONLY.
+
+This package restates, with plain ``torch`` CPU ops and Python loops, what the
+reference's CPU code paths compute for packing, padding, un-padding, masks and
+nested multi-head attention.  Every function cites the reference file:line it
+follows.  It exists so that the HIP kernels can be checked for parity; nothing
+in the shipped package (``nestedtensor_amd``) imports it.  Only ``tests/``,
+``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` use it,
+and only as the checker / the timed CPU baseline.
+
+The arithmetic below the reference's own code lives in ATen (``at::matmul``,
+``at::softmax``, ``at::constant_pad_nd``, ``at::stack``, ``at::masked_select``),
+which the reference pins at torch 1.11.0.dev20220202 and which is not vendored
+in its tree; the oracle calls the same ATen entry points of the installed
+torch.  Padding, un-padding and masks are pure data movement, so their results
+do not depend on the ATen version and parity is bit-exact.  Attention parity is
+tolerance-based.
+
+Pinning (what each part was checked against, see tests/test_oracle_*.py):
+
+* pack / nested_size / size / nested_stride: literal cases of
+  test/test_nested_tensor_class.py:199-231, 256-265, 449-472 and the closed
+  form ``buffer == cat(flatten(t_i))``.
+* to_tensor_mask / to_mask: literal cases of
+  test/test_nested_tensor_masking.py:11-142, ``to_mask == to_tensor_mask()[1]``
+  (test/test_nested_tensor_class.py:809-817) and the closed form
+  ``mask[b, i...] = all(i_k < size[b, k])``.
+* nt_from_tensor_mask: literal cases of
+  test/test_nested_tensor_masking.py:146-452.
+* to_padded_tensor: literal case of test/test_nested_tensor_masking.py:454-477,
+  ``torch.nn.utils.rnn.pad_sequence`` and core ``torch.nested`` as independent
+  library cross-checks.
+* from_padded_tensor: round trip with to_padded_tensor and ``padded[mask]``.
+* min_mha: ``torch.nn.MultiheadAttention`` per sequence (the reference's own
+  differential, test/test_nested_tensor_functional.py:648-667) and dense
+  attention with ``key_padding_mask`` (:1118-1140), plus an fp64 brute force.
+* bt_min_mha: equality with min_mha at 1e-5 for zero out-bias
+  (test/test_nested_tensor_functional.py:1115).
+
+Two reference behaviours are restated here but deliberately not followed by
+the product: the uint8-vs-bool mask dtype of merge_tensor_mask
+(masking.cpp:149-157, 31) and the double push of 0-d constituents in the CPU
+to_padded_tensor (masking.cpp:644-647).
+"""
+
+from .nt import RefNestedTensor, ref_nested_tensor  # noqa: F401
+from .masking import (  # noqa: F401
+    get_max_size,
+    merge_tensor_mask,
+    pad_tensor_to_shape,
+    pad_nt,
+    to_tensor_mask,
+    to_mask,
+    to_padded_tensor,
+    from_padded_tensor,
+    nt_from_tensor_mask,
+    nt_from_tensor_mask_vectorised,
+    nested_tensor_from_tensor_mask,
+    nested_tensor_from_padded_tensor,
+)
+from .mha import min_mha, bt_min_mha  # noqa: F401

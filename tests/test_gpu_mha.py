@@ -1,0 +1,231 @@
+"""Parity of the HIP nested multi-head attention path with the CPU oracle.
+
+Tolerances (BASELINE north_star): fp32 <= 1e-5 relative to the output scale
+(max |a-b| / max |b|), fp16 / bf16 <= 2e-2 absolute.  The shape list is the
+reference's (test/test_nested_tensor_functional.py:1142-1160) plus the BASELINE
+configurations C3 (BERT-base, fp16) and C4 (bf16, high raggedness)."""
+
+import random
+
+import pytest
+import torch
+
+import nestedtensor_amd as nt
+import oracle
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda", 0)
+
+FP32_REL = 1e-5
+HALF_ABS = 2e-2
+
+
+def make_case(E, lens, seed, dtype, w_std=0.02, bias_std=0.0, x_std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    xs = [(torch.randn(L, E, generator=g) * x_std).to(dtype) for L in lens]
+    W_in = (torch.randn(3 * E, E, generator=g) * w_std).to(dtype)
+    W_out = (torch.randn(E, E, generator=g) * w_std).to(dtype)
+    b_in = (torch.randn(3 * E, generator=g) * bias_std).to(dtype)
+    b_out = (torch.randn(E, generator=g) * bias_std).to(dtype)
+    return xs, W_in, b_in, W_out, b_out
+
+
+def check(got_nt, exp_parts, dtype, exp64=None):
+    got = got_nt._impl.buffer.float().cpu()
+    exp = torch.cat([p.reshape(-1) for p in exp_parts]).float()
+    assert got.shape == exp.shape
+    assert torch.isfinite(got).all()
+    err = (got - exp).abs().max().item()
+    if dtype == torch.float32:
+        scale = max(exp.abs().max().item(), 1e-30)
+        assert err / scale <= FP32_REL, (err, scale)
+    else:
+        assert err <= HALF_ABS, err
+    if exp64 is not None:
+        # the fused path accumulates in fp32 and must not be further from the
+        # float64 answer than the reference's own dtype-rounded chain, up to
+        # one unit of output rounding
+        e64 = torch.cat([p.reshape(-1) for p in exp64]).float()
+        assert (got - e64).abs().max().item() <= (exp - e64).abs().max().item() + HALF_ABS / 4
+    return err
+
+
+def run_min_mha(H, hd, xs, W_in, b_in, W_out, b_out, dtype, via="op"):
+    E = H * hd
+    a = nt.nested_tensor(xs, device=DEV, dtype=dtype)
+    args = (H, hd, 0.0, False, a, a, a, W_in.to(DEV), b_in.to(DEV), float(hd) ** -0.5,
+            W_out.to(DEV), b_out.to(DEV))
+    return torch.ops.nestedtensor.min_mha(*args)
+
+
+REF_SHAPES = [  # (num_heads, batch_size, seq_len_, head_size)
+    (2, 1, 2, 1), (1, 3, 5, 4), (2, 3, 5, 2), (2, 1, 2, 2), (8, 8, 50, 16),
+    (16, 64, 50, 16), (4, 32, 50, 256), (16, 32, 50, 64),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("H,B,Lmax,hd", REF_SHAPES)
+def test_min_mha_reference_shapes(dtype, H, B, Lmax, hd):
+    random.seed(H * 1000 + B)
+    lens = [random.randint(1, Lmax) for _ in range(B)]
+    E = H * hd
+    xs, W_in, b_in, W_out, b_out = make_case(E, lens, 17, dtype, w_std=E ** -0.5, bias_std=0.1)
+    got = run_min_mha(H, hd, xs, W_in, b_in, W_out, b_out, dtype)
+    ref = oracle.ref_nested_tensor(xs, dtype=dtype)
+    exp = oracle.min_mha(H, hd, 0.0, False, ref, ref, ref, W_in, b_in, hd ** -0.5, W_out, b_out)
+    check(got, exp, dtype)
+    assert got.nested_size() == nt.nested_tensor(xs).nested_size()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_bt_min_mha_op_and_module_hook(dtype):
+    # test_nested_tensor_functional.py:1087-1140: bt_min_mha == mha(nt, nt, nt)
+    # == dense MHA with key_padding_mask (zero biases, as nn.MultiheadAttention
+    # initialises them)
+    random.seed(3)
+    H, hd, B, Lmax = 8, 16, 8, 50
+    E = H * hd
+    lens = [random.randint(1, Lmax) for _ in range(B)]
+    torch.manual_seed(1010)
+    mha = torch.nn.MultiheadAttention(E, H).to(dtype).eval()
+    xs = [torch.randn(L, E).to(dtype) for L in lens]
+    a = nt.nested_tensor(xs, device=DEV, dtype=dtype)
+    W_in = mha.in_proj_weight.detach().clone()
+    b_in = mha.in_proj_bias.detach().clone()
+    W_out = mha.out_proj.weight.detach().clone()
+    b_out = mha.out_proj.bias.detach().clone()
+    with torch.inference_mode():
+        r_bt = torch.ops.nestedtensor.bt_min_mha(H, hd, 0.5, False, a, a, a, W_in.to(DEV), b_in.to(DEV),
+                                                 float(hd) ** -0.5, W_out.to(DEV), b_in.to(DEV))
+        mha_dev = mha.to(DEV)
+        r_mod, w = mha_dev(a, a, a)
+    assert w is None and isinstance(r_mod, nt.NestedTensor)
+    assert torch.equal(r_bt._impl.buffer, r_mod._impl.buffer)       # zero out-bias: same result
+    ref = oracle.ref_nested_tensor(xs, dtype=dtype)
+    exp_bt = oracle.bt_min_mha(H, hd, 0.5, False, ref, ref, ref, W_in, b_in, hd ** -0.5, W_out, b_in)
+    exp = oracle.min_mha(H, hd, 0.0, False, ref, ref, ref, W_in, b_in, hd ** -0.5, W_out, b_out)
+    check(r_bt, exp, dtype)
+    check(r_bt, exp_bt, dtype)
+    # dense differential of the reference test: atol 5e-4 (fp32)
+    if dtype == torch.float32:
+        mha_cpu = mha.to("cpu").float()
+        padded = torch.nn.utils.rnn.pad_sequence(xs)
+        kpm = torch.ones(B, max(lens), dtype=torch.bool)
+        for b, L in enumerate(lens):
+            kpm[b, :L] = False
+        with torch.no_grad():
+            dense, _ = mha_cpu(padded, padded, padded, key_padding_mask=kpm, need_weights=False)
+        dense = dense.transpose(0, 1) * (~kpm).unsqueeze(-1)
+        assert torch.allclose(r_bt.to_padded_tensor(padding=0).cpu(), dense, atol=5e-4, rtol=1e-8)
+
+
+def test_bt_min_mha_ignores_out_bias_and_min_mha_adds_it():
+    H, hd = 2, 64
+    E = H * hd
+    xs, W_in, b_in, W_out, b_out = make_case(E, [5, 70, 33], 4, torch.float16, bias_std=0.5)
+    a = nt.nested_tensor(xs, device=DEV, dtype=torch.float16)
+    args = (H, hd, 0.0, False, a, a, a, W_in.to(DEV), b_in.to(DEV), hd ** -0.5, W_out.to(DEV))
+    r_bt = torch.ops.nestedtensor.bt_min_mha(*args, b_out.to(DEV))
+    r_min = torch.ops.nestedtensor.min_mha(*args, b_out.to(DEV))
+    r_zero = torch.ops.nestedtensor.min_mha(*args, torch.zeros_like(b_out).to(DEV))
+    assert torch.equal(r_bt._impl.buffer, r_zero._impl.buffer)
+    assert not torch.equal(r_bt._impl.buffer, r_min._impl.buffer)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_cross_attention_different_kv_lengths(dtype):
+    H, hd = 4, 64
+    E = H * hd
+    g = torch.Generator().manual_seed(5)
+    q = [torch.randn(L, E, generator=g).to(dtype) for L in (3, 130, 64)]
+    kv = [torch.randn(L, E, generator=g).to(dtype) for L in (77, 2, 200)]
+    _, W_in, b_in, W_out, b_out = make_case(E, [1], 6, dtype, w_std=E ** -0.5, bias_std=0.1)
+    qa, ka = nt.nested_tensor(q, device=DEV, dtype=dtype), nt.nested_tensor(kv, device=DEV, dtype=dtype)
+    got = torch.ops.nestedtensor.min_mha(H, hd, 0.0, False, qa, ka, ka, W_in.to(DEV), b_in.to(DEV),
+                                         hd ** -0.5, W_out.to(DEV), b_out.to(DEV))
+    rq, rk = oracle.ref_nested_tensor(q, dtype=dtype), oracle.ref_nested_tensor(kv, dtype=dtype)
+    exp = oracle.min_mha(H, hd, 0.0, False, rq, rk, rk, W_in, b_in, hd ** -0.5, W_out, b_out)
+    check(got, exp, dtype)
+
+
+def test_mha_input_errors():
+    a = nt.nested_tensor([torch.randn(3, 4), torch.randn(2, 4)], device=DEV)
+    b2 = nt.nested_tensor([torch.randn(3), torch.randn(2)], device=DEV)
+    W, bi, Wo, bo = (torch.randn(12, 4, device=DEV), torch.randn(12, device=DEV),
+                     torch.randn(4, 4, device=DEV), torch.randn(4, device=DEV))
+    with pytest.raises(RuntimeError, match="query needs to be 3 dim."):
+        torch.ops.nestedtensor.min_mha(2, 2, 0.0, False, b2, a, a, W, bi, 1.0, Wo, bo)
+    with pytest.raises(RuntimeError, match="key needs to be 3 dim."):
+        torch.ops.nestedtensor.bt_min_mha(2, 2, 0.0, False, a, b2, a, W, bi, 1.0, Wo, bo)
+    with pytest.raises(RuntimeError, match="Input projection bias needs to be defined."):
+        torch.ops.nestedtensor.min_mha(2, 2, 0.0, False, a, a, a, W, None, 1.0, Wo, bo)
+    irregular = nt.nested_tensor([torch.randn(3, 4), torch.randn(2, 5)], device=DEV)
+    with pytest.raises(RuntimeError, match="query's third dimension must be regular."):
+        torch.ops.nestedtensor.min_mha(2, 2, 0.0, False, irregular, a, a, W, bi, 1.0, Wo, bo)
+
+
+def _c3():
+    g = torch.Generator().manual_seed(1010 + 2)
+    lens = [int(v) for v in torch.randint(32, 513, (32,), generator=g)]
+    E = 768
+    xs = [torch.randn(L, E, generator=g).half() for L in lens]
+    W_in = (torch.randn(3 * E, E, generator=g) * 0.02).half()
+    W_out = (torch.randn(E, E, generator=g) * 0.02).half()
+    return lens, xs, W_in, torch.zeros(3 * E).half(), W_out, torch.zeros(E).half()
+
+
+def test_config_c3_bert_base_fp16():
+    lens, xs, W_in, b_in, W_out, b_out = _c3()
+    got = run_min_mha(12, 64, xs, W_in, b_in, W_out, b_out, torch.float16)
+    ref = oracle.ref_nested_tensor(xs, dtype=torch.float16)
+    exp = oracle.min_mha(12, 64, 0.0, False, ref, ref, ref, W_in, b_in, 64 ** -0.5, W_out, b_out)
+    ref64 = oracle.ref_nested_tensor([x.double() for x in xs], dtype=torch.float64)
+    exp64 = oracle.min_mha(12, 64, 0.0, False, ref64, ref64, ref64, W_in.double(), b_in.double(),
+                           64 ** -0.5, W_out.double(), b_out.double())
+    err = check(got, exp, torch.float16, exp64)
+    print("C3 fp16 max abs err vs oracle: %.3e" % err)
+    # the module route gives the same tensor
+    mha = torch.nn.MultiheadAttention(768, 12).half().eval()
+    with torch.no_grad():
+        mha.in_proj_weight.copy_(W_in)
+        mha.in_proj_bias.zero_()
+        mha.out_proj.weight.copy_(W_out)
+        mha.out_proj.bias.zero_()
+    a = nt.nested_tensor(xs, device=DEV, dtype=torch.float16)
+    with torch.inference_mode():
+        r_mod, _ = mha.to(DEV)(a, a, a)
+    assert torch.equal(r_mod._impl.buffer, got._impl.buffer)
+
+
+def test_config_c4_bf16_high_raggedness():
+    g = torch.Generator().manual_seed(1010 + 3)
+    raw = torch.empty(128).exponential_(1.0 / 96.0, generator=g)
+    lens = [int(v) for v in raw.round().clamp(8, 512)]
+    E, H = 1024, 16
+    xs = [torch.randn(L, E, generator=g).bfloat16() for L in lens]
+    W_in = (torch.randn(3 * E, E, generator=g) * 0.02).bfloat16()
+    W_out = (torch.randn(E, E, generator=g) * 0.02).bfloat16()
+    b_in, b_out = torch.zeros(3 * E).bfloat16(), torch.zeros(E).bfloat16()
+    a = nt.nested_tensor(xs, device=DEV, dtype=torch.bfloat16)
+    got = torch.ops.nestedtensor.bt_min_mha(H, 64, 0.0, False, a, a, a, W_in.to(DEV), b_in.to(DEV),
+                                            64 ** -0.5, W_out.to(DEV), b_out.to(DEV))
+    ref = oracle.ref_nested_tensor(xs, dtype=torch.bfloat16)
+    exp = oracle.min_mha(H, 64, 0.0, False, ref, ref, ref, W_in, b_in, 64 ** -0.5, W_out, b_out)
+    err = check(got, exp, torch.bfloat16)
+    print("C4 bf16 max abs err vs oracle: %.3e" % err)
+
+
+def test_linear_packed_fast_path():
+    # F.linear on a NestedTensor: one GEMM on the packed view (matmul.cpp:13-41)
+    g = torch.Generator().manual_seed(8)
+    for dtype, tol in ((torch.float32, 1e-5), (torch.float16, 2e-2)):
+        xs = [torch.randn(L, 96, generator=g).to(dtype) for L in (5, 131, 64)]
+        W = (torch.randn(200, 96, generator=g) * 0.1).to(dtype)
+        b = torch.randn(200, generator=g).to(dtype)
+        a = nt.nested_tensor(xs, device=DEV, dtype=dtype)
+        y = torch.nn.functional.linear(a, W.to(DEV), b.to(DEV))
+        assert y.size() == (3, None, 200)
+        for yi, xi in zip(y.unbind(), xs):
+            exp = torch.nn.functional.linear(xi, W, b).float()
+            assert (yi.float().cpu() - exp).abs().max() <= tol * max(1.0, exp.abs().max().item())
