@@ -1,0 +1,295 @@
+#!/usr/bin/env python3
+"""Benchmark of the ragged hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one pass over BASELINE configuration C5: 4096 fp16 constituents
+[L_i, 4096], L_i uniform in [1, 2048] (1.7e10 elements, 34 GB packed), padded to
+the chunk maximum in chunks of 512 constituents (nt_add_padding) and un-padded
+again (nt_remove_padding).  All data is generated on the device and is resident
+in HBM before the timed region.  `value` is the algorithmic bytes of the whole
+step (pad: valid read + padded written; un-pad: valid read + valid written)
+divided by the step time.
+
+The same JSON line carries
+  roofline     - the dominant kernel (row_kernel<2, pad>): algorithmic bytes per
+                 launch / mean launch time from HIP events, against 8 TB/s;
+  cpu_baseline - the CPU oracle (the reference's CPU algorithm restated) timed on
+                 a bounded sample of the same workload on the host cores;
+  mha          - nested BERT-base self-attention (configuration C3) tokens/s and
+                 its MFMA roofline fraction.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, GB/s
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, TFLOP/s
+
+METRIC = "ragged->padded HBM GB/s + nested BERT MHA tokens/s (B=32, L<=512, d=768)"
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--chunk", type=int, default=512, help="constituents per chunk")
+    ap.add_argument("--batch", type=int, default=4096, help="constituents in total (C5: 4096)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-mha", action="store_true", help="skip the C3 attention leg")
+    return ap.parse_args()
+
+
+def build_c5(torch, nt_impl, dev, batch, chunk):
+    """Lengths on the host (seeded), values on the device, chunk by chunk."""
+    g = torch.Generator().manual_seed(1010 + 4)
+    lengths = torch.randint(1, 2049, (batch,), generator=g)
+    E = 4096
+    total_rows = int(lengths.sum())
+    packed = torch.empty(total_rows * E, dtype=torch.float16, device=dev)
+    torch.manual_seed(1010 + 4)
+    chunks = []
+    row0 = 0
+    for c0 in range(0, batch, chunk):
+        ls = lengths[c0:c0 + chunk]
+        rows = int(ls.sum())
+        view = packed[row0 * E:(row0 + rows) * E]
+        # N(0,1) values, generated in place in slabs to bound temporaries
+        slab = 1 << 28
+        for s in range(0, view.numel(), slab):
+            view[s:s + slab].normal_()
+        sizes = torch.stack([ls, torch.full_like(ls, E)], 1).contiguous()
+        impl = nt_impl(view, sizes)
+        chunks.append(impl)
+        row0 += rows
+    return lengths, packed, chunks
+
+
+def bench_c5(args, torch, dev):
+    from nestedtensor_amd import _C
+    from nestedtensor_amd.impl import NestedTensorImpl
+
+    lengths, packed, chunks = build_c5(torch, NestedTensorImpl, dev, args.batch, args.chunk)
+    E, eb = 4096, 2
+    max_padded = max(c.B * c.max_sizes()[0] * E for c in chunks)
+    max_valid = max(c.numel() for c in chunks)
+    padded_buf = torch.empty(max_padded, dtype=torch.float16, device=dev)
+    unpacked_buf = torch.empty(max_valid, dtype=torch.float16, device=dev)
+    stream = _C.current_stream(dev)
+
+    meta = []
+    for c in chunks:
+        ext = c.max_sizes()
+        meta.append(dict(impl=c, ext=_C.i64_array(ext), offsets=c.offsets_dev(), sizes=c.sizes_dev(),
+                         valid_bytes=c.numel() * eb, padded_bytes=c.B * ext[0] * E * eb))
+    torch.cuda.synchronize()
+
+    def pad(m):
+        _C.check(_C.lib.nt_add_padding(_C.ptr(m["impl"].buffer), _C.ptr(padded_buf), _C.ptr(m["offsets"]),
+                                       _C.ptr(m["sizes"]), m["impl"].B, 2, 1, m["ext"], eb, 0, stream))
+
+    def unpad(m):
+        _C.check(_C.lib.nt_remove_padding(_C.ptr(padded_buf), _C.ptr(unpacked_buf), _C.ptr(m["offsets"]),
+                                          _C.ptr(m["sizes"]), m["impl"].B, 2, 1, m["ext"], eb, stream))
+
+    # warm-up, with the size-independent parity property of the full-size run:
+    # un-pad(pad(x)) == x bit-exact, and the padding region reads as the pad value
+    for w in range(max(args.warmup, 1)):
+        for m in meta:
+            pad(m)
+            unpad(m)
+            if w == 0:
+                n = m["impl"].numel()
+                assert torch.equal(unpacked_buf[:n].view(torch.int16), m["impl"].buffer.view(torch.int16)), \
+                    "round trip is not bit-exact"
+                B, L = m["impl"].B, m["impl"].max_sizes()[0]
+                pv = padded_buf[:B * L * E].view(B, L, E)
+                lens = m["impl"].sizes[:, 0]
+                b_short = int(torch.argmin(lens))
+                assert bool((pv[b_short, int(lens[b_short]):] == 0).all()), "padding region is not the pad value"
+    torch.cuda.synchronize()
+
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(len(meta) * args.steps)]
+    step_start = torch.cuda.Event(enable_timing=True)
+    step_end = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    step_start.record()
+    i = 0
+    for s in range(args.steps):
+        for m in meta:
+            e = ev[i]
+            e[0].record()
+            pad(m)
+            e[1].record()
+            unpad(m)
+            e[2].record()
+            i += 1
+    step_end.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    total_ms = step_start.elapsed_time(step_end)
+    ms_per_step = total_ms / args.steps
+
+    pad_ms = [e[0].elapsed_time(e[1]) for e in ev]
+    unpad_ms = [e[1].elapsed_time(e[2]) for e in ev]
+    pad_bytes = [m["valid_bytes"] + m["padded_bytes"] for m in meta] * args.steps
+    unpad_bytes = [2 * m["valid_bytes"] for m in meta] * args.steps
+    step_bytes = sum(m["valid_bytes"] + m["padded_bytes"] + 2 * m["valid_bytes"] for m in meta)
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    pad_gbs = sum(pad_bytes) / (sum(pad_ms) * 1e-3) / 1e9
+    unpad_gbs = sum(unpad_bytes) / (sum(unpad_ms) * 1e-3) / 1e9
+    res = dict(
+        value=value, ms_per_step=ms_per_step, wall_ms_per_step=wall_ms / args.steps,
+        roofline=dict(bound="hbm", kernel="row_kernel<2, pad> (nt_add_padding)",
+                      achieved=pad_gbs, peak=HBM_PEAK_GBS, unit="GB/s", frac=pad_gbs / HBM_PEAK_GBS,
+                      traffic=None,
+                      bytes_per_launch=sum(pad_bytes) / len(pad_bytes),
+                      ms_per_launch=sum(pad_ms) / len(pad_ms), launches=len(pad_ms)),
+        unpad=dict(kernel="row_kernel<2, unpad> (nt_remove_padding)", achieved=unpad_gbs,
+                   peak=HBM_PEAK_GBS, unit="GB/s", frac=unpad_gbs / HBM_PEAK_GBS,
+                   bytes_per_launch=sum(unpad_bytes) / len(unpad_bytes),
+                   ms_per_launch=sum(unpad_ms) / len(unpad_ms)),
+        workload=dict(constituents=int(lengths.numel()), packed_elements=int(lengths.sum()) * E,
+                      packed_GB=int(lengths.sum()) * E * eb / 1e9,
+                      padded_GB=sum(m["padded_bytes"] for m in meta) / 1e9, chunks=len(meta)))
+    del padded_buf, unpacked_buf, packed, chunks, meta
+    torch.cuda.empty_cache()
+    return res
+
+
+def cpu_baseline_c5(torch, n_sample=96):
+    """The oracle's to_padded_tensor + from_padded_tensor on the first n_sample
+    constituents of C5 (same seeded lengths), timed on the host cores."""
+    import oracle
+    torch.set_num_threads(os.cpu_count() or 1)
+    g = torch.Generator().manual_seed(1010 + 4)
+    lengths = torch.randint(1, 2049, (4096,), generator=g)[:n_sample]
+    E = 4096
+    parts = [torch.randn(int(l), E, generator=g).half() for l in lengths]
+    ref = oracle.ref_nested_tensor(parts, dtype=torch.float16)
+    valid = ref.buffer.numel() * 2
+    padded_bytes = n_sample * int(lengths.max()) * E * 2
+    best = None
+    for it in range(3):
+        t0 = time.perf_counter()
+        padded = oracle.to_padded_tensor(ref, 0)
+        t1 = time.perf_counter()
+        back = oracle.from_padded_tensor(padded, ref)
+        t2 = time.perf_counter()
+        if it == 0:
+            assert torch.equal(back.buffer.view(torch.int16), ref.buffer.view(torch.int16))
+        if best is None or (t2 - t0) < best[0]:
+            best = (t2 - t0, t1 - t0, t2 - t1)
+    step_bytes = valid + padded_bytes + 2 * valid
+    return dict(value=step_bytes / best[0] / 1e9, unit="GB/s", cores=torch.get_num_threads(),
+                kind="port",
+                sample="first %d of 4096 C5 constituents (%.2f GB packed fp16), oracle "
+                       "to_padded_tensor + from_padded_tensor, best of 3; pad %.2f GB/s, un-pad %.2f GB/s"
+                       % (n_sample, valid / 1e9, (valid + padded_bytes) / best[1] / 1e9,
+                          2 * valid / best[2] / 1e9),
+                host_cpus=os.cpu_count())
+
+
+def bench_mha_c3(args, torch, dev):
+    import nestedtensor_amd as nt
+    import oracle
+    g = torch.Generator().manual_seed(1010 + 2)
+    lens = [int(v) for v in torch.randint(32, 513, (32,), generator=g)]
+    E, H, hd = 768, 12, 64
+    xs = [torch.randn(L, E, generator=g).half() for L in lens]
+    W_in = (torch.randn(3 * E, E, generator=g) * 0.02).half()
+    W_out = (torch.randn(E, E, generator=g) * 0.02).half()
+    b_in, b_out = torch.zeros(3 * E).half(), torch.zeros(E).half()
+    a = nt.nested_tensor(xs, device=dev, dtype=torch.float16)
+    dW_in, db_in, dW_out, db_out = W_in.to(dev), b_in.to(dev), W_out.to(dev), b_out.to(dev)
+
+    def layer():
+        return torch.ops.nestedtensor.min_mha(H, hd, 0.0, False, a, a, a, dW_in, db_in, hd ** -0.5,
+                                              dW_out, db_out)
+
+    for _ in range(5):
+        out = layer()
+    torch.cuda.synchronize()
+    iters = 50
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        out = layer()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / iters
+    T = sum(lens)
+    flops = 8 * T * E * E + 4 * E * sum(L * L for L in lens)
+    res = dict(workload="C3: nested BERT-base self-attention, fp16, B=32, L~U[32,512], d=768, 12x64",
+               tokens=T, ms_per_layer=ms, tokens_per_s=T / (ms * 1e-3), flops=flops,
+               roofline=dict(bound="mfma", achieved=flops / (ms * 1e-3) / 1e12, peak=MFMA_F16_PEAK_TFLOPS,
+                             unit="TFLOP/s", frac=flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS))
+    if not args.no_cpu:
+        torch.set_num_threads(os.cpu_count() or 1)
+        ref = oracle.ref_nested_tensor(xs, dtype=torch.float16)
+        best = None
+        for it in range(2):
+            t0 = time.perf_counter()
+            exp = oracle.min_mha(H, hd, 0.0, False, ref, ref, ref, W_in, b_in, hd ** -0.5, W_out, b_out)
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        err = (out._impl.buffer.float().cpu() - torch.cat([p.reshape(-1) for p in exp]).float()).abs().max()
+        res["max_abs_err_vs_oracle"] = float(err)
+        res["cpu_baseline"] = dict(value=T / best, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
+                                   sample="full C3 layer, oracle min_mha in fp16 on the host, best of 2")
+    return res
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported "
+              "(the path shards by constituent ranges, see DESIGN.md)." % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+
+    c5 = bench_c5(args, torch, dev)
+    line = {
+        "metric": METRIC,
+        "value": c5["value"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": c5["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "C5: 4096 fp16 [L_i,4096], L_i~U[1,2048], pad to chunk max in chunks of %d "
+                               "+ reverse remove_padding; value = algorithmic GB per step / step time"
+                               % args.chunk,
+                   **c5["workload"]},
+        "roofline": c5["roofline"],
+        "unpad": c5["unpad"],
+    }
+    if not args.no_mha:
+        line["mha"] = bench_mha_c3(args, torch, dev)
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_c5(torch)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
