@@ -8,10 +8,38 @@
 // (or nothing, if some i_k >= s_k) and whose remainder is padding.  Rows are
 // decoded once per workgroup with scalar arithmetic; inside a row every lane
 // moves 16-byte chunks: destination-aligned 128-bit stores, 128-bit loads of
-// any alignment.  grid.x walks rows, grid.y strides over 16 KiB tiles of a row.
+// any alignment.  grid.x walks the 4 KiB tiles of a row, grid.y (and z) the rows,
+// so workgroups that are dispatched together touch one compact, contiguous
+// window of both buffers; measured on MI355X this ordering and one 16-byte
+// chunk per lane (many small workgroups) give the highest HBM throughput, well
+// above fewer workgroups with more chunks in flight per lane.
 //
 // All index math is int64: the largest configuration holds 1.7e10 elements.
 #include "nt_common.h"
+
+// Tuning knobs of the row kernels (compile-time).
+#ifndef NT_ROW_UNROLL
+#define NT_ROW_UNROLL 1          // 16-byte chunks in flight per lane
+#endif
+#ifndef NT_ROW_STREAM_STORE
+#define NT_ROW_STREAM_STORE 1    // non-temporal stores for the output
+#endif
+#ifndef NT_ROW_TILE_FAST
+#define NT_ROW_TILE_FAST 1       // 1: consecutive workgroups walk the tiles of one row
+#endif
+#ifndef NT_ROW_TARGET_WGS
+#define NT_ROW_TARGET_WGS (1 << 24)
+#endif
+// Workgroups per row at most; longer rows are looped over.  Every tile of a
+// padded row is written, so pad / mask take one workgroup per tile up to 16 MiB
+// rows; un-pad and pack move only the valid prefix, and fewer, looping
+// workgroups leave fewer of them without work on short rows.
+#ifndef NT_ROW_MAX_TILES_PAD
+#define NT_ROW_MAX_TILES_PAD 4096
+#endif
+#ifndef NT_ROW_MAX_TILES_UNPAD
+#define NT_ROW_MAX_TILES_UNPAD 1024
+#endif
 
 namespace nt {
 
@@ -58,13 +86,26 @@ __device__ __forceinline__ void move_elem(char* d, const char* s, int64_t pos, i
   *reinterpret_cast<T*>(d + pos) = v;
 }
 
+// Which workgroups share a row: grid.y by default (consecutive workgroups walk
+// different rows), grid.x when NT_ROW_TILE_FAST (consecutive workgroups walk the
+// tiles of one row).
+#if NT_ROW_TILE_FAST
+__device__ __forceinline__ unsigned tile_index() { return blockIdx.x; }
+__device__ __forceinline__ unsigned tile_count() { return gridDim.x; }
+__device__ __forceinline__ int64_t row_index() { return (int64_t)blockIdx.y + (int64_t)blockIdx.z * 65535; }
+#else
+__device__ __forceinline__ unsigned tile_index() { return blockIdx.y; }
+__device__ __forceinline__ unsigned tile_count() { return gridDim.y; }
+__device__ __forceinline__ int64_t row_index() { return blockIdx.x; }
+#endif
+
 // Cooperative move of one row: bytes [0, valid) come from s, bytes [valid, total)
 // are padding.  Called by every workgroup of the row's grid.y column.
 template <int EB, int MODE>
 __device__ __forceinline__ void move_row(char* d, const char* s, int64_t valid, int64_t total,
                                          const u32x4 pad) {
   constexpr int kThreads = 256;
-  constexpr int kUnroll = 4;
+  constexpr int kUnroll = NT_ROW_UNROLL;
   const int tid = threadIdx.x;
 
   int64_t head = (int64_t)((0 - (uintptr_t)d) & 15);
@@ -72,7 +113,7 @@ __device__ __forceinline__ void move_row(char* d, const char* s, int64_t valid, 
   const int64_t nvec = (total - head) >> 4;
   const int64_t tail_start = head + (nvec << 4);
 
-  if (blockIdx.y == 0) {
+  if (tile_index() == 0) {
     // unaligned edges of the destination row: fewer than 32 bytes
     const int64_t nedge = (head + (total - tail_start)) / EB;
     for (int64_t e = tid; e < nedge; e += kThreads) {
@@ -83,8 +124,8 @@ __device__ __forceinline__ void move_row(char* d, const char* s, int64_t valid, 
   }
 
   const int64_t tile_chunks = (int64_t)kThreads * kUnroll;
-  for (int64_t c0 = (int64_t)blockIdx.y * tile_chunks; c0 < nvec;
-       c0 += (int64_t)gridDim.y * tile_chunks) {
+  for (int64_t c0 = (int64_t)tile_index() * tile_chunks; c0 < nvec;
+       c0 += (int64_t)tile_count() * tile_chunks) {
     u32x4 v[kUnroll];
     int state[kUnroll];
 #pragma unroll
@@ -112,7 +153,11 @@ __device__ __forceinline__ void move_row(char* d, const char* s, int64_t valid, 
       const int64_t c = c0 + u * kThreads + tid;
       const int64_t pos = head + (c << 4);
       if (state[u] == 1) {
+#if NT_ROW_STREAM_STORE
         store16_stream(d + pos, v[u]);
+#else
+        store16(d + pos, v[u]);
+#endif
       } else if (state[u] == 2) {
 #pragma unroll
         for (int k = 0; k < 16; k += EB) {
@@ -125,7 +170,8 @@ __device__ __forceinline__ void move_row(char* d, const char* s, int64_t valid, 
 
 template <int EB, int MODE>
 __global__ __launch_bounds__(256) void row_kernel(RowParams p) {
-  const int64_t row = blockIdx.x;
+  const int64_t row = row_index();
+  if (row >= p.nrows) return;
   if (MODE == kPack) {
     const int64_t off = p.offsets[row];
     const int64_t n = (p.offsets[row + 1] - off) * EB;
@@ -202,16 +248,23 @@ static int launch_rows(int eb, const RowParams& p, int64_t max_row_bytes, hipStr
   if (p.nrows > 0x7fffffffLL) {
     return fail(NT_ERR_UNSUPPORTED, "row count %lld exceeds the grid limit", (long long)p.nrows);
   }
-  const int64_t tile_bytes = 256 * 4 * 16;
+  const int64_t tile_bytes = 256 * NT_ROW_UNROLL * 16;
   int64_t tiles = (max_row_bytes + tile_bytes - 1) / tile_bytes;
   // Enough workgroups to fill 256 CUs several times over, but long rows are
   // walked by a bounded number of workgroups that each loop over tiles.
-  int64_t y_cap = (1 << 20) / p.nrows;
+  int64_t y_cap = (int64_t)NT_ROW_TARGET_WGS / p.nrows;
   if (y_cap < 1) y_cap = 1;
-  if (y_cap > 1024) y_cap = 1024;
+  const int64_t max_tiles = (MODE == kPad || MODE == kOnes) ? NT_ROW_MAX_TILES_PAD : NT_ROW_MAX_TILES_UNPAD;
+  if (y_cap > max_tiles) y_cap = max_tiles;
   int64_t gy = tiles < y_cap ? tiles : y_cap;
   if (gy < 1) gy = 1;
+#if NT_ROW_TILE_FAST
+  const int64_t gz = (p.nrows + 65534) / 65535;
+  if (gz > 65535) return fail(NT_ERR_UNSUPPORTED, "row count %lld exceeds the grid limit", (long long)p.nrows);
+  dim3 grid((unsigned)gy, (unsigned)(p.nrows < 65535 ? p.nrows : 65535), (unsigned)gz);
+#else
   dim3 grid((unsigned)p.nrows, (unsigned)gy, 1);
+#endif
   dim3 block(256, 1, 1);
   switch (eb) {
     case 1: hipLaunchKernelGGL((row_kernel<1, MODE>), grid, block, 0, stream, p); break;
