@@ -31,6 +31,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, GB/s
+# HBM bytes per launch / algorithmic bytes per launch of the pad kernel, from the
+# rocprofv3 FETCH_SIZE and WRITE_SIZE runs of `bench.py --pmc-probe`, each scaled
+# by what the same counter reads for a 4 GiB plain copy (FETCH_SIZE: 2.0 KiB per
+# unit, WRITE_SIZE: 1.0 KiB per unit).
+PAD_TRAFFIC_RATIO = 1.0001
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, TFLOP/s
 
 METRIC = "ragged->padded HBM GB/s + nested BERT MHA tokens/s (B=32, L<=512, d=768)"
@@ -45,6 +50,9 @@ def parse():
     ap.add_argument("--batch", type=int, default=4096, help="constituents in total (C5: 4096)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-mha", action="store_true", help="skip the C3 attention leg")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="one plain copy of known size, then one pad and one un-pad launch of the "
+                         "first C5 chunk; meant to run under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
     return ap.parse_args()
 
 
@@ -152,7 +160,7 @@ def bench_c5(args, torch, dev):
         value=value, ms_per_step=ms_per_step, wall_ms_per_step=wall_ms / args.steps,
         roofline=dict(bound="hbm", kernel="row_kernel<2, pad> (nt_add_padding)",
                       achieved=pad_gbs, peak=HBM_PEAK_GBS, unit="GB/s", frac=pad_gbs / HBM_PEAK_GBS,
-                      traffic=None,
+                      traffic=PAD_TRAFFIC_RATIO * sum(pad_bytes) / len(pad_bytes),
                       bytes_per_launch=sum(pad_bytes) / len(pad_bytes),
                       ms_per_launch=sum(pad_ms) / len(pad_ms), launches=len(pad_ms)),
         unpad=dict(kernel="row_kernel<2, unpad> (nt_remove_padding)", achieved=unpad_gbs,
@@ -165,6 +173,35 @@ def bench_c5(args, torch, dev):
     del padded_buf, unpacked_buf, packed, chunks, meta
     torch.cuda.empty_cache()
     return res
+
+
+def pmc_probe(args, torch, dev):
+    """Three dispatches for hardware-counter runs: a plain device copy of 4 GiB
+    (reads 4 GiB, writes 4 GiB: the calibration for the counters' unit), one
+    nt_add_padding and one nt_remove_padding launch on the first C5 chunk."""
+    from nestedtensor_amd import _C
+    from nestedtensor_amd.impl import NestedTensorImpl
+    _, packed, chunks = build_c5(torch, NestedTensorImpl, dev, args.chunk, args.chunk)
+    m = chunks[0]
+    E, eb = 4096, 2
+    ext = m.max_sizes()
+    padded = torch.empty(m.B * ext[0] * E, dtype=torch.float16, device=dev)
+    back = torch.empty(m.numel(), dtype=torch.float16, device=dev)
+    src = torch.ones(1 << 31, dtype=torch.float16, device=dev)
+    dst = torch.empty_like(src)
+    offsets, sizes = m.offsets_dev(), m.sizes_dev()
+    stream = _C.current_stream(dev)
+    torch.cuda.synchronize()
+    dst.copy_(src)
+    _C.check(_C.lib.nt_add_padding(_C.ptr(m.buffer), _C.ptr(padded), _C.ptr(offsets), _C.ptr(sizes),
+                                   m.B, 2, 1, _C.i64_array(ext), eb, 0, stream))
+    _C.check(_C.lib.nt_remove_padding(_C.ptr(padded), _C.ptr(back), _C.ptr(offsets), _C.ptr(sizes),
+                                      m.B, 2, 1, _C.i64_array(ext), eb, stream))
+    torch.cuda.synchronize()
+    assert torch.equal(back.view(torch.int16), m.buffer.view(torch.int16))
+    print(json.dumps({"copy_bytes_read": src.numel() * 2, "copy_bytes_written": src.numel() * 2,
+                      "pad_valid_bytes": m.numel() * eb, "pad_padded_bytes": padded.numel() * eb,
+                      "unpad_valid_bytes": m.numel() * eb}))
 
 
 def cpu_baseline_c5(torch, n_sample=96):
@@ -263,6 +300,9 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
 
+    if args.pmc_probe:
+        pmc_probe(args, torch, dev)
+        return
     c5 = bench_c5(args, torch, dev)
     line = {
         "metric": METRIC,
