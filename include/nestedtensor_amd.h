@@ -151,6 +151,34 @@ int nt_varlen_attention(const void* q, int64_t ldq, const void* k, int64_t ldk,
                         int64_t num_heads, int64_t head_dim, int64_t max_q_len,
                         float scale, int dtype, void* stream);
 
+/* The fused in-projection of self-attention: [Q | K | V] = A * W^T + bias with
+ * W [3E, K]; Q and K are written row-major into QK[M, 2E] (row stride ldqk), V is
+ * written transposed, Vt[e][m] (row stride ldvt >= M; nt_varlen_attention_vt
+ * wants ldvt >= M + 72), which is the layout nt_varlen_attention_vt reads.  Replaces the packed in-projection
+ * at::matmul(query, attr_kernel.t()) + attr_bias of bt_min_mha
+ * (nestedtensor/csrc/cuda/mha.cpp:57) together with the chunk / reshape /
+ * transpose views that follow it (:60-69), and stands where the unwired
+ * add_QKV_bias_padding kernel (nestedtensor/csrc/cuda/attention.cu:107-174)
+ * was meant to go. */
+int nt_linear_qkv(const void* A, int64_t lda, const void* W, const void* bias, void* QK,
+                  int64_t ldqk, void* Vt, int64_t ldvt, int64_t M, int64_t E, int64_t K,
+                  int dtype, void* stream);
+
+/* Self-attention (query, key and value are one nested tensor) on the output of
+ * nt_linear_qkv: Q at column h*64 and K at column k_col + h*64 of QK, V^T in Vt;
+ * head_dim is 64, dtype f16 or bf16.  `schedule` is a device array of n_work
+ * int32[4] work items {first token of the sequence, sequence length, first query
+ * row of the tile (multiple of 128), 0}: one per 128-query tile of every
+ * sequence, in the order they should start (longest sequences first); a
+ * workgroup is launched per (item, head), so no padded tile is ever issued.  The
+ * rows of Vt must be readable up to 72 elements past the last token
+ * (ldvt >= total_tokens + 72); what is stored there is ignored.  Output and
+ * semantics as nt_varlen_attention. */
+int nt_varlen_attention_vt(const void* qk, int64_t ldqk, int64_t k_col, const void* vt,
+                           int64_t ldvt, void* out, int64_t ldo, const int32_t* schedule,
+                           int64_t n_work, int64_t num_heads, int64_t total_tokens, float scale,
+                           int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

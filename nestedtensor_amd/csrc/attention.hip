@@ -29,10 +29,23 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float acc16 __attribute__((ext_vector_type(16)));
 
+typedef float float2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
 template <typename T> struct AttnT;
 template <> struct AttnT<_Float16> {
   typedef half8 Frag;
   typedef half4 Half;
+  // two fp32 -> packed pair, round to nearest even (v_cvt_pk_f16_f32)
+  static __device__ __forceinline__ uint32_t cvt2(float a, float b) {
+    float2v x = {a, b};
+    half2v h = __builtin_convertvector(x, half2v);
+    uint32_t r;
+    __builtin_memcpy(&r, &h, 4);
+    return r;
+  }
+  static constexpr uint32_t kOnePair = 0x3c003c00u;   // (1.0, 1.0)
   static __device__ __forceinline__ acc16 mma(Frag a, Frag b, acc16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
@@ -40,6 +53,14 @@ template <> struct AttnT<_Float16> {
 template <> struct AttnT<__bf16> {
   typedef bf16x8 Frag;
   typedef bf16x4 Half;
+  static __device__ __forceinline__ uint32_t cvt2(float a, float b) {
+    float2v x = {a, b};
+    bf16x2 h = __builtin_convertvector(x, bf16x2);
+    uint32_t r;
+    __builtin_memcpy(&r, &h, 4);
+    return r;
+  }
+  static constexpr uint32_t kOnePair = 0x3f803f80u;
   static __device__ __forceinline__ acc16 mma(Frag a, Frag b, acc16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
@@ -253,6 +274,217 @@ __global__ __launch_bounds__(256) void varlen_attention_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// Self-attention kernel of the fused layer: Q and K come row-major from the
+// [T, 2E] projection buffer, V comes TRANSPOSED (Vt[h*64 + d][token], written
+// that way by the QKV GEMM epilogue), so a V^T tile is 64 rows of 64
+// key-contiguous values and needs no transposition on its way into LDS.
+//
+// LDS layout of the V^T tile: within each group of 16 keys the positions are
+// permuted (key = 8a + 4g + c  ->  position 8g + 4a + c) so that the eight keys a
+// lane group needs for one MFMA k-step -- the keys whose probabilities it
+// already holds in its score accumulators -- are one 16-byte read.
+
+// Work items {first token, length, first query row, 0} come from a schedule the
+// host builds from the nested size (longest sequences first, no item for a tile
+// that does not exist), so every workgroup that is launched has work and the
+// long sequences start first.
+#ifndef NT_ATTN_WAVES_PER_EU
+#define NT_ATTN_WAVES_PER_EU 3
+#endif
+
+template <typename T>
+__global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt_kernel(
+    const T* __restrict__ QK, int64_t ldqk, int64_t k_col, const T* __restrict__ Vt, int64_t ldvt,
+    T* __restrict__ O, int64_t ldo, const int4* __restrict__ schedule, float scale_log2e) {
+  typedef AttnT<T> AT;
+  typedef typename AT::Frag Frag;
+
+  __shared__ __align__(16) char lds_k[2][kKBytes];
+  __shared__ __align__(16) char lds_v[2][kVBytes];
+
+  const int4 item = schedule[blockIdx.x];
+  const int h = blockIdx.y;
+  const int64_t begin = item.x;
+  const int L = item.y;
+  const int q0 = item.z;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int g = lane >> 5;
+
+  const int q_row = q0 + wave * 32 + l32;
+  const bool wave_active = (q0 + wave * 32) < L;
+  Frag qf[4];
+  {
+    // rows past L read the last row; their results are never stored
+    const int qr = q_row < L ? q_row : L - 1;
+    const T* qp = QK + (begin + qr) * ldqk + h * kHd + g * 8;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      u32x4 v = load16_unaligned(reinterpret_cast<const char*>(qp + s * 16));
+      __builtin_memcpy(&qf[s], &v, 16);
+    }
+  }
+
+  acc16 o_acc[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o_acc[i][e] = 0.0f;
+  float m_run = -INFINITY;
+  float l_run = 0.0f;
+
+  const int ntiles = (L + kKTile - 1) / kKTile;
+  const T* kbase = QK + begin * ldqk + k_col + h * kHd;
+  const T* vbase = Vt + (int64_t)h * kHd * ldvt + begin;
+
+  // Each thread moves two 16-byte pieces of the K tile and two of the V^T tile.
+  // The loads are unconditional and unmasked (clamped addresses), so that the
+  // wavefront only waits for them where the data is stored to LDS.
+  const int r0 = tid >> 3;      // row of piece 0 (piece 1: r0 + 32)
+  const int cc = tid & 7;
+  u32x4 rk[2], rv[2];
+  auto gload = [&](int t_in) {
+    const int t = t_in < ntiles ? t_in : ntiles - 1;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r = r0 + i * 32;
+      int kr = t * kKTile + r;
+      kr = kr < L ? kr : L - 1;        // rows past L: their scores are masked below
+      rk[i] = load16_unaligned(reinterpret_cast<const char*>(kbase + (int64_t)kr * ldqk + cc * 8));
+      // V^T piece: keys key0 .. key0+7 of row d = r, read where it lies (the rows
+      // of Vt are readable 72 elements past the last token)
+      rv[i] = load16_unaligned(
+          reinterpret_cast<const char*>(vbase + (int64_t)r * ldvt + t * kKTile + cc * 8));
+    }
+  };
+  auto lstore = [&](int buf, int t) {
+    // keys at or past L are zeroed: a probability of exactly 0 must not meet a NaN
+    int nv = L - (t * kKTile + cc * 8);
+    nv = nv > 8 ? 8 : (nv < 0 ? 0 : nv);
+    const uint32_t m0 = nv >= 2 ? 0xffffffffu : (nv == 1 ? 0x0000ffffu : 0u);
+    const uint32_t m1 = nv >= 4 ? 0xffffffffu : (nv == 3 ? 0x0000ffffu : 0u);
+    const uint32_t m2 = nv >= 6 ? 0xffffffffu : (nv == 5 ? 0x0000ffffu : 0u);
+    const uint32_t m3 = nv >= 8 ? 0xffffffffu : (nv == 7 ? 0x0000ffffu : 0u);
+    // piece cc = keys 8cc .. 8cc+7 = (ks = cc/2, a = cc%2); its low half (g = 0)
+    // goes to position 16ks + 4a, its high half (g = 1) to 16ks + 8 + 4a.
+    const int ks = cc >> 1, a2 = cc & 1;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r = r0 + i * 32;
+      store16(&lds_k[buf][r * kKRow + cc * 16], rk[i]);
+      char* row = &lds_v[buf][r * kVRow];
+      const uint64_t lo = ((uint64_t)(rv[i].y & m1) << 32) | (rv[i].x & m0);
+      const uint64_t hi = ((uint64_t)(rv[i].w & m3) << 32) | (rv[i].z & m2);
+      *reinterpret_cast<uint64_t*>(row + (16 * ks + 4 * a2) * 2) = lo;
+      *reinterpret_cast<uint64_t*>(row + (16 * ks + 8 + 4 * a2) * 2) = hi;
+    }
+  };
+
+  gload(0);
+  lstore(0, 0);
+  __syncthreads();
+
+  for (int t = 0; t < ntiles; ++t) {
+    const int buf = t & 1;
+    gload(t + 1);   // past the end: re-reads the last tile, never stored
+
+    if (wave_active) {
+      acc16 s_acc[2];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s_acc[kb][e] = 0.0f;
+        const char* krow = &lds_k[buf][(kb * 32 + l32) * kKRow + g * 16];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          Frag kf = *reinterpret_cast<const Frag*>(krow + s * 32);
+          s_acc[kb] = AT::mma(kf, qf[s], s_acc[kb]);
+        }
+      }
+      // s_acc[kb][e] = score(key = 64 t + 32 kb + 8 (e/4) + 4 g + e%4, q = l32)
+      const int key_base = t * kKTile;
+      if (key_base + kKTile > L) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int key = key_base + kb * 32 + 8 * (e >> 2) + 4 * g + (e & 3);
+            if (key >= L) s_acc[kb][e] = -INFINITY;
+          }
+      }
+      float m_tile = s_acc[0][0];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) m_tile = fmaxf(m_tile, s_acc[kb][e]);
+      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
+      const float m_new = fmaxf(m_run, m_tile);   // finite: every tile holds a valid key
+      // raw v_exp_f32: arguments are <= 0, results in [0, 1]
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
+      const float m_scaled = m_new * scale_log2e;
+      m_run = m_new;
+      Frag pf[4];   // P^T as B-operand: k-step ks = 2 kb + half uses s_acc[kb][8 half .. +8]
+      float l_tile = 0.0f;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          uint32_t w[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float p0 =
+                __builtin_amdgcn_exp2f(fmaf(s_acc[kb][half * 8 + 2 * j], scale_log2e, -m_scaled));
+            const float p1 =
+                __builtin_amdgcn_exp2f(fmaf(s_acc[kb][half * 8 + 2 * j + 1], scale_log2e, -m_scaled));
+            l_tile += p0 + p1;
+            w[j] = AT::cvt2(p0, p1);
+          }
+          __builtin_memcpy(&pf[kb * 2 + half], w, 16);
+        }
+      }
+      l_run = l_run * alpha + l_tile;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+
+      // O^T += V^T P^T
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+        for (int db = 0; db < 2; ++db) {
+          const char* vrow = &lds_v[buf][(db * 32 + l32) * kVRow + g * 16];
+          Frag vf = *reinterpret_cast<const Frag*>(vrow + ks * 32);
+          o_acc[db] = AT::mma(vf, pf[ks], o_acc[db]);
+        }
+      }
+    }
+
+    lstore(buf ^ 1, t + 1);   // past the end: harmless, the buffer is not read again
+    __syncthreads();
+  }
+
+  if (!wave_active || q_row >= L) return;
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+  T* op = O + (begin + q_row) * ldo + h * kHd;
+#pragma unroll
+  for (int db = 0; db < 2; ++db) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      // d = 32 db + 8 r + 4 g + (0..3)
+      uint32_t w0 = AT::cvt2(o_acc[db][r * 4 + 0] * inv, o_acc[db][r * 4 + 1] * inv);
+      uint32_t w1 = AT::cvt2(o_acc[db][r * 4 + 2] * inv, o_acc[db][r * 4 + 3] * inv);
+      uint64_t bits = ((uint64_t)w1 << 32) | w0;
+      __builtin_memcpy(reinterpret_cast<char*>(op + db * 32 + 8 * r + 4 * g), &bits, 8);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Generic kernel: any head_dim, any dtype, fp32 math.  One wavefront per
 // (query row, head); keys in groups of 64 (one per lane), online softmax.
 
@@ -405,4 +637,40 @@ extern "C" int nt_varlen_attention(const void* q, int64_t ldq, const void* k, in
     default:
       return fail(NT_ERR_INVALID_ARGUMENT, "attention: unknown dtype %d", dtype);
   }
+}
+
+extern "C" int nt_varlen_attention_vt(const void* qk, int64_t ldqk, int64_t k_col, const void* vt,
+                                      int64_t ldvt, void* out, int64_t ldo,
+                                      const int32_t* schedule, int64_t n_work, int64_t num_heads,
+                                      int64_t total_tokens, float scale, int dtype, void* stream) {
+  if (n_work < 0 || num_heads < 1 || total_tokens < 0) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "attention_vt: bad shape");
+  }
+  if (n_work == 0) return NT_OK;
+  if (!qk || !vt || !out || !schedule) return fail(NT_ERR_INVALID_ARGUMENT, "attention_vt: NULL pointer");
+  if (n_work > 0x7fffffffLL || num_heads > 65535 || total_tokens > 0x7fffffffLL) {
+    return fail(NT_ERR_UNSUPPORTED, "attention_vt: too many work items, heads or tokens");
+  }
+  const int64_t E = num_heads * kHd;
+  if (ldqk < k_col + E || ldo < E || ldvt < total_tokens + 72) {
+    return fail(NT_ERR_INVALID_ARGUMENT,
+                "attention_vt: row strides too small (ldvt must be >= total_tokens + 72)");
+  }
+  dim3 grid((unsigned)n_work, (unsigned)num_heads, 1);
+  const float scale_log2e = scale * 1.4426950408889634f;
+  hipStream_t s = (hipStream_t)stream;
+  const int4* sched = reinterpret_cast<const int4*>(schedule);
+  if (dtype == NT_F16) {
+    hipLaunchKernelGGL((varlen_attention_vt_kernel<_Float16>), grid, dim3(256), 0, s,
+                       static_cast<const _Float16*>(qk), ldqk, k_col,
+                       static_cast<const _Float16*>(vt), ldvt, static_cast<_Float16*>(out), ldo,
+                       sched, scale_log2e);
+  } else if (dtype == NT_BF16) {
+    hipLaunchKernelGGL((varlen_attention_vt_kernel<__bf16>), grid, dim3(256), 0, s,
+                       static_cast<const __bf16*>(qk), ldqk, k_col, static_cast<const __bf16*>(vt),
+                       ldvt, static_cast<__bf16*>(out), ldo, sched, scale_log2e);
+  } else {
+    return fail(NT_ERR_UNSUPPORTED, "attention_vt: dtype must be f16 or bf16");
+  }
+  return check_launch("varlen_attention_vt_kernel");
 }

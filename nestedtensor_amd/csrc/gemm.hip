@@ -4,13 +4,24 @@
 //
 // A is the packed token buffer viewed as [T, E] (no padded rows exist), W is a
 // torch Linear weight, so both operands are K-contiguous: every MFMA operand
-// fragment is one 16-byte run of a row.  Workgroup tile 128 x 128, 256 threads
-// as 2 x 2 wavefronts of 64 x 64 (2 x 2 MFMA 32x32 blocks each), K tiles of
-// 128 bytes double-buffered in LDS with rows padded to 144 bytes so that the
-// 128-bit fragment reads of 16 consecutive lanes fall into distinct banks.
-// Global loads of tile k+1 are issued before the MFMAs of tile k.
-// fp32 accumulation for all types; f16 / bf16 use v_mfma_f32_32x32x16_*,
-// fp32 uses v_mfma_f32_32x32x2_f32.
+// fragment is one 16-byte run of a row.  A workgroup owns a BM x BN tile of C,
+// its wavefronts a WAVES_M x WAVES_N grid of (WM*32) x (WN*32) sub-tiles made of
+// 32x32 MFMA blocks (fp32 accumulate; f16 / bf16: v_mfma_f32_32x32x16_*, fp32:
+// v_mfma_f32_32x32x2_f32).  K is walked in tiles of BKB bytes per row,
+// double-buffered in LDS; LDS rows are padded by 16 bytes so that the 128-bit
+// fragment reads of 16 consecutive lanes fall into distinct banks.
+//
+// Global loads run PF K-tiles ahead of the MFMAs (register staging), because one
+// K-tile of MFMA work is far shorter than the L2 / HBM latency.
+//
+// Epilogues:
+//   plain  - C row-major + bias;
+//   QKV    - the fused in-projection of self-attention: columns [0, n_split)
+//            (Q and K) go row-major into C, columns [n_split, N) (V) are written
+//            TRANSPOSED into Vt[n - n_split][m] so that the attention kernel
+//            finds V^T tiles key-contiguous.  V tiles run the MFMAs with swapped
+//            operands, which leaves C^T in the accumulators and keeps the
+//            stores coalesced.
 #include "nt_common.h"
 
 namespace nt {
@@ -27,8 +38,6 @@ template <> struct Mma<_Float16> {
   static __device__ __forceinline__ acc16 run(Frag a, Frag b, acc16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
-  static __device__ __forceinline__ _Float16 from_float(float x) { return (_Float16)x; }
-  static __device__ __forceinline__ float to_float(_Float16 x) { return (float)x; }
 };
 
 template <> struct Mma<__bf16> {
@@ -37,8 +46,6 @@ template <> struct Mma<__bf16> {
   static __device__ __forceinline__ acc16 run(Frag a, Frag b, acc16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
-  static __device__ __forceinline__ __bf16 from_float(float x) { return (__bf16)x; }
-  static __device__ __forceinline__ float to_float(__bf16 x) { return (float)x; }
 };
 
 template <> struct Mma<float> {
@@ -47,22 +54,57 @@ template <> struct Mma<float> {
   static __device__ __forceinline__ acc16 run(Frag a, Frag b, acc16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
   }
-  static __device__ __forceinline__ float from_float(float x) { return x; }
-  static __device__ __forceinline__ float to_float(float x) { return x; }
 };
 
-constexpr int kBM = 128;
-constexpr int kBN = 128;
-constexpr int kRowBytes = 128;            // K-tile bytes per row
-constexpr int kLdsRowBytes = 144;         // padded
-constexpr int kTileLdsBytes = (kBM + kBN) * kLdsRowBytes;
+template <int WAVES_M_, int WAVES_N_, int WM_, int WN_, int BKB_, int PF_>
+struct GemmCfg {
+  static constexpr int kPF = PF_;                     // K tiles in flight in registers
+  static constexpr int kWavesM = WAVES_M_, kWavesN = WAVES_N_, kWM = WM_, kWN = WN_;
+  static constexpr int kThreads = 64 * WAVES_M_ * WAVES_N_;
+  static constexpr int kBM = WAVES_M_ * WM_ * 32;
+  static constexpr int kBN = WAVES_N_ * WN_ * 32;
+  static constexpr int kRowBytes = BKB_;              // K-tile bytes per row
+  static constexpr int kLdsRow = BKB_ + 16;           // padded LDS row
+  static constexpr int kChunksPerRow = BKB_ / 16;
+  static constexpr int kChunks = (kBM + kBN) * kChunksPerRow;
+  static constexpr int kPerA = kBM * kChunksPerRow / kThreads;   // A pieces per thread
+  static constexpr int kPerB = kBN * kChunksPerRow / kThreads;   // W pieces per thread
+  static constexpr int kPerThread = kPerA + kPerB;
+  static constexpr int kBufBytes = (kBM + kBN) * kLdsRow;
+  static_assert((kBM * kChunksPerRow) % kThreads == 0 && (kBN * kChunksPerRow) % kThreads == 0,
+                "tile pieces must divide among the threads");
+};
 
-// 16-byte piece `cc` (0..7) of row `row` of a K tile starting at element k0.
-// Out-of-range rows / K tails read as zero.
 template <typename T>
+struct GemmArgs {
+  const T* A;
+  int64_t lda;
+  const T* W;
+  const T* bias;
+  T* C;
+  int64_t ldc;
+  int64_t M, N, K;
+  T* Vt;            // QKV epilogue: transposed destination of columns >= n_split
+  int64_t ldvt;
+  int64_t n_split;
+};
+
+// 16-byte piece of a row at element k.
+// ALIGNED_K (K is a multiple of the K tile): branch-free and mask-free.
+// Out-of-range rows are clamped to the last row -- they only feed accumulators
+// that are never stored -- and the caller clamps the K tile index, so every
+// address is valid and nothing has to be zeroed.  This matters: control flow
+// around the loads, or a mask applied to the loaded value, makes the wavefront
+// wait for the load right away and serialises the global-load / MFMA pipeline.
+// Otherwise (any K): element-wise tail handling.
+template <typename T, bool ALIGNED_K>
 __device__ __forceinline__ u32x4 load_chunk(const T* base, int64_t ld, int64_t row, int64_t nrows,
                                             int64_t k, int64_t K) {
   constexpr int kPer = 16 / sizeof(T);
+  if (ALIGNED_K) {
+    const int64_t r = row < nrows ? row : nrows - 1;
+    return load16_unaligned(reinterpret_cast<const char*>(base + r * ld + k));
+  }
   u32x4 v = {0, 0, 0, 0};
   if (row < nrows) {
     const T* p = base + row * ld + k;
@@ -78,134 +120,267 @@ __device__ __forceinline__ u32x4 load_chunk(const T* base, int64_t ld, int64_t r
   return v;
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void linear_kernel(const T* __restrict__ A, int64_t lda,
-                                                     const T* __restrict__ W,
-                                                     const T* __restrict__ bias,
-                                                     T* __restrict__ C, int64_t ldc, int64_t M,
-                                                     int64_t N, int64_t K) {
+enum { kEpiPlain = 0, kEpiQkv = 1 };
+
+// One BM x BN tile.  SWAP runs the MFMAs with the operands exchanged, which
+// leaves C^T in the accumulators, and stores into Vt (the V part of the fused
+// QKV projection).
+template <typename T, class Cfg, bool SWAP, bool ALIGNED_K>
+__device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int64_t n0, char* lds) {
   typedef Mma<T> MM;
   typedef typename MM::Frag Frag;
-  constexpr int kPer = 16 / sizeof(T);          // elements per 16-byte chunk
-  constexpr int kBK = kRowBytes / sizeof(T);    // elements per K tile
-  constexpr int kSteps = kBK / MM::kK;          // MFMA steps per K tile
+  constexpr int kPer = 16 / sizeof(T);
+  constexpr int kBK = Cfg::kRowBytes / sizeof(T);
+  constexpr int kSteps = kBK / MM::kK;
   constexpr int kFragBytes = (MM::kK / 2) * sizeof(T);
-
-  extern __shared__ __align__(16) char lds[];
+  constexpr int WM = Cfg::kWM, WN = Cfg::kWN, PF = Cfg::kPF;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1;   // wavefront row (0..1)
-  const int wn = wave & 1;    // wavefront col (0..1)
+  const int wm = wave / Cfg::kWavesN;
+  const int wn = wave % Cfg::kWavesN;
   const int l32 = lane & 31;
   const int g = lane >> 5;
 
-  // Tiles of one column panel are adjacent in launch order, so workgroups that
-  // run together share the same W panel in L2.
-  const int64_t tiles_m = (M + kBM - 1) / kBM;
-  const int64_t tile = blockIdx.x;
-  const int64_t tm = tile % tiles_m;
-  const int64_t tn = tile / tiles_m;
-  const int64_t m0 = tm * kBM;
-  const int64_t n0 = tn * kBN;
-
-  acc16 acc[2][2];
+  acc16 acc[WM][WN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < WN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  const int64_t nk = (K + kBK - 1) / kBK;
-  u32x4 ra[4], rb[4];
+  const int64_t nk = (a.K + kBK - 1) / kBK;
+  u32x4 stage[PF][Cfg::kPerThread];
 
-  auto gload = [&](int64_t kt) {
+  auto gload = [&](int slot, int64_t kt_in) {
+    // with ALIGNED_K tiles past the end re-read the last tile (never consumed)
+    const int64_t kt = (ALIGNED_K && kt_in >= nk) ? nk - 1 : kt_in;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + i * 256;
-      const int row = c >> 3;
-      const int cc = c & 7;
-      const int64_t k = kt * kBK + cc * kPer;
-      ra[i] = load_chunk<T>(A, lda, m0 + row, M, k, K);
-      rb[i] = load_chunk<T>(W, K, n0 + row, N, k, K);
+    for (int i = 0; i < Cfg::kPerA; ++i) {
+      const int c = tid + i * Cfg::kThreads;
+      const int row = c / Cfg::kChunksPerRow;
+      const int cc = c % Cfg::kChunksPerRow;
+      stage[slot][i] = load_chunk<T, ALIGNED_K>(a.A, a.lda, m0 + row, a.M, kt * kBK + cc * kPer, a.K);
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::kPerB; ++i) {
+      const int c = tid + i * Cfg::kThreads;
+      const int row = c / Cfg::kChunksPerRow;
+      const int cc = c % Cfg::kChunksPerRow;
+      stage[slot][Cfg::kPerA + i] =
+          load_chunk<T, ALIGNED_K>(a.W, a.K, n0 + row, a.N, kt * kBK + cc * kPer, a.K);
     }
   };
-  auto lstore = [&](int buf) {
-    char* base = lds + buf * kTileLdsBytes;
+  auto lstore = [&](int slot, int buf) {
+    char* base = lds + buf * Cfg::kBufBytes;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + i * 256;
-      const int row = c >> 3;
-      const int cc = c & 7;
-      store16(base + row * kLdsRowBytes + cc * 16, ra[i]);
-      store16(base + (kBM + row) * kLdsRowBytes + cc * 16, rb[i]);
+    for (int i = 0; i < Cfg::kPerA; ++i) {
+      const int c = tid + i * Cfg::kThreads;
+      store16(base + (c / Cfg::kChunksPerRow) * Cfg::kLdsRow + (c % Cfg::kChunksPerRow) * 16,
+              stage[slot][i]);
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::kPerB; ++i) {
+      const int c = tid + i * Cfg::kThreads;
+      store16(base + (Cfg::kBM + c / Cfg::kChunksPerRow) * Cfg::kLdsRow +
+                  (c % Cfg::kChunksPerRow) * 16,
+              stage[slot][Cfg::kPerA + i]);
     }
   };
-
-  gload(0);
-  lstore(0);
-  __syncthreads();
-
-  for (int64_t kt = 0; kt < nk; ++kt) {
-    const int buf = (int)(kt & 1);
-    if (kt + 1 < nk) gload(kt + 1);
-    const char* a_base = lds + buf * kTileLdsBytes + (wm * 64 + l32) * kLdsRowBytes;
-    const char* b_base = lds + buf * kTileLdsBytes + (kBM + wn * 64 + l32) * kLdsRowBytes;
+  auto compute = [&](int buf) {
+    const char* a_base = lds + buf * Cfg::kBufBytes + (wm * WM * 32 + l32) * Cfg::kLdsRow;
+    const char* b_base =
+        lds + buf * Cfg::kBufBytes + (Cfg::kBM + wn * WN * 32 + l32) * Cfg::kLdsRow;
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
       const int koff = s * MM::kK * (int)sizeof(T) + g * kFragBytes;
-      Frag fa[2], fb[2];
+      Frag fa[WM], fb[WN];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        fa[i] = *reinterpret_cast<const Frag*>(a_base + i * 32 * kLdsRowBytes + koff);
-        fb[i] = *reinterpret_cast<const Frag*>(b_base + i * 32 * kLdsRowBytes + koff);
-      }
+      for (int i = 0; i < WM; ++i)
+        fa[i] = *reinterpret_cast<const Frag*>(a_base + i * 32 * Cfg::kLdsRow + koff);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int j = 0; j < WN; ++j)
+        fb[j] = *reinterpret_cast<const Frag*>(b_base + j * 32 * Cfg::kLdsRow + koff);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = MM::run(fa[i], fb[j], acc[i][j]);
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+          if (SWAP) {
+            acc[i][j] = MM::run(fb[j], fa[i], acc[i][j]);
+          } else {
+            acc[i][j] = MM::run(fa[i], fb[j], acc[i][j]);
+          }
+        }
     }
-    if (kt + 1 < nk) lstore(buf ^ 1);
-    __syncthreads();
+  };
+
+  // Pipeline: K tiles kt+1 .. kt+PF are in flight from global memory in
+  // registers while tile kt is multiplied out of LDS.  With ALIGNED_K the loads
+  // and LDS stores of the loop body are straight-line code (loads past the last K
+  // tile re-read it and hit the cache), so the compiler can wait for exactly the
+  // oldest tile in flight instead of for every outstanding load.
+#pragma unroll
+  for (int j = 0; j < PF; ++j) {
+    if (ALIGNED_K || j < nk) gload(j, j);
+  }
+  lstore(0, 0);
+  if (ALIGNED_K || PF < nk) gload(0, PF);
+  __syncthreads();
+  for (int64_t kt0 = 0; kt0 < nk; kt0 += PF) {
+#pragma unroll
+    for (int j = 0; j < PF; ++j) {
+      const int64_t kt = kt0 + j;
+      const int buf = (j + (int)(kt0 & 1) * (PF & 1)) & 1;   // == kt & 1
+      const int slot = (j + 1) % PF;
+      if (ALIGNED_K) {
+        lstore(slot, buf ^ 1);
+        gload(slot, kt + 1 + PF);
+        if (kt < nk) compute(buf);   // uniform; false only in the last, partial group
+        __syncthreads();
+      } else if (kt < nk) {
+        if (kt + 1 < nk) lstore(slot, buf ^ 1);
+        if (kt + 1 + PF < nk) gload(slot, kt + 1 + PF);
+        compute(buf);
+        __syncthreads();
+      }
+    }
   }
 
-  // Epilogue: acc[i][j][e] is C[row, col] with
-  //   row = m0 + wm*64 + i*32 + 8*(e/4) + 4*g + e%4,  col = n0 + wn*64 + j*32 + l32.
+  if (!SWAP) {
+    // acc[i][j][e] = C[row, col], row = .. + i*32 + 8*(e/4) + 4*g + e%4, col = .. + j*32 + l32
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int64_t col = n0 + wn * 64 + j * 32 + l32;
-    if (col >= N) continue;
-    const float bv = bias ? MM::to_float(bias[col]) : 0.0f;
+    for (int j = 0; j < WN; ++j) {
+      const int64_t col = n0 + (wn * WN + j) * 32 + l32;
+      if (col >= a.N) continue;
+      const float bv = a.bias ? (float)a.bias[col] : 0.0f;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < WM; ++i) {
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int64_t row = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * g + (e & 3);
-        if (row < M) C[row * ldc + col] = MM::from_float(acc[i][j][e] + bv);
+        for (int e = 0; e < 16; ++e) {
+          const int64_t row = m0 + (wm * WM + i) * 32 + 8 * (e >> 2) + 4 * g + (e & 3);
+          if (row < a.M) a.C[row * a.ldc + col] = (T)(acc[i][j][e] + bv);
+        }
+      }
+    }
+  } else {
+    // acc[i][j][e] = C[row, col], col = .. + j*32 + 8*(e/4) + 4*g + e%4, row = .. + i*32 + l32
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+      const int64_t row = m0 + (wm * WM + i) * 32 + l32;
+      if (row >= a.M) continue;
+#pragma unroll
+      for (int j = 0; j < WN; ++j) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int64_t col = n0 + (wn * WN + j) * 32 + 8 * (e >> 2) + 4 * g + (e & 3);
+          if (col < a.N) {
+            const float bv = a.bias ? (float)a.bias[col] : 0.0f;
+            a.Vt[(col - a.n_split) * a.ldvt + row] = (T)(acc[i][j][e] + bv);
+          }
+        }
       }
     }
   }
 }
 
-template <typename T>
-static int launch_linear(const void* A, int64_t lda, const void* W, const void* bias, void* C,
-                         int64_t ldc, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
-  const int64_t tiles = ((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN);
-  if (tiles > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "linear: too many tiles");
+// Workgroup i runs on XCD i % 8 and every XCD has its own L2.  The tile order
+// gives XCD x the row tiles x, x + 8, x + 16, ... for every column panel, one
+// column panel after the other: its share of A (an eighth of the rows) stays
+// L2-resident while the W panels stream through, so A leaves HBM once instead
+// of once per column panel.
+template <typename T, class Cfg, int EPI, bool ALIGNED_K>
+__global__ __launch_bounds__(Cfg::kThreads) void linear_kernel(GemmArgs<T> a) {
+  extern __shared__ __align__(16) char lds[];
+  const int64_t tiles_m = (a.M + Cfg::kBM - 1) / Cfg::kBM;
+  const int64_t per_xcd = (tiles_m + 7) / 8;
+  const int64_t xcd = blockIdx.x & 7;
+  const int64_t local = blockIdx.x >> 3;
+  const int64_t tn = local / per_xcd;
+  const int64_t tm = (local - tn * per_xcd) * 8 + xcd;
+  if (tm >= tiles_m) return;
+  const int64_t m0 = tm * Cfg::kBM;
+  const int64_t n0 = tn * Cfg::kBN;
+  if (EPI == kEpiQkv && n0 >= a.n_split) {
+    gemm_tile<T, Cfg, true, ALIGNED_K>(a, m0, n0, lds);
+  } else {
+    gemm_tile<T, Cfg, false, ALIGNED_K>(a, m0, n0, lds);
+  }
+}
+
+template <typename T, class Cfg, int EPI, bool ALIGNED_K>
+static int launch_kernel(const GemmArgs<T>& a, hipStream_t stream) {
+  const int64_t tiles_m = (a.M + Cfg::kBM - 1) / Cfg::kBM;
+  const int64_t tiles_n = (a.N + Cfg::kBN - 1) / Cfg::kBN;
+  const int64_t wgs = ((tiles_m + 7) / 8) * 8 * tiles_n;
+  if (wgs > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "linear: too many tiles");
+  const int lds_bytes = 2 * Cfg::kBufBytes;
   static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(linear_kernel<T>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       2 * kTileLdsBytes);
+  if (!attr_set && lds_bytes > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(linear_kernel<T, Cfg, EPI, ALIGNED_K>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return fail(NT_ERR_HIP, "linear: %s", hipGetErrorString(e));
     attr_set = true;
   }
-  hipLaunchKernelGGL((linear_kernel<T>), dim3((unsigned)tiles), dim3(256), 2 * kTileLdsBytes,
-                     stream, static_cast<const T*>(A), lda, static_cast<const T*>(W),
-                     static_cast<const T*>(bias), static_cast<T*>(C), ldc, M, N, K);
+  hipLaunchKernelGGL((linear_kernel<T, Cfg, EPI, ALIGNED_K>), dim3((unsigned)wgs),
+                     dim3(Cfg::kThreads), lds_bytes, stream, a);
   return check_launch("linear_kernel");
+}
+
+template <typename T, class Cfg, int EPI>
+static int launch_cfg(const GemmArgs<T>& a, hipStream_t stream) {
+  // the branch-free loads need whole K tiles and at least one row
+  const bool aligned = a.K > 0 && a.K % (Cfg::kRowBytes / (int64_t)sizeof(T)) == 0 && a.M > 0 && a.N > 0;
+  if (aligned) return launch_kernel<T, Cfg, EPI, true>(a, stream);
+  return launch_kernel<T, Cfg, EPI, false>(a, stream);
+}
+
+#ifndef NT_GEMM_CFG
+#define NT_GEMM_CFG 4, 2, 2, 2, 128, 1
+#endif
+typedef GemmCfg<NT_GEMM_CFG> DefaultCfg;
+
+template <typename T>
+static int launch_linear(GemmArgs<T> a, bool qkv, hipStream_t stream) {
+  if (qkv) {
+    if (a.n_split % DefaultCfg::kBN != 0) {
+      return fail(NT_ERR_UNSUPPORTED, "linear: QKV split %lld is not a multiple of the column tile",
+                  (long long)a.n_split);
+    }
+    return launch_cfg<T, DefaultCfg, kEpiQkv>(a, stream);
+  }
+  return launch_cfg<T, DefaultCfg, kEpiPlain>(a, stream);
+}
+
+static int check_linear(const void* A, int64_t lda, const void* W, const void* C, int64_t ldc,
+                        int64_t M, int64_t N, int64_t K) {
+  if (M < 0 || N < 0 || K < 0 || lda < K || ldc < 0) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "linear: bad shape M=%lld N=%lld K=%lld lda=%lld ldc=%lld",
+                (long long)M, (long long)N, (long long)K, (long long)lda, (long long)ldc);
+  }
+  if (M > 0 && N > 0 && (!A || !W || !C)) return fail(NT_ERR_INVALID_ARGUMENT, "linear: NULL pointer");
+  return NT_OK;
+}
+
+template <typename T>
+static GemmArgs<T> make_args(const void* A, int64_t lda, const void* W, const void* bias, void* C,
+                             int64_t ldc, int64_t M, int64_t N, int64_t K) {
+  GemmArgs<T> a;
+  a.A = static_cast<const T*>(A);
+  a.lda = lda;
+  a.W = static_cast<const T*>(W);
+  a.bias = static_cast<const T*>(bias);
+  a.C = static_cast<T*>(C);
+  a.ldc = ldc;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.Vt = nullptr;
+  a.ldvt = 0;
+  a.n_split = N;
+  return a;
 }
 
 }  // namespace nt
@@ -214,17 +389,44 @@ using namespace nt;
 
 extern "C" int nt_linear(const void* A, int64_t lda, const void* W, const void* bias, void* C,
                          int64_t ldc, int64_t M, int64_t N, int64_t K, int dtype, void* stream) {
-  if (M < 0 || N < 0 || K < 0 || lda < K || ldc < N) {
-    return fail(NT_ERR_INVALID_ARGUMENT, "linear: bad shape M=%lld N=%lld K=%lld lda=%lld ldc=%lld",
-                (long long)M, (long long)N, (long long)K, (long long)lda, (long long)ldc);
-  }
+  int rc = check_linear(A, lda, W, C, ldc, M, N, K);
+  if (rc != NT_OK) return rc;
+  if (ldc < N) return fail(NT_ERR_INVALID_ARGUMENT, "linear: ldc %lld < N %lld", (long long)ldc, (long long)N);
   if (M == 0 || N == 0) return NT_OK;
-  if (!A || !W || !C) return fail(NT_ERR_INVALID_ARGUMENT, "linear: NULL pointer");
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case NT_F32: return launch_linear<float>(A, lda, W, bias, C, ldc, M, N, K, s);
-    case NT_F16: return launch_linear<_Float16>(A, lda, W, bias, C, ldc, M, N, K, s);
-    case NT_BF16: return launch_linear<__bf16>(A, lda, W, bias, C, ldc, M, N, K, s);
+    case NT_F32: return launch_linear<float>(make_args<float>(A, lda, W, bias, C, ldc, M, N, K), false, s);
+    case NT_F16: return launch_linear<_Float16>(make_args<_Float16>(A, lda, W, bias, C, ldc, M, N, K), false, s);
+    case NT_BF16: return launch_linear<__bf16>(make_args<__bf16>(A, lda, W, bias, C, ldc, M, N, K), false, s);
     default: return fail(NT_ERR_INVALID_ARGUMENT, "linear: unknown dtype %d", dtype);
   }
+}
+
+extern "C" int nt_linear_qkv(const void* A, int64_t lda, const void* W, const void* bias, void* QK,
+                             int64_t ldqk, void* Vt, int64_t ldvt, int64_t M, int64_t E, int64_t K,
+                             int dtype, void* stream) {
+  int rc = check_linear(A, lda, W, QK, ldqk, M, 3 * E, K);
+  if (rc != NT_OK) return rc;
+  if (ldqk < 2 * E || ldvt < M) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "linear_qkv: ldqk %lld < 2E or ldvt %lld < M",
+                (long long)ldqk, (long long)ldvt);
+  }
+  if (M == 0 || E == 0) return NT_OK;
+  if (!Vt) return fail(NT_ERR_INVALID_ARGUMENT, "linear_qkv: Vt is NULL");
+  hipStream_t s = (hipStream_t)stream;
+#define NT_QKV_CASE(TYPE)                                                       \
+  {                                                                             \
+    GemmArgs<TYPE> a = make_args<TYPE>(A, lda, W, bias, QK, ldqk, M, 3 * E, K); \
+    a.Vt = static_cast<TYPE*>(Vt);                                              \
+    a.ldvt = ldvt;                                                              \
+    a.n_split = 2 * E;                                                          \
+    return launch_linear<TYPE>(a, true, s);                                     \
+  }
+  switch (dtype) {
+    case NT_F32: NT_QKV_CASE(float)
+    case NT_F16: NT_QKV_CASE(_Float16)
+    case NT_BF16: NT_QKV_CASE(__bf16)
+    default: return fail(NT_ERR_INVALID_ARGUMENT, "linear_qkv: unknown dtype %d", dtype);
+  }
+#undef NT_QKV_CASE
 }

@@ -18,7 +18,7 @@ from . import _C
 
 class NestedTensorImpl:
     __slots__ = ("buffer", "sizes", "_opt_sizes", "_sizes_dev", "_offsets_dev",
-                 "_row_offsets_dev", "_max_sizes")
+                 "_row_offsets_dev", "_max_sizes", "_attn_schedule")
 
     def __init__(self, buffer, sizes):
         """buffer: 1-D contiguous tensor; sizes: CPU int64 [B, D], or 0-d for an
@@ -35,6 +35,7 @@ class NestedTensorImpl:
         self._offsets_dev = None
         self._row_offsets_dev = None
         self._max_sizes = None
+        self._attn_schedule = None
 
     # ---- host metadata ----------------------------------------------------
     @property
@@ -106,6 +107,26 @@ class NestedTensorImpl:
             self._row_offsets_dev = device_offsets(first, self.B, 1)
         return self._row_offsets_dev
 
+    def attention_schedule(self, q_tile=128):
+        """Work list of the self-attention kernel, built from the host copy of the
+        nested size and cached on the device: int32 [n_work, 4] rows
+        {first token, length, first query row of the tile, 0}, one per q_tile
+        query rows of every sequence, longest sequences first (they take the
+        most key tiles, so they should start first).  Tiles that do not exist
+        are never listed, hence never launched."""
+        if self._attn_schedule is None:
+            lens = self.sizes[:, 0]
+            starts = torch.cumsum(lens, 0) - lens
+            order = torch.argsort(lens, descending=True, stable=True)
+            lens_o, starts_o = lens[order], starts[order]
+            ntile = (lens_o + q_tile - 1) // q_tile
+            seq = torch.repeat_interleave(torch.arange(lens_o.numel()), ntile)
+            first = torch.cumsum(ntile, 0) - ntile
+            q0 = (torch.arange(int(ntile.sum())) - first[seq]) * q_tile
+            items = torch.stack([starts_o[seq], lens_o[seq], q0, torch.zeros_like(q0)], 1)
+            self._attn_schedule = items.to(torch.int32).contiguous().to(self.buffer.device)
+        return self._attn_schedule
+
     def with_buffer(self, buffer):
         """Same nested size over another buffer; shares the cached metadata when
         the device matches."""
@@ -116,6 +137,7 @@ class NestedTensorImpl:
             out._sizes_dev = self._sizes_dev
             out._offsets_dev = self._offsets_dev
             out._row_offsets_dev = self._row_offsets_dev
+            out._attn_schedule = self._attn_schedule
         return out
 
 

@@ -355,27 +355,51 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
     same = (key is query or key.buffer.data_ptr() == query.buffer.data_ptr()) and \
         (value is query or value.buffer.data_ptr() == query.buffer.data_ptr()) and \
         torch.equal(key.sizes, query.sizes)
-    if same:
-        qkv = linear(xq, W, in_proj_bias)                       # [T, 3E]
-        q_t, k_t, v_t = qkv, qkv, qkv
-        qc, kc, vc = 0, E, 2 * E
-        ld = 3 * E
-        ldq = ldk = ldv = ld
-    else:
-        b = in_proj_bias
-        q_t = linear(xq, W[0:E], None if b is None else b[0:E])
-        k_t = linear(key.buffer.reshape(-1, E), W[E:2 * E], None if b is None else b[E:2 * E])
-        v_t = linear(value.buffer.reshape(-1, E), W[2 * E:], None if b is None else b[2 * E:])
-        qc = kc = vc = 0
-        ldq = ldk = ldv = E
-    attn = torch.empty((xq.size(0), E), dtype=dtype, device=dev)
+    T_tokens = xq.size(0)
     max_q = int(query.sizes[:, 0].max()) if query.B > 0 else 0
-    with torch.cuda.device(dev):
-        _C.check(_C.lib.nt_varlen_attention(
-            _offset_ptr(q_t, qc), ldq, _offset_ptr(k_t, kc), ldk, _offset_ptr(v_t, vc), ldv,
-            _C.ptr(attn), E, _C.ptr(query.row_offsets_dev()), _C.ptr(key.row_offsets_dev()),
-            query.B, num_heads, head_dim, max_q, float(scaling), _C.dtype_code(dtype),
-            _C.current_stream(dev)))
+    attn = torch.empty((T_tokens, E), dtype=dtype, device=dev)
+    fused = same and head_dim == 64 and dtype in (torch.float16, torch.bfloat16) and (2 * E) % 128 == 0
+    if in_proj_bias is not None:
+        in_proj_bias = in_proj_bias.contiguous()
+        if in_proj_bias.dtype != dtype:
+            raise RuntimeError("linear: input, weight and bias must have the same dtype")
+    if W.dtype != dtype:
+        raise RuntimeError("linear: input, weight and bias must have the same dtype")
+    if fused:
+        # self-attention, head_dim 64: Q|K row-major + V transposed straight out of
+        # the projection GEMM, attention reads both without any re-layout pass
+        ldvt = (T_tokens + 72 + 7) // 8 * 8   # rows readable 72 elements past the last token
+        qk = torch.empty((T_tokens, 2 * E), dtype=dtype, device=dev)
+        vt = torch.empty((E, ldvt), dtype=dtype, device=dev)
+        with torch.cuda.device(dev):
+            stream = _C.current_stream(dev)
+            _C.check(_C.lib.nt_linear_qkv(
+                _C.ptr(xq), xq.stride(0), _C.ptr(W), _C.ptr(in_proj_bias), _C.ptr(qk), 2 * E,
+                _C.ptr(vt), ldvt, T_tokens, E, E, _C.dtype_code(dtype), stream))
+            sched = query.attention_schedule()
+            _C.check(_C.lib.nt_varlen_attention_vt(
+                _C.ptr(qk), 2 * E, E, _C.ptr(vt), ldvt, _C.ptr(attn), E,
+                _C.ptr(sched), sched.size(0), num_heads, T_tokens,
+                float(scaling), _C.dtype_code(dtype), stream))
+    else:
+        if same:
+            qkv = linear(xq, W, in_proj_bias)                       # [T, 3E]
+            q_t, k_t, v_t = qkv, qkv, qkv
+            qc, kc, vc = 0, E, 2 * E
+            ldq = ldk = ldv = 3 * E
+        else:
+            b = in_proj_bias
+            q_t = linear(xq, W[0:E], None if b is None else b[0:E])
+            k_t = linear(key.buffer.reshape(-1, E), W[E:2 * E], None if b is None else b[E:2 * E])
+            v_t = linear(value.buffer.reshape(-1, E), W[2 * E:], None if b is None else b[2 * E:])
+            qc = kc = vc = 0
+            ldq = ldk = ldv = E
+        with torch.cuda.device(dev):
+            _C.check(_C.lib.nt_varlen_attention(
+                _offset_ptr(q_t, qc), ldq, _offset_ptr(k_t, kc), ldk, _offset_ptr(v_t, vc), ldv,
+                _C.ptr(attn), E, _C.ptr(query.row_offsets_dev()), _C.ptr(key.row_offsets_dev()),
+                query.B, num_heads, head_dim, max_q, float(scaling), _C.dtype_code(dtype),
+                _C.current_stream(dev)))
     out = linear(attn, out_proj_weight, out_proj_bias)
     return query.with_buffer(out.reshape(-1))
 
