@@ -40,8 +40,11 @@ enum {
   NT_ERR_WORKSPACE = 4
 };
 
-/* element types of the attention path */
-enum { NT_F32 = 0, NT_F16 = 1, NT_BF16 = 2 };
+/* element types: the first three are the types of the attention path */
+enum {
+  NT_F32 = 0, NT_F16 = 1, NT_BF16 = 2,
+  NT_F64 = 3, NT_I8 = 4, NT_U8 = 5, NT_I16 = 6, NT_I32 = 7, NT_I64 = 8
+};
 
 /* No reference counterpart: ABI handshake and error text. */
 int nt_abi_version(void);
@@ -103,12 +106,21 @@ int nt_pack(const void* const* srcs, void* packed, const int64_t* offsets, int64
 /* ---- mask -> nested size, compaction ----------------------------------- */
 
 /* Row statistics of a byte mask viewed as [R, M] (nonzero = true):
- * counts[r] = number of true entries in row r (int32).  One wavefront per row
- * with ballot + popcount.  The reference has no device counterpart: it reads
- * every mask element with .item<bool>() on the host
- * (nestedtensor/csrc/masking.cpp:190-201). */
+ * counts[r] = number of true entries in row r (int32); prefix[r] (may be NULL)
+ * = 1 iff those are exactly the first counts[r] entries of the row.  One
+ * wavefront per row, 16 mask bytes per lane and step, ballot + popcount.  The
+ * reference has no device counterpart: it reads every mask element with
+ * .item<bool>() on the host (nestedtensor/csrc/masking.cpp:190-201). */
 int nt_mask_row_counts(const uint8_t* mask, int64_t R, int64_t M, int32_t* counts,
-                       void* stream);
+                       uint8_t* prefix, void* stream);
+
+/* The same statistics for the mask `data != padding` of a dense tensor viewed as
+ * [R, M] elements of type elem_type, without materialising the mask; the
+ * comparison is the one of the element type (NaN != x is true, -0.0 != 0.0 is
+ * false).  Replaces `mask = (tensor != padding)` followed by the host walk in
+ * nested_tensor_from_padded_tensor (nestedtensor/nested/masking.py:12-14). */
+int nt_value_row_counts(const void* data, int elem_type, double padding, int64_t R, int64_t M,
+                        int32_t* counts, uint8_t* prefix, void* stream);
 
 /* Compaction of the rows of `data` viewed as [R, M, chunk_bytes]: the kept
  * chunks of row r (mask[r, m] != 0) are written, in order, starting at byte

@@ -16,6 +16,8 @@ LIB_PATH = os.path.join(_HERE, "libnestedtensor_amd.so")
 
 NT_OK = 0
 NT_F32, NT_F16, NT_BF16 = 0, 1, 2
+ELEM_TYPE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2, torch.float64: 3, torch.int8: 4,
+             torch.uint8: 5, torch.int16: 6, torch.int32: 7, torch.int64: 8}
 
 _c_void_p = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -36,7 +38,9 @@ SIGNATURES = {
                                  ctypes.POINTER(_i64), _int, _c_void_p]),
     "nt_build_mask": (_int, [_c_void_p, _c_void_p, _i64, _i64, _i64, ctypes.POINTER(_i64), _c_void_p]),
     "nt_pack": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _int, _c_void_p]),
-    "nt_mask_row_counts": (_int, [_c_void_p, _i64, _i64, _c_void_p, _c_void_p]),
+    "nt_mask_row_counts": (_int, [_c_void_p, _i64, _i64, _c_void_p, _c_void_p, _c_void_p]),
+    "nt_value_row_counts": (_int, [_c_void_p, _int, ctypes.c_double, _i64, _i64, _c_void_p, _c_void_p,
+                                   _c_void_p]),
     "nt_compact_rows": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _c_void_p, _c_void_p]),
     "nt_scan_workspace_bytes": (_size_t, [_i64]),
     "nt_exclusive_scan_i32": (_int, [_c_void_p, _i64, _c_void_p, _c_void_p, _size_t, _c_void_p]),

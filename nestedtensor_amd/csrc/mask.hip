@@ -16,19 +16,101 @@ namespace nt {
 
 constexpr int kRowsPerBlock = 4;  // one wavefront per row, 4 rows per workgroup
 
-__global__ __launch_bounds__(kWave * kRowsPerBlock) void mask_row_counts_kernel(
-    const uint8_t* mask, int64_t R, int64_t M, int32_t* counts) {
+// Predicates: a mask byte is kept if non-zero; a data element is kept if it
+// differs from the padding value with the comparison of its type (so NaN != x is
+// true and -0.0 != 0.0 is false, as for `tensor != padding` in torch).
+struct NonZeroByte {
+  typedef uint8_t type;
+  __device__ __forceinline__ bool operator()(uint8_t x) const { return x != 0; }
+};
+template <typename T, typename C>
+struct NotEqual {
+  typedef T type;
+  C pad;
+  __device__ __forceinline__ bool operator()(T x) const { return (C)x != pad; }
+};
+
+// counts[r] = kept entries of row r; prefix[r] = 1 iff the kept entries are
+// exactly the first counts[r] entries of the row.  One wavefront per row; a lane
+// looks at VEC consecutive entries per step (VEC * sizeof(T) == 16 when rows are
+// 16-byte aligned, else 1); ballots over the lanes' "full / non-empty / is a
+// prefix" flags decide prefix-ness without any serial scan.
+template <typename P, int VEC>
+__global__ __launch_bounds__(kWave * kRowsPerBlock) void row_counts_kernel(
+    const typename P::type* __restrict__ data, int64_t R, int64_t M, P pred,
+    int32_t* __restrict__ counts, uint8_t* __restrict__ prefix) {
+  typedef typename P::type T;
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
   if (row >= R) return;
-  const uint8_t* m = mask + row * M;
+  const T* m = data + row * M;
   int32_t count = 0;
-  for (int64_t base = 0; base < M; base += kWave) {
-    const int64_t i = base + lane;
-    const bool keep = (i < M) && (m[i] != 0);
-    count += __popcll(__ballot(keep));
+  bool is_prefix = true;
+  bool ended = false;   // an entry that is not kept has been seen (wave-uniform)
+  for (int64_t base = 0; base < M; base += (int64_t)kWave * VEC) {
+    const int64_t i0 = base + (int64_t)lane * VEC;
+    T v[VEC];
+    if (VEC == 1) {
+      if (i0 < M) v[0] = m[i0];
+    } else {
+      if (i0 + VEC <= M) {
+        u32x4 raw = *reinterpret_cast<const u32x4*>(m + i0);
+        __builtin_memcpy(v, &raw, 16);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          if (i0 + j < M) v[j] = m[i0 + j];
+        }
+      }
+    }
+    uint32_t flags = 0;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      if (i0 + j < M && pred(v[j])) flags |= 1u << j;
+    }
+    const int cnt = __popc(flags);
+    count += cnt;
+    // entries of this lane that exist (the last lanes of the last step hold fewer)
+    int64_t here = M - i0;
+    const int exist = here >= VEC ? VEC : (here > 0 ? (int)here : 0);
+    const uint64_t full = __ballot(cnt == exist && exist > 0);
+    const uint64_t nonempty = __ballot(cnt > 0);
+    const uint64_t lane_ok = __ballot(flags == ((1u << cnt) - 1u));
+    const uint64_t present = __ballot(exist > 0);
+    const int q = __popcll(nonempty);
+    const uint64_t low_q = q >= 64 ? ~0ull : ((1ull << q) - 1ull);
+    const uint64_t low_qm1 = q == 0 ? 0ull : (low_q >> 1);
+    bool ok = (lane_ok == ~0ull) && (nonempty == low_q) && ((full & low_qm1) == low_qm1);
+    if (ended && nonempty != 0) ok = false;
+    is_prefix = is_prefix && ok;
+    if (full != present) ended = true;
   }
-  if (lane == 0) counts[row] = count;
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) count += __shfl_xor(count, off, kWave);
+  if (lane == 0) {
+    counts[row] = count;
+    if (prefix) prefix[row] = is_prefix ? 1 : 0;
+  }
+}
+
+template <typename P>
+static int launch_row_counts(const void* data, int64_t R, int64_t M, P pred, int32_t* counts,
+                             uint8_t* prefix, hipStream_t stream) {
+  typedef typename P::type T;
+  const int64_t blocks = (R + kRowsPerBlock - 1) / kRowsPerBlock;
+  if (blocks > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "row_counts: too many rows");
+  constexpr int kVec = 16 / sizeof(T);
+  const bool aligned = ((uintptr_t)data % 16 == 0) && ((M * (int64_t)sizeof(T)) % 16 == 0);
+  dim3 grid((unsigned)blocks), block(kWave * kRowsPerBlock);
+  const T* d = static_cast<const T*>(data);
+  if (aligned && kVec > 1) {
+    hipLaunchKernelGGL((row_counts_kernel<P, kVec>), grid, block, 0, stream, d, R, M, pred, counts,
+                       prefix);
+  } else {
+    hipLaunchKernelGGL((row_counts_kernel<P, 1>), grid, block, 0, stream, d, R, M, pred, counts,
+                       prefix);
+  }
+  return check_launch("row_counts_kernel");
 }
 
 // UNIT: bytes moved per lane step in the cooperative path (1, 2, 4, 8 or 16).
@@ -101,15 +183,31 @@ static int pick_unit(const void* a, const void* b, int64_t chunk_bytes) {
 using namespace nt;
 
 extern "C" int nt_mask_row_counts(const uint8_t* mask, int64_t R, int64_t M, int32_t* counts,
-                                  void* stream) {
+                                  uint8_t* prefix, void* stream) {
   if (R < 0 || M < 0) return fail(NT_ERR_INVALID_ARGUMENT, "mask_row_counts: negative extent");
   if (R == 0) return NT_OK;
   if (!counts || (M > 0 && !mask)) return fail(NT_ERR_INVALID_ARGUMENT, "mask_row_counts: NULL pointer");
-  const int64_t blocks = (R + kRowsPerBlock - 1) / kRowsPerBlock;
-  if (blocks > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "mask_row_counts: too many rows");
-  hipLaunchKernelGGL(mask_row_counts_kernel, dim3((unsigned)blocks), dim3(kWave * kRowsPerBlock),
-                     0, (hipStream_t)stream, mask, R, M, counts);
-  return check_launch("mask_row_counts_kernel");
+  return launch_row_counts(mask, R, M, NonZeroByte(), counts, prefix, (hipStream_t)stream);
+}
+
+extern "C" int nt_value_row_counts(const void* data, int elem_type, double padding, int64_t R,
+                                   int64_t M, int32_t* counts, uint8_t* prefix, void* stream) {
+  if (R < 0 || M < 0) return fail(NT_ERR_INVALID_ARGUMENT, "value_row_counts: negative extent");
+  if (R == 0) return NT_OK;
+  if (!counts || (M > 0 && !data)) return fail(NT_ERR_INVALID_ARGUMENT, "value_row_counts: NULL pointer");
+  hipStream_t s = (hipStream_t)stream;
+  switch (elem_type) {
+    case NT_F32: return launch_row_counts(data, R, M, NotEqual<float, float>{(float)padding}, counts, prefix, s);
+    case NT_F16: return launch_row_counts(data, R, M, NotEqual<_Float16, float>{(float)padding}, counts, prefix, s);
+    case NT_BF16: return launch_row_counts(data, R, M, NotEqual<__bf16, float>{(float)padding}, counts, prefix, s);
+    case NT_F64: return launch_row_counts(data, R, M, NotEqual<double, double>{padding}, counts, prefix, s);
+    case NT_I8: return launch_row_counts(data, R, M, NotEqual<int8_t, double>{padding}, counts, prefix, s);
+    case NT_U8: return launch_row_counts(data, R, M, NotEqual<uint8_t, double>{padding}, counts, prefix, s);
+    case NT_I16: return launch_row_counts(data, R, M, NotEqual<int16_t, double>{padding}, counts, prefix, s);
+    case NT_I32: return launch_row_counts(data, R, M, NotEqual<int32_t, double>{padding}, counts, prefix, s);
+    case NT_I64: return launch_row_counts(data, R, M, NotEqual<int64_t, double>{padding}, counts, prefix, s);
+    default: return fail(NT_ERR_INVALID_ARGUMENT, "value_row_counts: unknown element type %d", elem_type);
+  }
 }
 
 extern "C" int nt_compact_rows(const void* data, const uint8_t* mask, const int64_t* row_offsets,

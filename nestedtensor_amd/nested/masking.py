@@ -18,8 +18,23 @@ from . import nested
 
 
 def nested_tensor_from_padded_tensor(tensor, nested_dim=1, padding=-1):
-    mask = (tensor != padding)
-    return nested_tensor_from_tensor_mask(tensor, mask, nested_dim)
+    """``nested_tensor_from_tensor_mask(tensor, tensor != padding, nested_dim)``
+    (nested/masking.py:12-14).  On the device the mask is never materialised: the
+    keep-counts are taken straight from the data (nt_value_row_counts)."""
+    if tensor is None:
+        raise RuntimeError("Tensor can't be undefined (None).")
+    if tensor.dim() == 0:
+        raise RuntimeError("Can't construct nested tensor from a scalar.")
+    if nested_dim == 0:
+        raise RuntimeError("Nested dimension can't be 0.")
+    if nested_dim is not None and nested_dim > tensor.dim():
+        raise RuntimeError("Nested dimension ({0}) can't be bigger than data tensor dimension ({1}).".format(
+            nested_dim, tensor.dim()))
+    if not tensor.is_cuda or tensor.dim() < 2 or tensor.numel() < 2 or tensor.dtype not in _C.ELEM_TYPE:
+        mask = (tensor != padding)
+        return nested_tensor_from_tensor_mask(tensor, mask, nested_dim)
+    buffer, sizes = torch.ops.nestedtensor.nt_from_padded_tensor(tensor, float(padding), nested_dim)
+    return nested.NestedTensor(NestedTensorImpl(buffer, sizes)).contiguous()
 
 
 # Constructs nested tensor from passed tensor and mask.
@@ -116,11 +131,24 @@ def _compact(data, bmask, R, M, chunk_elems, total_kept, counts_dev):
 
 
 def _row_counts(bmask, R, M):
+    """Keep-count and is-a-prefix flag per row of a byte mask [R, M]."""
     counts = torch.empty(R, dtype=torch.int32, device=bmask.device)
+    prefix = torch.empty(R, dtype=torch.uint8, device=bmask.device)
     with torch.cuda.device(bmask.device):
         _C.check(_C.lib.nt_mask_row_counts(
-            _C.ptr(bmask), R, M, _C.ptr(counts), _C.current_stream(bmask.device)))
-    return counts
+            _C.ptr(bmask), R, M, _C.ptr(counts), _C.ptr(prefix), _C.current_stream(bmask.device)))
+    return counts, prefix
+
+
+def _value_row_counts(tensor, padding, R, M):
+    """The same for the mask ``tensor != padding`` without building it."""
+    counts = torch.empty(R, dtype=torch.int32, device=tensor.device)
+    prefix = torch.empty(R, dtype=torch.uint8, device=tensor.device)
+    with torch.cuda.device(tensor.device):
+        _C.check(_C.lib.nt_value_row_counts(
+            _C.ptr(tensor), _C.ELEM_TYPE[tensor.dtype], float(padding), R, M, _C.ptr(counts),
+            _C.ptr(prefix), _C.current_stream(tensor.device)))
+    return counts, prefix
 
 
 def _from_mask_native(tensor, mask, nested_dim):
@@ -155,7 +183,7 @@ def _from_mask_native(tensor, mask, nested_dim):
         # true keeps tensor[i] whole; false drops it (0-d mask[i]) or leaves an
         # empty constituent of shape [1, .., 1, 0].
         row_elems = tensor[0].numel() if B > 0 else 0
-        counts = _row_counts(bmask, 1, B)
+        counts, _ = _row_counts(bmask, 1, B)
         kept = int(counts.item())
         keep_host = mask.reshape(B).to(torch.bool).cpu()
         buf = _compact(tensor, bmask, 1, B, row_elems, kept, counts)
@@ -174,15 +202,39 @@ def _from_mask_native(tensor, mask, nested_dim):
             "Mask of shape %s does not match the leading dimensions of the data tensor %s."
             % (tuple(mask.shape), tuple(tensor.shape)))
 
-    # General case.  Rows = everything but the last mask dim.
-    M = mask.size(-1)
-    R = mask.numel() // M if M > 0 else 0
-    rest = list(tensor.shape[mask.dim():])
+    return _from_rows(tensor, mask.dim(), lambda R, M: _row_counts(bmask, R, M), lambda: bmask)
+
+
+def _from_value_native(tensor, padding, nested_dim):
+    """nested_tensor_from_padded_tensor on the device: the mask is
+    ``tensor != padding`` with the dims of the data."""
+    if nested_dim != 1:
+        raise RuntimeError("Only nested_dim of 1 is currently supported.")
+    _C.require_device(tensor, "nested_tensor_from_padded_tensor")
+    tensor = tensor.contiguous()
+    return _from_rows(tensor, tensor.dim(),
+                      lambda R, M: _value_row_counts(tensor, padding, R, M),
+                      lambda: _as_byte_mask(tensor != padding))
+
+
+def _from_rows(tensor, mask_dims, count_rows, byte_mask):
+    """General case of nt_from_tensor_mask (masking.cpp:203-222) for a mask over
+    the first `mask_dims` dims of `tensor`.  Rows = everything but the last mask
+    dim.  `count_rows(R, M)` gives device (counts, prefix flags); `byte_mask()`
+    materialises the mask, which only the non-prefix path needs."""
+    B = tensor.size(0)
+    inner_mask_shape = tuple(tensor.shape[1:mask_dims])
+    M = tensor.size(mask_dims - 1)
+    R = 1
+    for v in tensor.shape[:mask_dims - 1]:
+        R *= v
+    rest = list(tensor.shape[mask_dims:])
     chunk = 1
     for v in rest:
         chunk *= v
-    counts_dev = _row_counts(bmask, R, M)
+    counts_dev, prefix_dev = count_rows(R, M)
     counts = counts_dev.cpu().to(torch.int64).reshape((B,) + inner_mask_shape[:-1])
+    all_prefix = bool(prefix_dev.min().item()) if R > 0 else True
 
     # Nested size from the counts: at every mask level the extent is the number
     # of children that keep anything (masking.cpp:203-222); the selection must
@@ -191,7 +243,10 @@ def _from_mask_native(tensor, mask, nested_dim):
     total = flat.sum(1)
     extents = [flat.max(1).values]
     alive = counts > 0
+    leading = all_prefix            # kept children come first at every level
     while alive.dim() > 1:
+        if leading and alive.size(-1) > 1:
+            leading = bool((alive[..., 1:] <= alive[..., :-1]).all())
         c = alive.sum(-1)
         extents.append(c.reshape(B, -1).max(1).values)
         alive = c > 0
@@ -205,7 +260,12 @@ def _from_mask_native(tensor, mask, nested_dim):
             shapes.append(list(inner_mask_shape[:-1]) + [0])
         else:
             shapes.append([int(v) for v in extents[b]] + rest)
-    buf = _compact(tensor, bmask, R, M, chunk, int(total.sum()), counts_dev)
+    if leading:
+        # Every constituent keeps a leading box: this is the length-based un-pad
+        # (nt_remove_padding) with the nested size just derived.
+        target = _impl_from_shapes(torch.empty(0, dtype=tensor.dtype, device=tensor.device), shapes)
+        return ops.from_padded_tensor(tensor, target)
+    buf = _compact(tensor, byte_mask(), R, M, chunk, int(total.sum()), counts_dev)
     return _impl_from_shapes(buf, shapes)
 
 
@@ -232,3 +292,14 @@ def _nt_from_tensor_mask_op(tensor, mask, nested_dim):
 # wrapper, so it returns the lowered pair (packed buffer, sizes[B, D]) that
 # nt_from_tensor_mask() above wraps; sizes is 0-d for an empty result.
 ops._lib.impl("nt_from_tensor_mask", _nt_from_tensor_mask_op, "CompositeExplicitAutograd")
+
+
+def _nt_from_padded_tensor_op(tensor, padding, nested_dim):
+    impl = _from_value_native(tensor, padding, nested_dim)
+    return impl.buffer, impl.sizes
+
+
+# No counterpart among the reference's ops (it builds the mask in Python,
+# nested/masking.py:12-14); same lowered return convention as above.
+ops._lib.define("nt_from_padded_tensor(Tensor tensor, float padding, int nested_dim) -> (Tensor, Tensor)")
+ops._lib.impl("nt_from_padded_tensor", _nt_from_padded_tensor_op, "CompositeExplicitAutograd")

@@ -258,6 +258,8 @@ def from_padded_tensor(padded, target):
     out = torch.empty(target.numel(), dtype=padded.dtype, device=dev)
     res = target.with_buffer(out)
     eb = _elem_bytes(padded.dtype)
+    if out.numel() == 0:
+        return res
     with torch.cuda.device(dev):
         _C.check(_C.lib.nt_remove_padding(
             _C.ptr(padded), _C.ptr(out), _C.ptr(res.offsets_dev()), _C.ptr(res.sizes_dev()),

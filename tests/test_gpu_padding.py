@@ -352,3 +352,71 @@ def test_config_c2_images_tensor_mask_round_trip():
     exp_parts = oracle.nt_from_tensor_mask_vectorised(exp_d, exp_m.to(torch.bool))
     nt_matches(back, exp_parts, torch.float32)
     nt_matches(back, parts, torch.float32)
+
+
+# ---- row statistics kernels (C ABI level) -------------------------------------------
+
+def _cpu_counts_prefix(keep):
+    counts = keep.sum(1).to(torch.int32)
+    M = keep.size(1)
+    idx = torch.arange(M).unsqueeze(0)
+    prefix = (keep == (idx < counts.unsqueeze(1))).all(1).to(torch.uint8)
+    return counts, prefix
+
+
+@pytest.mark.parametrize("M", [1, 7, 16, 33, 64, 100, 1024, 1029, 4096])
+def test_mask_row_counts_and_prefix_flags(M):
+    g = torch.Generator().manual_seed(M)
+    R = 37
+    keep = torch.zeros(R, M, dtype=torch.bool)
+    for r in range(R):
+        kind = r % 4
+        n = int(torch.randint(0, M + 1, (1,), generator=g))
+        if kind == 0:
+            keep[r, :n] = True                                   # prefix
+        elif kind == 1:
+            keep[r] = torch.rand(M, generator=g) < 0.5           # random subset
+        elif kind == 2:
+            keep[r, :n] = True
+            if M > 1:
+                keep[r, int(torch.randint(0, M, (1,), generator=g))] ^= True   # prefix with one flip
+        else:
+            keep[r, M - n:] = True                               # suffix
+    exp_c, exp_p = _cpu_counts_prefix(keep)
+    mask = keep.to(DEV).view(torch.uint8)
+    counts = torch.empty(R, dtype=torch.int32, device=DEV)
+    prefix = torch.empty(R, dtype=torch.uint8, device=DEV)
+    _C.check(_C.lib.nt_mask_row_counts(_C.ptr(mask), R, M, _C.ptr(counts), _C.ptr(prefix), _C.current_stream(DEV)))
+    assert torch.equal(counts.cpu(), exp_c)
+    assert torch.equal(prefix.cpu(), exp_p)
+    # value mode on the same pattern: kept = 1.5, dropped = padding (-1)
+    for dtype in (torch.float16, torch.float32, torch.bfloat16, torch.int64, torch.float64):
+        data = torch.where(keep, torch.tensor(3, dtype=dtype), torch.tensor(-1, dtype=dtype)).to(DEV)
+        _C.check(_C.lib.nt_value_row_counts(_C.ptr(data), _C.ELEM_TYPE[dtype], -1.0, R, M, _C.ptr(counts),
+                                            _C.ptr(prefix), _C.current_stream(DEV)))
+        assert torch.equal(counts.cpu(), exp_c), dtype
+        assert torch.equal(prefix.cpu(), exp_p), dtype
+
+
+def test_from_padded_value_comparison_semantics():
+    # `tensor != padding` of torch: NaN is kept, -0.0 equals the padding 0.0
+    t = torch.tensor([[1.0, float("nan"), 0.0, 0.0], [2.0, -0.0, 0.0, 0.0], [3.0, 4.0, 5.0, 6.0]])
+    exp = oracle.nested_tensor_from_padded_tensor(t, padding=0.0)
+    got = nt.nested_tensor_from_padded_tensor(t.to(DEV), padding=0.0)
+    assert got.nested_size().unbind() == exp.nested_size()
+    bits_equal(got._impl.buffer, exp.buffer)
+
+
+def test_from_padded_value_non_prefix_takes_compaction_path():
+    t = torch.tensor([[[1.0, -1.0, 2.0, -1.0], [3.0, -1.0, 4.0, -1.0]],
+                      [[5.0, 6.0, -1.0, -1.0], [7.0, 8.0, -1.0, -1.0]]])
+    exp = oracle.nested_tensor_from_padded_tensor(t)
+    got = nt.nested_tensor_from_padded_tensor(t.to(DEV))
+    assert got.nested_size().unbind() == exp.nested_size()
+    bits_equal(got._impl.buffer, exp.buffer)
+    # rows that are dropped in the middle: kept children are not leading
+    t2 = torch.tensor([[[1.0, 2.0], [-1.0, -1.0], [3.0, 4.0]]])
+    exp2 = oracle.nested_tensor_from_padded_tensor(t2)
+    got2 = nt.nested_tensor_from_padded_tensor(t2.to(DEV))
+    assert got2.nested_size().unbind() == exp2.nested_size()
+    bits_equal(got2._impl.buffer, exp2.buffer)
