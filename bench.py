@@ -17,7 +17,10 @@ The same JSON line carries
   cpu_baseline - the CPU oracle (the reference's CPU algorithm restated) timed on
                  a bounded sample of the same workload on the host cores;
   mha          - nested BERT-base self-attention (configuration C3) tokens/s and
-                 its MFMA roofline fraction.
+                 its MFMA roofline fraction;
+  rows         - the remaining rows of the path (to_tensor_mask, to_mask,
+                 nested_tensor_from_tensor_mask / _from_padded_tensor, pack, the
+                 offsets scan, C4 attention) on configurations C1, C2 and C4.
 """
 
 import argparse
@@ -50,6 +53,7 @@ def parse():
     ap.add_argument("--batch", type=int, default=4096, help="constituents in total (C5: 4096)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-mha", action="store_true", help="skip the C3 attention leg")
+    ap.add_argument("--no-rows", action="store_true", help="skip the per-row measurements (C1, C2, C4)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="one plain copy of known size, then one pad and one un-pad launch of the "
                          "first C5 chunk; meant to run under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
@@ -287,6 +291,132 @@ def bench_mha_c3(args, torch, dev):
     return res
 
 
+def _time_gpu(torch, fn, iters=20, warmup=3):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def _time_cpu(fn, runs=2):
+    best = None
+    for _ in range(runs):
+        t0 = time.perf_counter()
+        fn()
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    return best * 1e3
+
+
+def bench_rows(args, torch, dev):
+    """The other rows of the hot path, each on the BASELINE configuration that
+    exercises it, through the package's Python surface (so allocation of the
+    result and, for dense -> nested, the device-to-host copy of the row counts
+    are inside the timed region).  GB/s = algorithmic bytes / time."""
+    import nestedtensor_amd as nt
+    import oracle
+    from nestedtensor_amd import _C
+    from nestedtensor_amd.impl import device_offsets
+    rows = {}
+    cpu = not args.no_cpu
+    if cpu:
+        torch.set_num_threads(os.cpu_count() or 1)
+
+    def entry(ms, nbytes, cpu_ms=None, **kw):
+        d = dict(ms=ms, GBps=nbytes / (ms * 1e-3) / 1e9, frac_of_hbm_peak=nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                 algorithmic_bytes=nbytes)
+        if cpu_ms is not None:
+            d["cpu_oracle_ms"] = cpu_ms
+            d["cpu_oracle_GBps"] = nbytes / (cpu_ms * 1e-3) / 1e9
+        d.update(kw)
+        return d
+
+    # ---- C1: 64 fp32 [L_i, 256], round trip ---------------------------------
+    g = torch.Generator().manual_seed(1010 + 0)
+    lengths = torch.randint(1, 129, (64,), generator=g)
+    lengths[0] = 128
+    parts = [torch.randn(int(l), 256, generator=g) for l in lengths]
+    a = nt.nested_tensor(parts, device=dev)
+    ref = oracle.ref_nested_tensor(parts)
+    nvalid, npadded = a.numel(), 64 * 128 * 256
+    padded = a.to_padded_tensor(-1e30)
+    ms_pad = _time_gpu(torch, lambda: a.to_padded_tensor(0))
+    ms_back = _time_gpu(torch, lambda: nt.nested_tensor_from_padded_tensor(padded, padding=-1e30))
+    ms_len = _time_gpu(torch, lambda: nt.from_padded_tensor(padded, a))
+    back = nt.nested_tensor_from_padded_tensor(padded, padding=-1e30)
+    assert torch.equal(back._impl.buffer.view(torch.int32).cpu(), ref.buffer.view(torch.int32))
+    c_pad = c_back = None
+    if cpu:
+        cp = oracle.to_padded_tensor(ref, -1e30)
+        c_pad = _time_cpu(lambda: oracle.to_padded_tensor(ref, 0), 3)
+        c_back = _time_cpu(lambda: oracle.from_padded_tensor(cp, ref), 3)
+    rows["C1_to_padded_tensor"] = entry(ms_pad, 4 * (nvalid + npadded), c_pad)
+    rows["C1_nested_tensor_from_padded_tensor"] = entry(
+        ms_back, 4 * (npadded + 2 * nvalid), None,
+        note="value-based; includes the device-to-host copy of the row counts")
+    rows["C1_from_padded_tensor_length_based"] = entry(ms_len, 4 * 2 * nvalid, c_back)
+
+    # ---- C2: 16 fp32 images [3, H_i, W_i] -----------------------------------
+    g = torch.Generator().manual_seed(1010 + 1)
+    hw = torch.randint(480, 1025, (16, 2), generator=g)
+    imgs = [torch.rand(3, int(h), int(w), generator=g) for h, w in hw]
+    a2 = nt.nested_tensor(imgs, device=dev)
+    nvalid2 = a2.numel()
+    mx = a2._impl.max_sizes()
+    npadded2 = 16 * mx[0] * mx[1] * mx[2]
+    data, mask = a2.to_tensor_mask()
+    ms_tm = _time_gpu(torch, lambda: a2.to_tensor_mask())
+    ms_m = _time_gpu(torch, lambda: torch.ops.nestedtensor.to_mask(a2, 4))
+    ms_fm = _time_gpu(torch, lambda: nt.nested_tensor_from_tensor_mask(data, mask), iters=10)
+    dev_imgs = [p.to(dev) for p in imgs]
+    ms_pack = _time_gpu(torch, lambda: nt.nested_tensor(dev_imgs, device=dev), iters=10)
+    back2 = nt.nested_tensor_from_tensor_mask(data, mask)
+    assert torch.equal(back2._impl.buffer, a2._impl.buffer)
+    c_tm = c_fm = None
+    if cpu:
+        ref2 = oracle.ref_nested_tensor(imgs)
+        c_tm = _time_cpu(lambda: oracle.to_tensor_mask(ref2), 1)
+        dcpu, mcpu = data.cpu(), mask.cpu()
+        c_fm = _time_cpu(lambda: oracle.nt_from_tensor_mask_vectorised(dcpu, mcpu), 1)
+    rows["C2_to_tensor_mask"] = entry(ms_tm, 4 * (nvalid2 + npadded2) + npadded2, c_tm)
+    rows["C2_to_mask"] = entry(ms_m, npadded2)
+    rows["C2_nested_tensor_from_tensor_mask"] = entry(
+        ms_fm, npadded2 + 2 * 4 * nvalid2, c_fm,
+        note="includes the device-to-host copy of the row counts; CPU figure is the vectorised "
+             "restatement, the reference's literal walk does one host call per mask element")
+    rows["C2_nested_tensor_pack_from_device_tensors"] = entry(ms_pack, 2 * 4 * nvalid2)
+
+    # ---- metadata scan --------------------------------------------------------
+    sizes = torch.randint(1, 2049, (4096, 2), dtype=torch.int64).to(dev)
+    ms_scan = _time_gpu(torch, lambda: device_offsets(sizes, 4096, 2))
+    rows["offsets_scan_B4096"] = dict(ms=ms_scan)
+
+    # ---- C4: bt_min_mha bf16, high raggedness ---------------------------------
+    g = torch.Generator().manual_seed(1010 + 3)
+    raw = torch.empty(128).exponential_(1.0 / 96.0, generator=g)
+    lens = [int(v) for v in raw.round().clamp(8, 512)]
+    E, H = 1024, 16
+    xs = [torch.randn(L, E, generator=g).bfloat16() for L in lens]
+    W_in = (torch.randn(3 * E, E, generator=g) * 0.02).bfloat16().to(dev)
+    W_out = (torch.randn(E, E, generator=g) * 0.02).bfloat16().to(dev)
+    b_in, b_out = torch.zeros(3 * E).bfloat16().to(dev), torch.zeros(E).bfloat16().to(dev)
+    a4 = nt.nested_tensor(xs, device=dev, dtype=torch.bfloat16)
+    ms4 = _time_gpu(torch, lambda: torch.ops.nestedtensor.bt_min_mha(
+        H, 64, 0.0, False, a4, a4, a4, W_in, b_in, 64 ** -0.5, W_out, b_out), iters=50, warmup=5)
+    T4 = sum(lens)
+    fl4 = 8 * T4 * E * E + 4 * E * sum(L * L for L in lens)
+    rows["C4_bt_min_mha_bf16"] = dict(ms=ms4, tokens=T4, tokens_per_s=T4 / (ms4 * 1e-3), flops=fl4,
+                                      TFLOPs=fl4 / (ms4 * 1e-3) / 1e12,
+                                      frac_of_mfma_peak=fl4 / (ms4 * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS)
+    return rows
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -326,6 +456,8 @@ def main():
     }
     if not args.no_mha:
         line["mha"] = bench_mha_c3(args, torch, dev)
+    if not args.no_rows:
+        line["rows"] = bench_rows(args, torch, dev)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_c5(torch)
     print(json.dumps(line))

@@ -101,12 +101,11 @@ __device__ __forceinline__ int64_t row_index() { return blockIdx.x; }
 
 // Cooperative move of one row: bytes [0, valid) come from s, bytes [valid, total)
 // are padding.  Called by every workgroup of the row's grid.y column.
-template <int EB, int MODE>
+template <int EB, int MODE, int kThreads>
 __device__ __forceinline__ void move_row(char* d, const char* s, int64_t valid, int64_t total,
                                          const u32x4 pad) {
-  constexpr int kThreads = 256;
   constexpr int kUnroll = NT_ROW_UNROLL;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x & (kThreads - 1);   // 256: the workgroup, 64: one wavefront
 
   int64_t head = (int64_t)((0 - (uintptr_t)d) & 15);
   if (head > total) head = total;
@@ -168,15 +167,18 @@ __device__ __forceinline__ void move_row(char* d, const char* s, int64_t valid, 
   }
 }
 
-template <int EB, int MODE>
+// WAVE_ROWS: rows of at most 1 KiB -- every wavefront of the workgroup takes a row
+// of its own (4 rows per workgroup) instead of 192 lanes idling on one row.
+template <int EB, int MODE, bool WAVE_ROWS>
 __global__ __launch_bounds__(256) void row_kernel(RowParams p) {
-  const int64_t row = row_index();
+  constexpr int kT = WAVE_ROWS ? 64 : 256;
+  const int64_t row = WAVE_ROWS ? row_index() * 4 + (threadIdx.x >> 6) : row_index();
   if (row >= p.nrows) return;
   if (MODE == kPack) {
     const int64_t off = p.offsets[row];
     const int64_t n = (p.offsets[row + 1] - off) * EB;
-    move_row<EB, kUnpad>(p.dst + off * EB, reinterpret_cast<const char*>(p.srcs[row]), n, n,
-                         p.pad);
+    move_row<EB, kUnpad, kT>(p.dst + off * EB, reinterpret_cast<const char*>(p.srcs[row]), n, n,
+                             p.pad);
     return;
   }
   int64_t b, src_off = 0, last;
@@ -206,14 +208,14 @@ __global__ __launch_bounds__(256) void row_kernel(RowParams p) {
   const int64_t row_bytes = Mlast * p.inner * EB;
   const int64_t valid = inside ? last * p.inner * EB : 0;
   if (MODE == kOnes) {
-    move_row<EB, kOnes>(p.dst + row * row_bytes, nullptr, valid, row_bytes, p.pad);
+    move_row<EB, kOnes, kT>(p.dst + row * row_bytes, nullptr, valid, row_bytes, p.pad);
   } else {
     const int64_t packed_byte = (p.offsets[b] + src_off * p.inner) * EB;
     if (MODE == kPad) {
-      move_row<EB, kPad>(p.dst + row * row_bytes, p.src + packed_byte, valid, row_bytes, p.pad);
+      move_row<EB, kPad, kT>(p.dst + row * row_bytes, p.src + packed_byte, valid, row_bytes, p.pad);
     } else {
       if (valid > 0) {
-        move_row<EB, kUnpad>(p.dst + packed_byte, p.src + row * row_bytes, valid, valid, p.pad);
+        move_row<EB, kUnpad, kT>(p.dst + packed_byte, p.src + row * row_bytes, valid, valid, p.pad);
       }
     }
   }
@@ -242,38 +244,45 @@ static u32x4 replicate_pad(int eb, uint64_t bits) {
   return r;
 }
 
-template <int MODE>
-static int launch_rows(int eb, const RowParams& p, int64_t max_row_bytes, hipStream_t stream) {
-  if (p.nrows == 0 || max_row_bytes == 0) return NT_OK;
-  if (p.nrows > 0x7fffffffLL) {
-    return fail(NT_ERR_UNSUPPORTED, "row count %lld exceeds the grid limit", (long long)p.nrows);
-  }
-  const int64_t tile_bytes = 256 * NT_ROW_UNROLL * 16;
+template <int MODE, bool WAVE_ROWS>
+static int launch_rows_t(int eb, const RowParams& p, int64_t max_row_bytes, hipStream_t stream) {
+  const int64_t grid_rows = WAVE_ROWS ? (p.nrows + 3) / 4 : p.nrows;
+  const int64_t tile_bytes = (WAVE_ROWS ? 64 : 256) * NT_ROW_UNROLL * 16;
   int64_t tiles = (max_row_bytes + tile_bytes - 1) / tile_bytes;
-  // Enough workgroups to fill 256 CUs several times over, but long rows are
+  // Enough workgroups to fill 256 CUs many times over, but very long rows are
   // walked by a bounded number of workgroups that each loop over tiles.
-  int64_t y_cap = (int64_t)NT_ROW_TARGET_WGS / p.nrows;
+  int64_t y_cap = (int64_t)NT_ROW_TARGET_WGS / grid_rows;
   if (y_cap < 1) y_cap = 1;
   const int64_t max_tiles = (MODE == kPad || MODE == kOnes) ? NT_ROW_MAX_TILES_PAD : NT_ROW_MAX_TILES_UNPAD;
   if (y_cap > max_tiles) y_cap = max_tiles;
   int64_t gy = tiles < y_cap ? tiles : y_cap;
   if (gy < 1) gy = 1;
 #if NT_ROW_TILE_FAST
-  const int64_t gz = (p.nrows + 65534) / 65535;
+  const int64_t gz = (grid_rows + 65534) / 65535;
   if (gz > 65535) return fail(NT_ERR_UNSUPPORTED, "row count %lld exceeds the grid limit", (long long)p.nrows);
-  dim3 grid((unsigned)gy, (unsigned)(p.nrows < 65535 ? p.nrows : 65535), (unsigned)gz);
+  dim3 grid((unsigned)gy, (unsigned)(grid_rows < 65535 ? grid_rows : 65535), (unsigned)gz);
 #else
-  dim3 grid((unsigned)p.nrows, (unsigned)gy, 1);
+  dim3 grid((unsigned)grid_rows, (unsigned)gy, 1);
 #endif
   dim3 block(256, 1, 1);
   switch (eb) {
-    case 1: hipLaunchKernelGGL((row_kernel<1, MODE>), grid, block, 0, stream, p); break;
-    case 2: hipLaunchKernelGGL((row_kernel<2, MODE>), grid, block, 0, stream, p); break;
-    case 4: hipLaunchKernelGGL((row_kernel<4, MODE>), grid, block, 0, stream, p); break;
-    case 8: hipLaunchKernelGGL((row_kernel<8, MODE>), grid, block, 0, stream, p); break;
+    case 1: hipLaunchKernelGGL((row_kernel<1, MODE, WAVE_ROWS>), grid, block, 0, stream, p); break;
+    case 2: hipLaunchKernelGGL((row_kernel<2, MODE, WAVE_ROWS>), grid, block, 0, stream, p); break;
+    case 4: hipLaunchKernelGGL((row_kernel<4, MODE, WAVE_ROWS>), grid, block, 0, stream, p); break;
+    case 8: hipLaunchKernelGGL((row_kernel<8, MODE, WAVE_ROWS>), grid, block, 0, stream, p); break;
     default: return fail(NT_ERR_INVALID_ARGUMENT, "elem_bytes must be 1, 2, 4 or 8, got %d", eb);
   }
   return check_launch("row_kernel");
+}
+
+template <int MODE>
+static int launch_rows(int eb, const RowParams& p, int64_t max_row_bytes, hipStream_t stream) {
+  if (p.nrows == 0 || max_row_bytes == 0) return NT_OK;
+  if (p.nrows > 0x7fffffffLL) {
+    return fail(NT_ERR_UNSUPPORTED, "row count %lld exceeds the grid limit", (long long)p.nrows);
+  }
+  if (max_row_bytes <= 1024 && MODE != kPack) return launch_rows_t<MODE, true>(eb, p, max_row_bytes, stream);
+  return launch_rows_t<MODE, false>(eb, p, max_row_bytes, stream);
 }
 
 // Fills the geometry shared by pad / unpad / mask from the host-side extents.

@@ -233,8 +233,13 @@ def _from_rows(tensor, mask_dims, count_rows, byte_mask):
     for v in rest:
         chunk *= v
     counts_dev, prefix_dev = count_rows(R, M)
-    counts = counts_dev.cpu().to(torch.int64).reshape((B,) + inner_mask_shape[:-1])
-    all_prefix = bool(prefix_dev.min().item()) if R > 0 else True
+    # one device-to-host copy: the row counts plus "every row keeps a prefix"
+    if R > 0:
+        host = torch.cat([counts_dev, prefix_dev.min().to(torch.int32).reshape(1)]).cpu()
+        counts, all_prefix = host[:-1], bool(host[-1])
+    else:
+        counts, all_prefix = counts_dev.cpu(), True
+    counts = counts.to(torch.int64).reshape((B,) + inner_mask_shape[:-1])
 
     # Nested size from the counts: at every mask level the extent is the number
     # of children that keep anything (masking.cpp:203-222); the selection must
