@@ -295,15 +295,20 @@ __global__ __launch_bounds__(256) void varlen_attention_kernel(
 template <typename T>
 __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt_kernel(
     const T* __restrict__ QK, int64_t ldqk, int64_t k_col, const T* __restrict__ Vt, int64_t ldvt,
-    T* __restrict__ O, int64_t ldo, const int4* __restrict__ schedule, float scale_log2e) {
+    T* __restrict__ O, int64_t ldo, const int4* __restrict__ schedule, unsigned num_heads,
+    float scale_log2e) {
   typedef AttnT<T> AT;
   typedef typename AT::Frag Frag;
 
   __shared__ __align__(16) char lds_k[2][kKBytes];
   __shared__ __align__(16) char lds_v[2][kVBytes];
 
-  const int4 item = schedule[blockIdx.x];
-  const int h = blockIdx.y;
+  // Head fastest: the schedule lists the longest sequences first, and this way
+  // their items of ALL heads are dispatched before any short item (with the
+  // item index fastest, the long items of the last heads would start last and
+  // run alone at the end).
+  const int h = (int)(blockIdx.x % num_heads);
+  const int4 item = schedule[blockIdx.x / num_heads];
   const int64_t begin = item.x;
   const int L = item.y;
   const int q0 = item.z;
@@ -390,6 +395,8 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
   for (int t = 0; t < ntiles; ++t) {
     const int buf = t & 1;
     gload(t + 1);   // past the end: re-reads the last tile, never stored
+    // keep the loads above the MFMA / softmax work (the scheduler would sink them)
+    __builtin_amdgcn_sched_barrier(0);
 
     if (wave_active) {
       acc16 s_acc[2];
@@ -446,10 +453,14 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
         }
       }
       l_run = l_run * alpha + l_tile;
+      // the running maxima settle after the first tiles; then alpha is 1 in
+      // every lane and the 32 multiplications are skipped (wavefront-uniform)
+      if (__any(alpha != 1.0f)) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+          for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+      }
 
       // O^T += V^T P^T
 #pragma unroll
@@ -656,7 +667,10 @@ extern "C" int nt_varlen_attention_vt(const void* qk, int64_t ldqk, int64_t k_co
     return fail(NT_ERR_INVALID_ARGUMENT,
                 "attention_vt: row strides too small (ldvt must be >= total_tokens + 72)");
   }
-  dim3 grid((unsigned)n_work, (unsigned)num_heads, 1);
+  if (n_work * num_heads > 0x7fffffffLL) {
+    return fail(NT_ERR_UNSUPPORTED, "attention_vt: too many workgroups");
+  }
+  dim3 grid((unsigned)(n_work * num_heads), 1, 1);
   const float scale_log2e = scale * 1.4426950408889634f;
   hipStream_t s = (hipStream_t)stream;
   const int4* sched = reinterpret_cast<const int4*>(schedule);
@@ -664,11 +678,11 @@ extern "C" int nt_varlen_attention_vt(const void* qk, int64_t ldqk, int64_t k_co
     hipLaunchKernelGGL((varlen_attention_vt_kernel<_Float16>), grid, dim3(256), 0, s,
                        static_cast<const _Float16*>(qk), ldqk, k_col,
                        static_cast<const _Float16*>(vt), ldvt, static_cast<_Float16*>(out), ldo,
-                       sched, scale_log2e);
+                       sched, (unsigned)num_heads, scale_log2e);
   } else if (dtype == NT_BF16) {
     hipLaunchKernelGGL((varlen_attention_vt_kernel<__bf16>), grid, dim3(256), 0, s,
                        static_cast<const __bf16*>(qk), ldqk, k_col, static_cast<const __bf16*>(vt),
-                       ldvt, static_cast<__bf16*>(out), ldo, sched, scale_log2e);
+                       ldvt, static_cast<__bf16*>(out), ldo, sched, (unsigned)num_heads, scale_log2e);
   } else {
     return fail(NT_ERR_UNSUPPORTED, "attention_vt: dtype must be f16 or bf16");
   }

@@ -9,10 +9,15 @@
 // 32x32 MFMA blocks (fp32 accumulate; f16 / bf16: v_mfma_f32_32x32x16_*, fp32:
 // v_mfma_f32_32x32x2_f32).  K is walked in tiles of BKB bytes per row,
 // double-buffered in LDS; LDS rows are padded by 16 bytes so that the 128-bit
-// fragment reads of 16 consecutive lanes fall into distinct banks.
+// fragment reads of 16 consecutive lanes fall into distinct banks.  Global
+// loads run ahead of the MFMAs through registers, because one K tile of MFMA
+// work is far shorter than the L2 / HBM latency.
 //
-// Global loads run PF K-tiles ahead of the MFMAs (register staging), because one
-// K-tile of MFMA work is far shorter than the L2 / HBM latency.
+// Three tile shapes are compiled (256x128, 256x192, 256x256, eight wavefronts
+// each); the launcher picks per problem the one with the least rounds x tile
+// cost over the CUs.  The bigger tiles read less LDS per MFMA and win once the
+// grid is several rounds deep; the smaller ones quantise better on the
+// projection shapes of one attention layer.
 //
 // Epilogues:
 //   plain  - C row-major + bias;
@@ -23,6 +28,14 @@
 //            operands, which leaves C^T in the accumulators and keeps the
 //            stores coalesced.
 #include "nt_common.h"
+
+// Compile-time tuning knobs.
+#ifndef NT_GEMM_WAVES_PER_EU
+#define NT_GEMM_WAVES_PER_EU 2           // wavefronts per SIMD the kernels are compiled for
+#endif
+#ifndef NT_GEMM_FORCE_CFG
+#define NT_GEMM_FORCE_CFG (-1)           // 0, 1, 2: always that tile shape (experiments)
+#endif
 
 namespace nt {
 
@@ -154,97 +167,145 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
   const int64_t nk = (a.K + kBK - 1) / kBK;
   u32x4 stage[PF][Cfg::kPerThread];
 
-  auto gload = [&](int slot, int64_t kt_in) {
-    // with ALIGNED_K tiles past the end re-read the last tile (never consumed)
-    const int64_t kt = (ALIGNED_K && kt_in >= nk) ? nk - 1 : kt_in;
-#pragma unroll
-    for (int i = 0; i < Cfg::kPerA; ++i) {
-      const int c = tid + i * Cfg::kThreads;
+  if (ALIGNED_K) {
+    // Straight-line K loop (loads past the last K tile re-read it and are never
+    // consumed).  Every k-step issues, in this order: the LDS fragment reads of the
+    // NEXT k-step, its own MFMAs, and its share of the LDS stores of K tile kt + 1
+    // and of the global loads of K tile kt + 2.  The matrix pipe runs the MFMAs
+    // asynchronously, so the LDS and memory instructions behind them execute in
+    // their shadow; issued as one block after the barrier they would run while
+    // no wavefront of the workgroup has MFMAs in flight.
+    constexpr int kN = Cfg::kPerThread;
+    auto gload_one = [&](int slot, int i, int64_t kt_in) {
+      const int64_t kt = kt_in >= nk ? nk - 1 : kt_in;
+      const bool is_a = i < Cfg::kPerA;
+      const int c = tid + (is_a ? i : i - Cfg::kPerA) * Cfg::kThreads;
       const int row = c / Cfg::kChunksPerRow;
-      const int cc = c % Cfg::kChunksPerRow;
-      stage[slot][i] = load_chunk<T, ALIGNED_K>(a.A, a.lda, m0 + row, a.M, kt * kBK + cc * kPer, a.K);
-    }
-#pragma unroll
-    for (int i = 0; i < Cfg::kPerB; ++i) {
-      const int c = tid + i * Cfg::kThreads;
-      const int row = c / Cfg::kChunksPerRow;
-      const int cc = c % Cfg::kChunksPerRow;
-      stage[slot][Cfg::kPerA + i] =
-          load_chunk<T, ALIGNED_K>(a.W, a.K, n0 + row, a.N, kt * kBK + cc * kPer, a.K);
-    }
-  };
-  auto lstore = [&](int slot, int buf) {
-    char* base = lds + buf * Cfg::kBufBytes;
-#pragma unroll
-    for (int i = 0; i < Cfg::kPerA; ++i) {
-      const int c = tid + i * Cfg::kThreads;
-      store16(base + (c / Cfg::kChunksPerRow) * Cfg::kLdsRow + (c % Cfg::kChunksPerRow) * 16,
+      const int64_t k = kt * kBK + (c % Cfg::kChunksPerRow) * kPer;
+      stage[slot][i] = is_a ? load_chunk<T, true>(a.A, a.lda, m0 + row, a.M, k, a.K)
+                            : load_chunk<T, true>(a.W, a.K, n0 + row, a.N, k, a.K);
+    };
+    auto lstore_one = [&](int slot, int i, int buf) {
+      const bool is_a = i < Cfg::kPerA;
+      const int c = tid + (is_a ? i : i - Cfg::kPerA) * Cfg::kThreads;
+      const int row = (is_a ? 0 : Cfg::kBM) + c / Cfg::kChunksPerRow;
+      store16(lds + buf * Cfg::kBufBytes + row * Cfg::kLdsRow + (c % Cfg::kChunksPerRow) * 16,
               stage[slot][i]);
-    }
-#pragma unroll
-    for (int i = 0; i < Cfg::kPerB; ++i) {
-      const int c = tid + i * Cfg::kThreads;
-      store16(base + (Cfg::kBM + c / Cfg::kChunksPerRow) * Cfg::kLdsRow +
-                  (c % Cfg::kChunksPerRow) * 16,
-              stage[slot][Cfg::kPerA + i]);
-    }
-  };
-  auto compute = [&](int buf) {
-    const char* a_base = lds + buf * Cfg::kBufBytes + (wm * WM * 32 + l32) * Cfg::kLdsRow;
-    const char* b_base =
-        lds + buf * Cfg::kBufBytes + (Cfg::kBM + wn * WN * 32 + l32) * Cfg::kLdsRow;
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s) {
+    };
+    auto read_frags = [&](Frag* fa, Frag* fb, int buf, int s) {
+      const char* a_base = lds + buf * Cfg::kBufBytes + (wm * WM * 32 + l32) * Cfg::kLdsRow;
+      const char* b_base =
+          lds + buf * Cfg::kBufBytes + (Cfg::kBM + wn * WN * 32 + l32) * Cfg::kLdsRow;
       const int koff = s * MM::kK * (int)sizeof(T) + g * kFragBytes;
-      Frag fa[WM], fb[WN];
 #pragma unroll
       for (int i = 0; i < WM; ++i)
         fa[i] = *reinterpret_cast<const Frag*>(a_base + i * 32 * Cfg::kLdsRow + koff);
 #pragma unroll
       for (int j = 0; j < WN; ++j)
         fb[j] = *reinterpret_cast<const Frag*>(b_base + j * 32 * Cfg::kLdsRow + koff);
-#pragma unroll
-      for (int i = 0; i < WM; ++i)
-#pragma unroll
-        for (int j = 0; j < WN; ++j) {
-          if (SWAP) {
-            acc[i][j] = MM::run(fb[j], fa[i], acc[i][j]);
-          } else {
-            acc[i][j] = MM::run(fa[i], fb[j], acc[i][j]);
-          }
-        }
-    }
-  };
+    };
 
-  // Pipeline: K tiles kt+1 .. kt+PF are in flight from global memory in
-  // registers while tile kt is multiplied out of LDS.  With ALIGNED_K the loads
-  // and LDS stores of the loop body are straight-line code (loads past the last K
-  // tile re-read it and hit the cache), so the compiler can wait for exactly the
-  // oldest tile in flight instead of for every outstanding load.
+    // K tile j waits in register slot j % PF; tile 0 goes to LDS right away
 #pragma unroll
-  for (int j = 0; j < PF; ++j) {
-    if (ALIGNED_K || j < nk) gload(j, j);
-  }
-  lstore(0, 0);
-  if (ALIGNED_K || PF < nk) gload(0, PF);
-  __syncthreads();
-  for (int64_t kt0 = 0; kt0 < nk; kt0 += PF) {
+    for (int i = 0; i < kN; ++i) gload_one(0, i, 0);
 #pragma unroll
-    for (int j = 0; j < PF; ++j) {
-      const int64_t kt = kt0 + j;
-      const int buf = (j + (int)(kt0 & 1) * (PF & 1)) & 1;   // == kt & 1
-      const int slot = (j + 1) % PF;
-      if (ALIGNED_K) {
-        lstore(slot, buf ^ 1);
-        gload(slot, kt + 1 + PF);
-        if (kt < nk) compute(buf);   // uniform; false only in the last, partial group
-        __syncthreads();
-      } else if (kt < nk) {
-        if (kt + 1 < nk) lstore(slot, buf ^ 1);
-        if (kt + 1 + PF < nk) gload(slot, kt + 1 + PF);
-        compute(buf);
+    for (int i = 0; i < kN; ++i) lstore_one(0, i, 0);
+#pragma unroll
+    for (int j = 1; j <= PF; ++j)
+#pragma unroll
+      for (int i = 0; i < kN; ++i) gload_one(j % PF, i, j);
+    __syncthreads();
+    for (int64_t kt0 = 0; kt0 < nk; kt0 += PF) {
+#pragma unroll
+      for (int j = 0; j < PF; ++j) {
+        const int64_t kt = kt0 + j;
+        if (PF > 1 && kt >= nk) break;                       // uniform: last, partial group
+        const int buf = (j + (int)(kt0 & 1) * (PF & 1)) & 1;   // == kt & 1
+        const int slot = (j + 1) % PF;                         // == (kt + 1) % PF
+        Frag fa[2][WM], fb[2][WN];
+        read_frags(fa[0], fb[0], buf, 0);
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+          if (s + 1 < kSteps) read_frags(fa[(s + 1) & 1], fb[(s + 1) & 1], buf, s + 1);
+#pragma unroll
+          for (int i = 0; i < WM; ++i)
+#pragma unroll
+            for (int jj = 0; jj < WN; ++jj) {
+              if (SWAP) {
+                acc[i][jj] = MM::run(fb[s & 1][jj], fa[s & 1][i], acc[i][jj]);
+              } else {
+                acc[i][jj] = MM::run(fa[s & 1][i], fb[s & 1][jj], acc[i][jj]);
+              }
+            }
+#pragma unroll
+          for (int i = s * kN / kSteps; i < (s + 1) * kN / kSteps; ++i) {
+            lstore_one(slot, i, buf ^ 1);
+            gload_one(slot, i, kt + 1 + PF);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
         __syncthreads();
       }
+    }
+  } else {
+    // Any K: element-wise tails, one K tile in registers ahead of the MFMAs.
+    auto gload = [&](int64_t kt) {
+#pragma unroll
+      for (int i = 0; i < Cfg::kPerA; ++i) {
+        const int c = tid + i * Cfg::kThreads;
+        stage[0][i] = load_chunk<T, false>(a.A, a.lda, m0 + c / Cfg::kChunksPerRow, a.M,
+                                           kt * kBK + (c % Cfg::kChunksPerRow) * kPer, a.K);
+      }
+#pragma unroll
+      for (int i = 0; i < Cfg::kPerB; ++i) {
+        const int c = tid + i * Cfg::kThreads;
+        stage[0][Cfg::kPerA + i] =
+            load_chunk<T, false>(a.W, a.K, n0 + c / Cfg::kChunksPerRow, a.N,
+                                 kt * kBK + (c % Cfg::kChunksPerRow) * kPer, a.K);
+      }
+    };
+    auto lstore = [&](int buf) {
+      char* base = lds + buf * Cfg::kBufBytes;
+#pragma unroll
+      for (int i = 0; i < Cfg::kPerThread; ++i) {
+        const bool is_a = i < Cfg::kPerA;
+        const int c = tid + (is_a ? i : i - Cfg::kPerA) * Cfg::kThreads;
+        const int row = (is_a ? 0 : Cfg::kBM) + c / Cfg::kChunksPerRow;
+        store16(base + row * Cfg::kLdsRow + (c % Cfg::kChunksPerRow) * 16, stage[0][i]);
+      }
+    };
+    gload(0);
+    lstore(0);
+    __syncthreads();
+    for (int64_t kt = 0; kt < nk; ++kt) {
+      const int buf = (int)(kt & 1);
+      if (kt + 1 < nk) gload(kt + 1);
+      const char* a_base = lds + buf * Cfg::kBufBytes + (wm * WM * 32 + l32) * Cfg::kLdsRow;
+      const char* b_base =
+          lds + buf * Cfg::kBufBytes + (Cfg::kBM + wn * WN * 32 + l32) * Cfg::kLdsRow;
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s) {
+        const int koff = s * MM::kK * (int)sizeof(T) + g * kFragBytes;
+        Frag fa[WM], fb[WN];
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+          fa[i] = *reinterpret_cast<const Frag*>(a_base + i * 32 * Cfg::kLdsRow + koff);
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+          fb[j] = *reinterpret_cast<const Frag*>(b_base + j * 32 * Cfg::kLdsRow + koff);
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+          for (int j = 0; j < WN; ++j) {
+            if (SWAP) {
+              acc[i][j] = MM::run(fb[j], fa[i], acc[i][j]);
+            } else {
+              acc[i][j] = MM::run(fa[i], fb[j], acc[i][j]);
+            }
+          }
+      }
+      if (kt + 1 < nk) lstore(buf ^ 1);
+      __syncthreads();
     }
   }
 
@@ -290,8 +351,12 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
 // column panel after the other: its share of A (an eighth of the rows) stays
 // L2-resident while the W panels stream through, so A leaves HBM once instead
 // of once per column panel.
+// The second launch bound (wavefronts per SIMD the kernel is compiled for) is
+// what lets the compiler keep a whole K tile of fragments in registers: left at
+// its default it schedules for maximum occupancy, keeps three fragments live
+// and waits for LDS in front of every MFMA.
 template <typename T, class Cfg, int EPI, bool ALIGNED_K>
-__global__ __launch_bounds__(Cfg::kThreads) void linear_kernel(GemmArgs<T> a) {
+__global__ __launch_bounds__(Cfg::kThreads, NT_GEMM_WAVES_PER_EU) void linear_kernel(GemmArgs<T> a) {
   extern __shared__ __align__(16) char lds[];
   const int64_t tiles_m = (a.M + Cfg::kBM - 1) / Cfg::kBM;
   const int64_t per_xcd = (tiles_m + 7) / 8;
@@ -331,27 +396,76 @@ static int launch_kernel(const GemmArgs<T>& a, hipStream_t stream) {
 
 template <typename T, class Cfg, int EPI>
 static int launch_cfg(const GemmArgs<T>& a, hipStream_t stream) {
-  // the branch-free loads need whole K tiles and at least one row
-  const bool aligned = a.K > 0 && a.K % (Cfg::kRowBytes / (int64_t)sizeof(T)) == 0 && a.M > 0 && a.N > 0;
+  // the branch-free loads need whole K tiles
+  const bool aligned = a.K > 0 && a.K % (Cfg::kRowBytes / (int64_t)sizeof(T)) == 0;
   if (aligned) return launch_kernel<T, Cfg, EPI, true>(a, stream);
   return launch_kernel<T, Cfg, EPI, false>(a, stream);
 }
 
-#ifndef NT_GEMM_CFG
-#define NT_GEMM_CFG 4, 2, 2, 2, 128, 1
-#endif
-typedef GemmCfg<NT_GEMM_CFG> DefaultCfg;
+// WAVES_M, WAVES_N, WM, WN, K-tile bytes, K tiles in flight in registers
+typedef GemmCfg<4, 2, 2, 2, 128, 1> Cfg128;   // 256 x 128
+typedef GemmCfg<4, 2, 2, 3, 128, 1> Cfg192;   // 256 x 192
+typedef GemmCfg<4, 2, 2, 4, 128, 1> Cfg256;   // 256 x 256
 
-template <typename T>
-static int launch_linear(GemmArgs<T> a, bool qkv, hipStream_t stream) {
-  if (qkv) {
-    if (a.n_split % DefaultCfg::kBN != 0) {
+// Tile shape with the least (rounds over the CUs) x (tile area / efficiency).
+// The efficiencies are the measured steady-state MFMA rates of the shapes
+// relative to 256x128 (less LDS traffic per MFMA with wider wavefront tiles).
+static int pick_cfg(int64_t M, int64_t N, int64_t n_split, int* which) {
+  static int num_cus = 0;
+  if (num_cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess ||
+        prop.multiProcessorCount < 1) {
+      return fail(NT_ERR_HIP, "linear: cannot query the device");
+    }
+    num_cus = prop.multiProcessorCount;
+  }
+  const int bn[3] = {Cfg128::kBN, Cfg192::kBN, Cfg256::kBN};
+  const double eff[3] = {1.0, 1.08, 1.15};
+  int best = -1;
+  double best_cost = 0.0;
+  for (int c = 0; c < 3; ++c) {
+    if (n_split % bn[c] != 0) continue;          // a tile must not straddle the K | V boundary
+    if (NT_GEMM_FORCE_CFG >= 0 && c != NT_GEMM_FORCE_CFG) continue;
+    const int64_t tiles = ((M + 255) / 256) * ((N + bn[c] - 1) / bn[c]);
+    const int64_t rounds = (tiles + num_cus - 1) / num_cus;
+    const double cost = (double)rounds * bn[c] / eff[c];
+    if (best < 0 || cost < best_cost) {
+      best = c;
+      best_cost = cost;
+    }
+  }
+  if (best < 0) {
+    return fail(NT_ERR_UNSUPPORTED, "linear: QKV split %lld is not a multiple of a column tile",
+                (long long)n_split);
+  }
+  *which = best;
+  return NT_OK;
+}
+
+template <typename T, int EPI>
+static int launch_epi(const GemmArgs<T>& a, hipStream_t stream) {
+  int which = 0;
+  // the fp32 path exists for parity checks; it is compiled for one shape only
+  if constexpr (sizeof(T) == 4) {
+    if (EPI == kEpiQkv && a.n_split % Cfg128::kBN != 0) {
       return fail(NT_ERR_UNSUPPORTED, "linear: QKV split %lld is not a multiple of the column tile",
                   (long long)a.n_split);
     }
-    return launch_cfg<T, DefaultCfg, kEpiQkv>(a, stream);
+    return launch_cfg<T, Cfg128, EPI>(a, stream);
+  } else {
+    const int rc = pick_cfg(a.M, a.N, EPI == kEpiQkv ? a.n_split : 0, &which);
+    if (rc != NT_OK) return rc;
+    if (which == 1) return launch_cfg<T, Cfg192, EPI>(a, stream);
+    if (which == 2) return launch_cfg<T, Cfg256, EPI>(a, stream);
+    return launch_cfg<T, Cfg128, EPI>(a, stream);
   }
-  return launch_cfg<T, DefaultCfg, kEpiPlain>(a, stream);
+}
+
+template <typename T>
+static int launch_linear(GemmArgs<T> a, bool qkv, hipStream_t stream) {
+  return qkv ? launch_epi<T, kEpiQkv>(a, stream) : launch_epi<T, kEpiPlain>(a, stream);
 }
 
 static int check_linear(const void* A, int64_t lda, const void* W, const void* C, int64_t ldc,

@@ -229,3 +229,48 @@ def test_linear_packed_fast_path():
         for yi, xi in zip(y.unbind(), xs):
             exp = torch.nn.functional.linear(xi, W, b).float()
             assert (yi.float().cpu() - exp).abs().max() <= tol * max(1.0, exp.abs().max().item())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [
+    (300, 200, 64),        # one round: 256 x 128 tiles, whole K tiles
+    (300, 200, 72),        # K tail: element-wise loads
+    (9813, 2304, 64),      # two rounds of 256 x 192 tiles beat three of 256 x 128
+    (9813, 2304, 40),
+    (4096, 4096, 64),      # one round of 256 x 256 tiles
+    (4100, 4090, 24),
+])
+def test_linear_tile_shapes(M, N, K, dtype):
+    # the launcher picks one of three tile shapes per problem; every shape, with
+    # and without a K tail, against an fp32 reference of the same product
+    from nestedtensor_amd import ops
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) * 0.25).to(dtype)
+    b = torch.randn(N, generator=g).to(dtype)
+    y = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV)).float().cpu()
+    exp = x.float() @ w.float().t() + b.float()
+    tol = 2e-2 if dtype == torch.float16 else 6e-2   # one rounding of |y| <= ~16 to the output type
+    assert (y - exp).abs().max().item() <= tol
+
+
+def test_linear_qkv_tile_shapes():
+    # fused in-projection: Q | K row-major, V transposed, on the shape that takes
+    # the 256 x 192 tiles (2E = 1536 is a multiple of 192) and on a small one
+    from nestedtensor_amd import _C
+    for (T, E) in ((9813, 768), (70, 64)):
+        g = torch.Generator().manual_seed(T)
+        x = torch.randn(T, E, generator=g).half()
+        w = (torch.randn(3 * E, E, generator=g) * 0.05).half()
+        b = torch.randn(3 * E, generator=g).half()
+        xd, wd, bd = x.to(DEV), w.to(DEV), b.to(DEV)
+        ldvt = (T + 72 + 7) // 8 * 8
+        qk = torch.empty(T, 2 * E, dtype=torch.float16, device=DEV)
+        vt = torch.zeros(E, ldvt, dtype=torch.float16, device=DEV)
+        _C.check(_C.lib.nt_linear_qkv(_C.ptr(xd), E, _C.ptr(wd), _C.ptr(bd), _C.ptr(qk), 2 * E,
+                                      _C.ptr(vt), ldvt, T, E, E, _C.dtype_code(torch.float16),
+                                      _C.current_stream(xd.device)))
+        exp = x.float() @ w.float().t() + b.float()
+        assert (qk.float().cpu() - exp[:, :2 * E]).abs().max().item() <= 2e-2
+        assert (vt[:, :T].float().cpu() - exp[:, 2 * E:].t()).abs().max().item() <= 2e-2
+        assert vt[:, T:].abs().max().item() == 0      # nothing written past the last token
