@@ -24,9 +24,7 @@
 //   QKV    - the fused in-projection of self-attention: columns [0, n_split)
 //            (Q and K) go row-major into C, columns [n_split, N) (V) are written
 //            TRANSPOSED into Vt[n - n_split][m] so that the attention kernel
-//            finds V^T tiles key-contiguous.  V tiles run the MFMAs with swapped
-//            operands, which leaves C^T in the accumulators and keeps the
-//            stores coalesced.
+//            finds V^T tiles key-contiguous.
 #include "nt_common.h"
 
 // Compile-time tuning knobs.
@@ -135,10 +133,19 @@ __device__ __forceinline__ u32x4 load_chunk(const T* base, int64_t ld, int64_t r
 
 enum { kEpiPlain = 0, kEpiQkv = 1 };
 
-// One BM x BN tile.  SWAP runs the MFMAs with the operands exchanged, which
-// leaves C^T in the accumulators, and stores into Vt (the V part of the fused
-// QKV projection).
-template <typename T, class Cfg, bool SWAP, bool ALIGNED_K>
+// One BM x BN tile.  VT_OUT marks a V tile of the fused QKV projection, whose
+// result goes transposed into Vt.
+//
+// The accumulators of a 32x32 MFMA block hold, per lane, four runs of four
+// consecutive rows of one column of D.  Both operand fragments have the same
+// register layout, so exchanging them transposes D for free: a tile that goes
+// row-major into C is computed as C^T (a lane then holds runs of four
+// consecutive COLUMNS of one row of C), a V tile as C (runs of four consecutive
+// tokens of one feature = consecutive elements of a Vt row).  The epilogue
+// moves each 32-row strip through a private LDS region of the wavefront, 8 or
+// 16 bytes per lane in, and back out as 16-byte pieces of whole rows, so the
+// global stores are row-contiguous instead of 2 bytes per lane.
+template <typename T, class Cfg, bool VT_OUT, bool ALIGNED_K>
 __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int64_t n0, char* lds) {
   typedef Mma<T> MM;
   typedef typename MM::Frag Frag;
@@ -166,6 +173,14 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
 
   const int64_t nk = (a.K + kBK - 1) / kBK;
   u32x4 stage[PF][Cfg::kPerThread];
+
+  // bias of the tile's columns as fp32, behind the tile buffers (visible after
+  // the first barrier below)
+  if (tid < Cfg::kBN) {
+    const int64_t col = n0 + tid;
+    reinterpret_cast<float*>(lds + 2 * Cfg::kBufBytes)[tid] =
+        (a.bias && col < a.N) ? (float)a.bias[col] : 0.0f;
+  }
 
   if (ALIGNED_K) {
     // Straight-line K loop (loads past the last K tile re-read it and are never
@@ -231,10 +246,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
           for (int i = 0; i < WM; ++i)
 #pragma unroll
             for (int jj = 0; jj < WN; ++jj) {
-              if (SWAP) {
-                acc[i][jj] = MM::run(fb[s & 1][jj], fa[s & 1][i], acc[i][jj]);
-              } else {
+              if (VT_OUT) {
                 acc[i][jj] = MM::run(fa[s & 1][i], fb[s & 1][jj], acc[i][jj]);
+              } else {
+                acc[i][jj] = MM::run(fb[s & 1][jj], fa[s & 1][i], acc[i][jj]);
               }
             }
 #pragma unroll
@@ -297,10 +312,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
         for (int i = 0; i < WM; ++i)
 #pragma unroll
           for (int j = 0; j < WN; ++j) {
-            if (SWAP) {
-              acc[i][j] = MM::run(fb[j], fa[i], acc[i][j]);
-            } else {
+            if (VT_OUT) {
               acc[i][j] = MM::run(fa[i], fb[j], acc[i][j]);
+            } else {
+              acc[i][j] = MM::run(fb[j], fa[i], acc[i][j]);
             }
           }
       }
@@ -309,39 +324,99 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
     }
   }
 
-  if (!SWAP) {
-    // acc[i][j][e] = C[row, col], row = .. + i*32 + 8*(e/4) + 4*g + e%4, col = .. + j*32 + l32
-#pragma unroll
-    for (int j = 0; j < WN; ++j) {
-      const int64_t col = n0 + (wn * WN + j) * 32 + l32;
-      if (col >= a.N) continue;
-      const float bv = a.bias ? (float)a.bias[col] : 0.0f;
-#pragma unroll
-      for (int i = 0; i < WM; ++i) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int64_t row = m0 + (wm * WM + i) * 32 + 8 * (e >> 2) + 4 * g + (e & 3);
-          if (row < a.M) a.C[row * a.ldc + col] = (T)(acc[i][j][e] + bv);
-        }
-      }
-    }
-  } else {
-    // acc[i][j][e] = C[row, col], col = .. + j*32 + 8*(e/4) + 4*g + e%4, row = .. + i*32 + l32
+  // ---- epilogue ----------------------------------------------------------
+  // (the K loop ended with a barrier: the tile buffers are free)
+  constexpr int kStripW = VT_OUT ? WM : WN;                    // 32-wide blocks per strip row
+  constexpr int kStripRow = kStripW * 32 * (int)sizeof(T) + 16;
+  constexpr int kCpr = kStripW * 32 * (int)sizeof(T) / 16;    // 16-byte pieces per strip row
+  static_assert((Cfg::kThreads / 64) * 32 * kStripRow <= 2 * Cfg::kBufBytes, "strips must fit");
+  char* strip = lds + wave * (32 * kStripRow);
+  const float* lds_bias = reinterpret_cast<const float*>(lds + 2 * Cfg::kBufBytes);
+  typedef T Quad __attribute__((ext_vector_type(4)));
+
+  if (!VT_OUT) {
+    // acc[i][j][e] = C[row, col], row = .. + i*32 + l32, col = .. + j*32 + 8*(e/4) + 4*g + e%4
+    const bool row_vec_ok = (a.ldc * (int64_t)sizeof(T)) % 16 == 0 &&
+                            reinterpret_cast<uintptr_t>(a.C) % 16 == 0;
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
-      const int64_t row = m0 + (wm * WM + i) * 32 + l32;
-      if (row >= a.M) continue;
 #pragma unroll
       for (int j = 0; j < WN; ++j) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int64_t col = n0 + (wn * WN + j) * 32 + 8 * (e >> 2) + 4 * g + (e & 3);
-          if (col < a.N) {
-            const float bv = a.bias ? (float)a.bias[col] : 0.0f;
-            a.Vt[(col - a.n_split) * a.ldvt + row] = (T)(acc[i][j][e] + bv);
+        for (int r = 0; r < 4; ++r) {
+          const int c0 = j * 32 + 8 * r + 4 * g;
+          const float4 bv = *reinterpret_cast<const float4*>(lds_bias + wn * WN * 32 + c0);
+          Quad q;
+          q[0] = (T)(acc[i][j][4 * r + 0] + bv.x);
+          q[1] = (T)(acc[i][j][4 * r + 1] + bv.y);
+          q[2] = (T)(acc[i][j][4 * r + 2] + bv.z);
+          q[3] = (T)(acc[i][j][4 * r + 3] + bv.w);
+          *reinterpret_cast<Quad*>(strip + l32 * kStripRow + c0 * (int)sizeof(T)) = q;
+        }
+      }
+      __builtin_amdgcn_wave_barrier();   // LDS serves a wavefront's accesses in order
+#pragma unroll
+      for (int it = 0; it < 32 * kCpr / 64; ++it) {
+        const int idx = it * 64 + lane;
+        const int r = idx / kCpr, c = idx % kCpr;
+        const int64_t row = m0 + (wm * WM + i) * 32 + r;
+        const int64_t col = n0 + wn * WN * 32 + c * kPer;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(strip + r * kStripRow + c * 16);
+        if (row < a.M && col < a.N) {
+          T* dst = a.C + row * a.ldc + col;
+          if (row_vec_ok && col + kPer <= a.N) {
+            store16(reinterpret_cast<char*>(dst), v);
+          } else {
+            T tmp[kPer];
+            __builtin_memcpy(tmp, &v, 16);
+#pragma unroll
+            for (int e = 0; e < kPer; ++e)
+              if (col + e < a.N) dst[e] = tmp[e];
           }
         }
       }
+      __builtin_amdgcn_wave_barrier();
+    }
+  } else {
+    // acc[i][j][e] = C[row, col], row = .. + i*32 + 8*(e/4) + 4*g + e%4, col = .. + j*32 + l32
+    const bool row_vec_ok = (a.ldvt * (int64_t)sizeof(T)) % 16 == 0 &&
+                            reinterpret_cast<uintptr_t>(a.Vt) % 16 == 0;
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+      const float bv = lds_bias[(wn * WN + j) * 32 + l32];
+#pragma unroll
+      for (int i = 0; i < WM; ++i) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          Quad q;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) q[e] = (T)(acc[i][j][4 * r + e] + bv);
+          *reinterpret_cast<Quad*>(strip + l32 * kStripRow +
+                                   (i * 32 + 8 * r + 4 * g) * (int)sizeof(T)) = q;
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int it = 0; it < 32 * kCpr / 64; ++it) {
+        const int idx = it * 64 + lane;
+        const int r = idx / kCpr, c = idx % kCpr;
+        const int64_t col = n0 + (wn * WN + j) * 32 + r;           // feature
+        const int64_t row = m0 + wm * WM * 32 + c * kPer;          // first token of the piece
+        const u32x4 v = *reinterpret_cast<const u32x4*>(strip + r * kStripRow + c * 16);
+        if (col < a.N && row < a.M) {
+          T* dst = a.Vt + (col - a.n_split) * a.ldvt + row;
+          if (row_vec_ok && row + kPer <= a.M) {
+            store16(reinterpret_cast<char*>(dst), v);
+          } else {
+            T tmp[kPer];
+            __builtin_memcpy(tmp, &v, 16);
+#pragma unroll
+            for (int e = 0; e < kPer; ++e)
+              if (row + e < a.M) dst[e] = tmp[e];
+          }
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
     }
   }
 }
@@ -368,7 +443,7 @@ __global__ __launch_bounds__(Cfg::kThreads, NT_GEMM_WAVES_PER_EU) void linear_ke
   const int64_t m0 = tm * Cfg::kBM;
   const int64_t n0 = tn * Cfg::kBN;
   if (EPI == kEpiQkv && n0 >= a.n_split) {
-    gemm_tile<T, Cfg, true, ALIGNED_K>(a, m0, n0, lds);
+    gemm_tile<T, Cfg, true, ALIGNED_K>(a, m0, n0, lds);    // V tile: transposed into Vt
   } else {
     gemm_tile<T, Cfg, false, ALIGNED_K>(a, m0, n0, lds);
   }
@@ -380,7 +455,7 @@ static int launch_kernel(const GemmArgs<T>& a, hipStream_t stream) {
   const int64_t tiles_n = (a.N + Cfg::kBN - 1) / Cfg::kBN;
   const int64_t wgs = ((tiles_m + 7) / 8) * 8 * tiles_n;
   if (wgs > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "linear: too many tiles");
-  const int lds_bytes = 2 * Cfg::kBufBytes;
+  const int lds_bytes = 2 * Cfg::kBufBytes + Cfg::kBN * (int)sizeof(float);
   static bool attr_set = false;
   if (!attr_set && lds_bytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(
