@@ -301,7 +301,7 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
   typedef typename AT::Frag Frag;
 
   __shared__ __align__(16) char lds_k[2][kKBytes];
-  __shared__ __align__(16) char lds_v[2][kVBytes];
+  __shared__ __align__(16) char lds_v[2][kVBytes + kVRow];   // row 64: ones (see below)
 
   // Head fastest: the schedule lists the longest sequences first, and this way
   // their items of ALL heads are dispatched before any short item (with the
@@ -339,147 +339,191 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
 #pragma unroll
     for (int e = 0; e < 16; ++e) o_acc[i][e] = 0.0f;
   float m_run = -INFINITY;
-  float l_run = 0.0f;
 
   const int ntiles = (L + kKTile - 1) / kKTile;
   const T* kbase = QK + begin * ldqk + k_col + h * kHd;
   const T* vbase = Vt + (int64_t)h * kHd * ldvt + begin;
 
-  // Each thread moves two 16-byte pieces of the K tile and two of the V^T tile.
+  // Each thread moves two 16-byte pieces of a K tile and two of a V^T tile.
   // The loads are unconditional and unmasked (clamped addresses), so that the
-  // wavefront only waits for them where the data is stored to LDS.
+  // wavefront only waits for them where the data is stored to LDS.  All per-thread
+  // addressing is set up once; a step only advances pointers.
   const int r0 = tid >> 3;      // row of piece 0 (piece 1: r0 + 32)
   const int cc = tid & 7;
   u32x4 rk[2], rv[2];
-  auto gload = [&](int t_in) {
-    const int t = t_in < ntiles ? t_in : ntiles - 1;
+  const char* k_last = reinterpret_cast<const char*>(kbase + (int64_t)(L - 1) * ldqk + cc * 8);
+  const int64_t k_step = (int64_t)kKTile * ldqk * (int64_t)sizeof(T);
+  const char* v_ptr[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    v_ptr[i] = reinterpret_cast<const char*>(vbase + (int64_t)(r0 + i * 32) * ldvt + cc * 8);
+  }
+  auto gload_k = [&](int t_in) {
+    const int t = t_in < ntiles ? t_in : ntiles - 1;   // past the end: re-read, never used
+    const char* tile = reinterpret_cast<const char*>(kbase + cc * 8) + t * k_step;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int r = r0 + i * 32;
-      int kr = t * kKTile + r;
-      kr = kr < L ? kr : L - 1;        // rows past L: their scores are masked below
-      rk[i] = load16_unaligned(reinterpret_cast<const char*>(kbase + (int64_t)kr * ldqk + cc * 8));
-      // V^T piece: keys key0 .. key0+7 of row d = r, read where it lies (the rows
-      // of Vt are readable 72 elements past the last token)
-      rv[i] = load16_unaligned(
-          reinterpret_cast<const char*>(vbase + (int64_t)r * ldvt + t * kKTile + cc * 8));
+      // rows past L read row L - 1 (a valid key: it cannot raise the row maximum)
+      const int kr = t * kKTile + r0 + i * 32;
+      const char* src = tile + (int64_t)(r0 + i * 32) * ldqk * (int64_t)sizeof(T);
+      rk[i] = load16_unaligned(kr < L ? src : k_last);
     }
   };
-  auto lstore = [&](int buf, int t) {
-    // keys at or past L are zeroed: a probability of exactly 0 must not meet a NaN
-    int nv = L - (t * kKTile + cc * 8);
-    nv = nv > 8 ? 8 : (nv < 0 ? 0 : nv);
-    const uint32_t m0 = nv >= 2 ? 0xffffffffu : (nv == 1 ? 0x0000ffffu : 0u);
-    const uint32_t m1 = nv >= 4 ? 0xffffffffu : (nv == 3 ? 0x0000ffffu : 0u);
-    const uint32_t m2 = nv >= 6 ? 0xffffffffu : (nv == 5 ? 0x0000ffffu : 0u);
-    const uint32_t m3 = nv >= 8 ? 0xffffffffu : (nv == 7 ? 0x0000ffffu : 0u);
-    // piece cc = keys 8cc .. 8cc+7 = (ks = cc/2, a = cc%2); its low half (g = 0)
-    // goes to position 16ks + 4a, its high half (g = 1) to 16ks + 8 + 4a.
-    const int ks = cc >> 1, a2 = cc & 1;
+  auto gload_v = [&](int t_in) {
+    const int t = t_in < ntiles ? t_in : ntiles - 1;
+    // V^T piece: keys key0 .. key0+7 of row d, read where it lies (the rows of Vt
+    // are readable 72 elements past the last token)
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int r = r0 + i * 32;
-      store16(&lds_k[buf][r * kKRow + cc * 16], rk[i]);
-      char* row = &lds_v[buf][r * kVRow];
+      rv[i] = load16_unaligned(v_ptr[i] + t * (kKTile * (int)sizeof(T)));
+    }
+  };
+  auto lstore_k = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) store16(&lds_k[buf][(r0 + i * 32) * kKRow + cc * 16], rk[i]);
+  };
+  // piece cc = keys 8cc .. 8cc+7 = (ks = cc/2, a = cc%2); its low half (g = 0)
+  // goes to position 16ks + 4a, its high half (g = 1) to 16ks + 8 + 4a.
+  const int v_lo = (16 * (cc >> 1) + 4 * (cc & 1)) * 2;
+  // keys at or past L are zeroed in the last tile: a probability must not meet
+  // a NaN there, and the ones row must not count them
+  uint32_t vm[4];
+  {
+    int nv = L - ((ntiles - 1) * kKTile + cc * 8);
+    nv = nv > 8 ? 8 : (nv < 0 ? 0 : nv);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      vm[j] = nv >= 2 * j + 2 ? 0xffffffffu : (nv == 2 * j + 1 ? 0x0000ffffu : 0u);
+    }
+  }
+  auto lstore_v = [&](int buf, int t) {
+    const bool last = t >= ntiles - 1;   // uniform
+    const uint32_t m0 = last ? vm[0] : 0xffffffffu, m1 = last ? vm[1] : 0xffffffffu;
+    const uint32_t m2 = last ? vm[2] : 0xffffffffu, m3 = last ? vm[3] : 0xffffffffu;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      char* row = &lds_v[buf][(r0 + i * 32) * kVRow + v_lo];
       const uint64_t lo = ((uint64_t)(rv[i].y & m1) << 32) | (rv[i].x & m0);
       const uint64_t hi = ((uint64_t)(rv[i].w & m3) << 32) | (rv[i].z & m2);
-      *reinterpret_cast<uint64_t*>(row + (16 * ks + 4 * a2) * 2) = lo;
-      *reinterpret_cast<uint64_t*>(row + (16 * ks + 8 + 4 * a2) * 2) = hi;
+      *reinterpret_cast<uint64_t*>(row) = lo;
+      *reinterpret_cast<uint64_t*>(row + 16) = hi;
+    }
+    if (r0 == 0) {
+      // row 64: 1 for every valid key.  Multiplied with P^T by the matrix pipe it
+      // yields the softmax denominators, and because it is zero past L (like the
+      // V^T rows) the keys of a partial tile need no masking of their scores.
+      char* row = &lds_v[buf][kHd * kVRow + v_lo];
+      const uint64_t lo = ((uint64_t)(AT::kOnePair & m1) << 32) | (AT::kOnePair & m0);
+      const uint64_t hi = ((uint64_t)(AT::kOnePair & m3) << 32) | (AT::kOnePair & m2);
+      *reinterpret_cast<uint64_t*>(row) = lo;
+      *reinterpret_cast<uint64_t*>(row + 16) = hi;
     }
   };
 
-  gload(0);
-  lstore(0, 0);
-  __syncthreads();
-
-  for (int t = 0; t < ntiles; ++t) {
-    const int buf = t & 1;
-    gload(t + 1);   // past the end: re-reads the last tile, never stored
-    // keep the loads above the MFMA / softmax work (the scheduler would sink them)
-    __builtin_amdgcn_sched_barrier(0);
-
-    if (wave_active) {
-      acc16 s_acc[2];
+  // S^T tile of K tile in lds_k[buf]:
+  // s[kb][e] = score(key = 64 t + 32 kb + 8 (e/4) + 4 g + e%4, q = l32)
+  auto scores = [&](acc16 (&sa)[2], int buf) {
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
+    for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s_acc[kb][e] = 0.0f;
-        const char* krow = &lds_k[buf][(kb * 32 + l32) * kKRow + g * 16];
+      for (int e = 0; e < 16; ++e) sa[kb][e] = 0.0f;
+      const char* krow = &lds_k[buf][(kb * 32 + l32) * kKRow + g * 16];
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          Frag kf = *reinterpret_cast<const Frag*>(krow + s * 32);
-          s_acc[kb] = AT::mma(kf, qf[s], s_acc[kb]);
-        }
-      }
-      // s_acc[kb][e] = score(key = 64 t + 32 kb + 8 (e/4) + 4 g + e%4, q = l32)
-      const int key_base = t * kKTile;
-      if (key_base + kKTile > L) {
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const int key = key_base + kb * 32 + 8 * (e >> 2) + 4 * g + (e & 3);
-            if (key >= L) s_acc[kb][e] = -INFINITY;
-          }
-      }
-      float m_tile = s_acc[0][0];
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) m_tile = fmaxf(m_tile, s_acc[kb][e]);
-      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
-      const float m_new = fmaxf(m_run, m_tile);   // finite: every tile holds a valid key
-      // raw v_exp_f32: arguments are <= 0, results in [0, 1]
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
-      const float m_scaled = m_new * scale_log2e;
-      m_run = m_new;
-      Frag pf[4];   // P^T as B-operand: k-step ks = 2 kb + half uses s_acc[kb][8 half .. +8]
-      float l_tile = 0.0f;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          uint32_t w[4];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const float p0 =
-                __builtin_amdgcn_exp2f(fmaf(s_acc[kb][half * 8 + 2 * j], scale_log2e, -m_scaled));
-            const float p1 =
-                __builtin_amdgcn_exp2f(fmaf(s_acc[kb][half * 8 + 2 * j + 1], scale_log2e, -m_scaled));
-            l_tile += p0 + p1;
-            w[j] = AT::cvt2(p0, p1);
-          }
-          __builtin_memcpy(&pf[kb * 2 + half], w, 16);
-        }
-      }
-      l_run = l_run * alpha + l_tile;
-      // the running maxima settle after the first tiles; then alpha is 1 in
-      // every lane and the 32 multiplications are skipped (wavefront-uniform)
-      if (__any(alpha != 1.0f)) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
-      }
-
-      // O^T += V^T P^T
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-#pragma unroll
-        for (int db = 0; db < 2; ++db) {
-          const char* vrow = &lds_v[buf][(db * 32 + l32) * kVRow + g * 16];
-          Frag vf = *reinterpret_cast<const Frag*>(vrow + ks * 32);
-          o_acc[db] = AT::mma(vf, pf[ks], o_acc[db]);
-        }
+      for (int s = 0; s < 4; ++s) {
+        Frag kf = *reinterpret_cast<const Frag*>(krow + s * 32);
+        sa[kb] = AT::mma(kf, qf[s], sa[kb]);
       }
     }
+  };
 
-    lstore(buf ^ 1, t + 1);   // past the end: harmless, the buffer is not read again
+  // Online softmax of one tile's scores, then O^T += V^T P^T and the
+  // denominators l += 1^T P^T from lds_v[vbuf].
+  //
+  // Keys past L in a partial tile: their K rows are copies of row L - 1, so they
+  // cannot raise the row maximum; their V^T columns and their entries of the ones
+  // row are zero, so they add nothing to O or l.  No score is ever masked.
+  acc16 l_acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) l_acc[e] = 0.0f;
+  auto softmax_pv = [&](acc16 (&sa)[2], int vbuf) {
+    float m_tile = sa[0][0];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) m_tile = fmaxf(m_tile, sa[kb][e]);
+    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
+    const float m_new = fmaxf(m_run, m_tile);   // finite: every tile holds a valid key
+    // raw v_exp_f32: arguments are <= 0, results in [0, 1]
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
+    const float m_scaled = m_new * scale_log2e;
+    m_run = m_new;
+    // the running maxima settle after the first tiles; then alpha is 1 in
+    // every lane and the multiplications are skipped (wavefront-uniform)
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+      l_acc[0] *= alpha;   // every element of l_acc holds the same sum; [0] is the one read
+    }
+    Frag pf[4];   // P^T as B-operand: k-step ks = 2 kb + half uses sa[kb][8 half .. +8]
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        uint32_t w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float p0 =
+              __builtin_amdgcn_exp2f(fmaf(sa[kb][half * 8 + 2 * j], scale_log2e, -m_scaled));
+          const float p1 =
+              __builtin_amdgcn_exp2f(fmaf(sa[kb][half * 8 + 2 * j + 1], scale_log2e, -m_scaled));
+          w[j] = AT::cvt2(p0, p1);
+        }
+        __builtin_memcpy(&pf[kb * 2 + half], w, 16);
+      }
+    }
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+      for (int db = 0; db < 2; ++db) {
+        const char* vrow = &lds_v[vbuf][(db * 32 + l32) * kVRow + g * 16];
+        Frag vf = *reinterpret_cast<const Frag*>(vrow + ks * 32);
+        o_acc[db] = AT::mma(vf, pf[ks], o_acc[db]);
+      }
+      // all 32 rows of this A-operand are the ones row: every lane gets l[q]
+      Frag of = *reinterpret_cast<const Frag*>(&lds_v[vbuf][kHd * kVRow + g * 16 + ks * 32]);
+      l_acc = AT::mma(of, pf[ks], l_acc);
+    }
+  };
+
+  // Tile t + 1 travels global -> registers while tile t is computed, and goes
+  // registers -> LDS (the other buffer) after the compute, before the barrier.
+  // Wavefronts of other workgroups on the SIMD (three fit) fill the matrix pipe
+  // while this one runs its softmax, and the other way round.
+  gload_k(0);
+  gload_v(0);
+  lstore_k(0);
+  lstore_v(0, 0);
+  __syncthreads();
+  for (int t = 0; t < ntiles; ++t) {
+    const int buf = t & 1;
+    gload_k(t + 1);   // past the end: re-reads the last tile
+    gload_v(t + 1);
+    // keep the loads above the MFMA / softmax work (the scheduler would sink them)
+    __builtin_amdgcn_sched_barrier(0);
+    if (wave_active) {
+      acc16 sa[2];
+      scores(sa, buf);
+      softmax_pv(sa, buf);
+    }
+    lstore_k(buf ^ 1);          // past the end: harmless, the buffer is not read again
+    lstore_v(buf ^ 1, t + 1);
     __syncthreads();
   }
 
   if (!wave_active || q_row >= L) return;
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  const float l_tot = l_acc[0];
   const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
   T* op = O + (begin + q_row) * ldo + h * kHd;
 #pragma unroll
