@@ -32,9 +32,9 @@ struct NotEqual {
 
 // counts[r] = kept entries of row r; prefix[r] = 1 iff the kept entries are
 // exactly the first counts[r] entries of the row.  One wavefront per row; a lane
-// looks at VEC consecutive entries per step (VEC * sizeof(T) == 16 when rows are
-// 16-byte aligned, else 1); ballots over the lanes' "full / non-empty / is a
-// prefix" flags decide prefix-ness without any serial scan.
+// looks at VEC consecutive entries per step (16 bytes; one entry for short
+// rows); ballots over the lanes' "full / non-empty / is a prefix" flags decide
+// prefix-ness without any serial scan.
 template <typename P, int VEC>
 __global__ __launch_bounds__(kWave * kRowsPerBlock) void row_counts_kernel(
     const typename P::type* __restrict__ data, int64_t R, int64_t M, P pred,
@@ -54,7 +54,8 @@ __global__ __launch_bounds__(kWave * kRowsPerBlock) void row_counts_kernel(
       if (i0 < M) v[0] = m[i0];
     } else {
       if (i0 + VEC <= M) {
-        u32x4 raw = *reinterpret_cast<const u32x4*>(m + i0);
+        // any alignment: the part runs in unaligned-access mode
+        u32x4 raw = load16_unaligned(reinterpret_cast<const char*>(m + i0));
         __builtin_memcpy(v, &raw, 16);
       } else {
 #pragma unroll
@@ -100,10 +101,10 @@ static int launch_row_counts(const void* data, int64_t R, int64_t M, P pred, int
   const int64_t blocks = (R + kRowsPerBlock - 1) / kRowsPerBlock;
   if (blocks > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "row_counts: too many rows");
   constexpr int kVec = 16 / sizeof(T);
-  const bool aligned = ((uintptr_t)data % 16 == 0) && ((M * (int64_t)sizeof(T)) % 16 == 0);
   dim3 grid((unsigned)blocks), block(kWave * kRowsPerBlock);
   const T* d = static_cast<const T*>(data);
-  if (aligned && kVec > 1) {
+  // short rows: one entry per lane keeps more lanes busy than 16 bytes per lane
+  if (M * (int64_t)sizeof(T) >= 256) {
     hipLaunchKernelGGL((row_counts_kernel<P, kVec>), grid, block, 0, stream, d, R, M, pred, counts,
                        prefix);
   } else {
