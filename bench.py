@@ -397,6 +397,31 @@ def bench_rows(args, torch, dev):
     ms_scan = _time_gpu(torch, lambda: device_offsets(sizes, 4096, 2))
     rows["offsets_scan_B4096"] = dict(ms=ms_scan)
 
+    # ---- row-wise ops either side of attention: C3 encoder width and a large buffer
+    from nestedtensor_amd import ops as _ops
+    for tag, lens_rw, E_rw in (("C3", [int(v) for v in torch.randint(32, 513, (32,), generator=torch.Generator().manual_seed(1012))], 768),
+                               ("large", [2048] * 256, 4096)):
+        T_rw = sum(lens_rw)
+        buf = torch.randn(T_rw * E_rw, device=dev, dtype=torch.float16)
+        sizes_rw = torch.tensor([[L, E_rw] for L in lens_rw], dtype=torch.int64)
+        from nestedtensor_amd.impl import NestedTensorImpl
+        x_rw = NestedTensorImpl(buf, sizes_rw)
+        r_rw = NestedTensorImpl(torch.randn_like(buf), sizes_rw)
+        w_rw, b_rw = torch.randn(E_rw, device=dev).half(), torch.randn(E_rw, device=dev).half()
+        nb = 2 * T_rw * E_rw
+        ms_ln = _time_gpu(torch, lambda: _ops.layer_norm(x_rw, (E_rw,), w_rw, b_rw, 1e-5))
+        ms_rln = _time_gpu(torch, lambda: _ops.layer_norm(x_rw, (E_rw,), w_rw, b_rw, 1e-5, residual=r_rw))
+        ms_add = _time_gpu(torch, lambda: _ops.add(x_rw, r_rw))
+        c_ln = None
+        if cpu and tag == "C3":
+            parts_rw = [p.reshape(L, E_rw) for p, L in zip(buf.cpu().split([L * E_rw for L in lens_rw]), lens_rw)]
+            ref_rw = oracle.ref_nested_tensor(parts_rw, dtype=torch.float16)
+            c_ln = _time_cpu(lambda: oracle.layer_norm(ref_rw, (E_rw,), w_rw.cpu(), b_rw.cpu(), 1e-5), 2)
+        rows[tag + "_layer_norm_fp16"] = entry(ms_ln, 2 * nb, c_ln, rows=T_rw, width=E_rw)
+        rows[tag + "_residual_layer_norm_fp16"] = entry(ms_rln, 3 * nb, None, rows=T_rw, width=E_rw)
+        rows[tag + "_packed_add_fp16"] = entry(ms_add, 3 * nb, None, rows=T_rw, width=E_rw)
+        del buf, x_rw, r_rw
+
     # ---- C4: bt_min_mha bf16, high raggedness ---------------------------------
     g = torch.Generator().manual_seed(1010 + 3)
     raw = torch.empty(128).exponential_(1.0 / 96.0, generator=g)

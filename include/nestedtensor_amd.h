@@ -191,6 +191,29 @@ int nt_varlen_attention_vt(const void* qk, int64_t ldqk, int64_t k_col, const vo
                            int64_t n_work, int64_t num_heads, int64_t total_tokens, float scale,
                            int dtype, void* stream);
 
+/* ---- row-wise ops on the packed buffer (the steps either side of attention
+ *      in an encoder layer) ------------------------------------------------ */
+
+/* out[r, :] = layer_norm(x[r, :] (+ residual[r, :])) * gamma + beta over the last
+ * dim of the packed [rows, n] view of a nested tensor whose last dim is regular;
+ * residual, gamma and beta may be NULL.  Mean and variance are two-pass fp32 sums
+ * (biased variance), rstd = 1 / sqrt(var + eps); with a residual the sum is first
+ * rounded to the storage type, as the reference's separate add does.  Replaces
+ * NestedTensor_layer_norm (nestedtensor/csrc/functions.cpp:65-112), whose device
+ * fast path is nestedtensor/csrc/cuda/layernorm.cpp:14-76 with the kernel of
+ * nestedtensor/csrc/cuda/transformer_kernels.cu:260-335, preceded by the packed
+ * residual add NestedTensor_add_Tensor (nestedtensor/csrc/BinaryOps.cpp:18-44). */
+int nt_layer_norm(const void* x, const void* residual, const void* gamma, const void* beta,
+                  void* out, int64_t rows, int64_t n, double eps, int dtype, void* stream);
+
+/* out[i] = a[i] + alpha * b[i % period], fp32 math, rounded to the storage type.
+ * period == numel: the sum of two nested tensors of equal nested size, done on
+ * their packed buffers (nestedtensor/csrc/BinaryOps.cpp:18-44).  period == n: a
+ * nested tensor with regular last dim n plus a 1-D tensor of n elements
+ * (nestedtensor/csrc/BinaryOps.cpp:97-107).  numel must be a multiple of period. */
+int nt_add_packed(const void* a, const void* b, double alpha, void* out, int64_t numel,
+                  int64_t period, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,6 +25,7 @@ _int = ctypes.c_int
 _u64 = ctypes.c_uint64
 _size_t = ctypes.c_size_t
 _f32 = ctypes.c_float
+_f64 = ctypes.c_double
 
 # name -> (restype, argtypes); must list every symbol of include/nestedtensor_amd.h
 SIGNATURES = {
@@ -53,6 +54,9 @@ SIGNATURES = {
     "nt_varlen_attention": (_int, [_c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64,
                                    _c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _f32, _int,
                                    _c_void_p]),
+    "nt_layer_norm": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _f64, _int,
+                             _c_void_p]),
+    "nt_add_packed": (_int, [_c_void_p, _c_void_p, _f64, _c_void_p, _i64, _i64, _int, _c_void_p]),
 }
 
 

@@ -1,0 +1,294 @@
+// Row-wise ops on the packed token buffer of a nested tensor (gfx950): layer
+// normalisation over the (regular) last dim, with an optional residual input, and
+// the two packed additions of the reference (nested + nested of equal nested
+// size, nested + 1-D vector over the last dim).  A nested tensor [B, L_i, n] is
+// one contiguous [T, n] matrix here, so none of these needs the nested size:
+// they are the per-constituent at::layer_norm / at::add of the reference
+// (nestedtensor/csrc/functions.cpp:65-112, BinaryOps.cpp:18-44, 97-107) done in
+// one launch over all constituents.  All are HBM-bound: every input element is
+// read once and every output element written once.
+//
+// Layer norm: one wavefront per row (a workgroup per row for wide rows).  The
+// row is read once into registers, 16 bytes per lane per piece; mean and variance
+// are the exact two-pass sums in fp32 (as the reference's kernel,
+// nestedtensor/csrc/cuda/transformer_kernels.cu:260-305), reduced with wave
+// shuffles.  Rows beyond 16 KiB, or not made of aligned 16-byte pieces, re-read
+// from cache instead of keeping the row in registers.  With a residual, the sum is rounded to the storage type before it
+// is normalised: that is what the reference computes, as two separate ops.
+#include "nt_common.h"
+
+namespace nt {
+
+constexpr int kNormRowsPerBlock = 4;   // one wavefront each
+
+template <typename T>
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+// x (+ residual) of one 16-byte piece as floats
+template <typename T>
+__device__ __forceinline__ void piece_values(u32x4 raw, u32x4 raw_res, bool has_res, float* f) {
+  constexpr int kPer = 16 / sizeof(T);
+  T a[kPer], r[kPer];
+  __builtin_memcpy(a, &raw, 16);
+  __builtin_memcpy(r, &raw_res, 16);
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    f[j] = has_res ? (float)(T)((float)a[j] + (float)r[j]) : (float)a[j];
+  }
+}
+
+// Rows of whole 16-byte pieces at 16-byte aligned addresses.  A row is handled by
+// WAVES wavefronts (1: four rows per workgroup, 4: the workgroup shares one row and
+// combines its partial sums through LDS); every lane keeps P pieces in registers,
+// so a row has at most 64 * WAVES * P pieces.
+template <typename T, int P, int WAVES>
+__global__ __launch_bounds__(kWave * kNormRowsPerBlock) void layer_norm_rows_kernel(
+    const T* __restrict__ x, const T* __restrict__ residual, const T* __restrict__ gamma,
+    const T* __restrict__ beta, T* __restrict__ out, int64_t rows, int n, float eps) {
+  constexpr int kPer = 16 / sizeof(T);
+  constexpr int kTeam = kWave * WAVES;                    // threads per row
+  constexpr int kRows = kNormRowsPerBlock / WAVES;        // rows per workgroup
+  __shared__ float red_sum[kNormRowsPerBlock], red_sq[kNormRowsPerBlock];
+  const int t = threadIdx.x % kTeam;
+  const int64_t row = (int64_t)blockIdx.x * kRows + threadIdx.x / kTeam;
+  if (row >= rows) return;   // WAVES == 4: the whole workgroup leaves together
+  const int pieces = n / kPer;
+  const char* xr = reinterpret_cast<const char*>(x + row * n);
+  const char* rr = reinterpret_cast<const char*>(residual + row * n);
+  const bool has_res = residual != nullptr;
+
+  auto team_sum = [&](float v, float* red) -> float {
+    v = wave_sum<T>(v);
+    if (WAVES == 1) return v;
+    if ((threadIdx.x & (kWave - 1)) == 0) red[threadIdx.x / kWave] = v;
+    __syncthreads();
+    float total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) total += red[w];
+    return total;
+  };
+
+  float f[P][kPer];
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    const int c = t + p * kTeam;
+    if (c < pieces) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(xr + c * 16);
+      u32x4 raw_res = raw;
+      if (has_res) raw_res = *reinterpret_cast<const u32x4*>(rr + c * 16);
+      piece_values<T>(raw, raw_res, has_res, f[p]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) f[p][j] = 0.0f;
+    }
+  }
+  float sum = 0.0f;
+#pragma unroll
+  for (int p = 0; p < P; ++p)
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) sum += f[p][j];
+  const float mean = team_sum(sum, red_sum) / (float)n;
+  float sq = 0.0f;
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    if (t + p * kTeam < pieces) {
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) sq += (f[p][j] - mean) * (f[p][j] - mean);
+    }
+  }
+  const float rstd = 1.0f / sqrtf(team_sum(sq, red_sq) / (float)n + eps);
+  char* orow = reinterpret_cast<char*>(out + row * n);
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    const int c = t + p * kTeam;
+    if (c < pieces) {
+      float g[kPer], b[kPer];
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        g[j] = 1.0f;
+        b[j] = 0.0f;
+      }
+      if (gamma) {
+        T tmp[kPer];
+        const u32x4 raw = load16_unaligned(reinterpret_cast<const char*>(gamma + c * kPer));
+        __builtin_memcpy(tmp, &raw, 16);
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) g[j] = (float)tmp[j];
+      }
+      if (beta) {
+        T tmp[kPer];
+        const u32x4 raw = load16_unaligned(reinterpret_cast<const char*>(beta + c * kPer));
+        __builtin_memcpy(tmp, &raw, 16);
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) b[j] = (float)tmp[j];
+      }
+      T y[kPer];
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        float v = (f[p][j] - mean) * rstd;
+        if (gamma) v = v * g[j];
+        if (beta) v = v + b[j];
+        y[j] = (T)v;
+      }
+      u32x4 o;
+      __builtin_memcpy(&o, y, 16);
+      store16_stream(orow + c * 16, o);
+    }
+  }
+}
+
+// Any n, any alignment: three passes over the row (the second and third hit the
+// cache), one element per lane per step.
+template <typename T>
+__global__ __launch_bounds__(kWave * kNormRowsPerBlock) void layer_norm_rows_generic_kernel(
+    const T* __restrict__ x, const T* __restrict__ residual, const T* __restrict__ gamma,
+    const T* __restrict__ beta, T* __restrict__ out, int64_t rows, int64_t n, float eps) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row = (int64_t)blockIdx.x * kNormRowsPerBlock + threadIdx.x / kWave;
+  if (row >= rows) return;
+  const T* xr = x + row * n;
+  const T* rr = residual ? residual + row * n : nullptr;
+  auto value = [&](int64_t i) -> float {
+    return rr ? (float)(T)((float)xr[i] + (float)rr[i]) : (float)xr[i];
+  };
+  float sum = 0.0f;
+  for (int64_t i = lane; i < n; i += kWave) sum += value(i);
+  const float mean = wave_sum<T>(sum) / (float)n;
+  float sq = 0.0f;
+  for (int64_t i = lane; i < n; i += kWave) {
+    const float d = value(i) - mean;
+    sq += d * d;
+  }
+  const float rstd = 1.0f / sqrtf(wave_sum<T>(sq) / (float)n + eps);
+  T* orow = out + row * n;
+  for (int64_t i = lane; i < n; i += kWave) {
+    float v = (value(i) - mean) * rstd;
+    if (gamma) v = v * (float)gamma[i];
+    if (beta) v = v + (float)beta[i];
+    orow[i] = (T)v;
+  }
+}
+
+template <typename T, int P, int WAVES>
+static int launch_layer_norm_vec(const void* x, const void* residual, const void* gamma,
+                                 const void* beta, void* out, int64_t rows, int64_t n, double eps,
+                                 hipStream_t stream) {
+  constexpr int kRows = kNormRowsPerBlock / WAVES;
+  const int64_t blocks = (rows + kRows - 1) / kRows;
+  if (blocks > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "layer_norm: too many rows");
+  hipLaunchKernelGGL((layer_norm_rows_kernel<T, P, WAVES>), dim3((unsigned)blocks),
+                     dim3(kWave * kNormRowsPerBlock), 0, stream, static_cast<const T*>(x),
+                     static_cast<const T*>(residual), static_cast<const T*>(gamma),
+                     static_cast<const T*>(beta), static_cast<T*>(out), rows, (int)n, (float)eps);
+  return check_launch("layer_norm_rows_kernel");
+}
+
+template <typename T>
+static int launch_layer_norm(const void* x, const void* residual, const void* gamma, const void* beta,
+                             void* out, int64_t rows, int64_t n, double eps, hipStream_t stream) {
+  constexpr int kPer = 16 / sizeof(T);
+  const uintptr_t align = (uintptr_t)x | (uintptr_t)out | (uintptr_t)(residual ? residual : x);
+  const int64_t pieces = n / kPer;
+  if (n % kPer == 0 && align % 16 == 0 && pieces <= kWave * 4 * 4) {
+    if (pieces <= 64) return launch_layer_norm_vec<T, 1, 1>(x, residual, gamma, beta, out, rows, n, eps, stream);
+    if (pieces <= 128) return launch_layer_norm_vec<T, 2, 1>(x, residual, gamma, beta, out, rows, n, eps, stream);
+    if (pieces <= 256) return launch_layer_norm_vec<T, 1, 4>(x, residual, gamma, beta, out, rows, n, eps, stream);
+    if (pieces <= 512) return launch_layer_norm_vec<T, 2, 4>(x, residual, gamma, beta, out, rows, n, eps, stream);
+    return launch_layer_norm_vec<T, 4, 4>(x, residual, gamma, beta, out, rows, n, eps, stream);
+  }
+  const int64_t blocks = (rows + kNormRowsPerBlock - 1) / kNormRowsPerBlock;
+  if (blocks > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "layer_norm: too many rows");
+  hipLaunchKernelGGL((layer_norm_rows_generic_kernel<T>), dim3((unsigned)blocks),
+                     dim3(kWave * kNormRowsPerBlock), 0, stream, static_cast<const T*>(x),
+                     static_cast<const T*>(residual), static_cast<const T*>(gamma),
+                     static_cast<const T*>(beta), static_cast<T*>(out), rows, n, (float)eps);
+  return check_launch("layer_norm_rows_generic_kernel");
+}
+
+// out[i] = a[i] + alpha * b[i % period]   (period == numel: plain packed add)
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void add_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                                                  float alpha, T* __restrict__ out, int64_t numel,
+                                                  int64_t period) {
+  constexpr int kPer = VEC ? 16 / sizeof(T) : 1;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x * kPer;
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * kPer; i < numel; i += stride) {
+    if (VEC) {
+      // period is a multiple of kPer here, so a piece never wraps
+      const u32x4 ra = *reinterpret_cast<const u32x4*>(a + i);
+      const u32x4 rb = *reinterpret_cast<const u32x4*>(b + (period == numel ? i : i % period));
+      T va[kPer], vb[kPer], vo[kPer];
+      __builtin_memcpy(va, &ra, 16);
+      __builtin_memcpy(vb, &rb, 16);
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) vo[j] = (T)((float)va[j] + alpha * (float)vb[j]);
+      u32x4 o;
+      __builtin_memcpy(&o, vo, 16);
+      store16_stream(reinterpret_cast<char*>(out + i), o);
+    } else {
+      out[i] = (T)((float)a[i] + alpha * (float)b[period == numel ? i : i % period]);
+    }
+  }
+}
+
+template <typename T>
+static int launch_add(const void* a, const void* b, double alpha, void* out, int64_t numel,
+                      int64_t period, hipStream_t stream) {
+  constexpr int kPer = 16 / sizeof(T);
+  const uintptr_t align = (uintptr_t)a | (uintptr_t)b | (uintptr_t)out;
+  const bool vec = align % 16 == 0 && numel % kPer == 0 && period % kPer == 0;
+  const int64_t per_thread = vec ? kPer : 1;
+  int64_t blocks = (numel + 256 * per_thread - 1) / (256 * per_thread);
+  if (blocks > (1 << 20)) blocks = 1 << 20;   // grid-stride beyond that
+  const T* pa = static_cast<const T*>(a);
+  const T* pb = static_cast<const T*>(b);
+  T* po = static_cast<T*>(out);
+  if (vec) {
+    hipLaunchKernelGGL((add_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, stream, pa, pb,
+                       (float)alpha, po, numel, period);
+  } else {
+    hipLaunchKernelGGL((add_kernel<T, false>), dim3((unsigned)blocks), dim3(256), 0, stream, pa, pb,
+                       (float)alpha, po, numel, period);
+  }
+  return check_launch("add_kernel");
+}
+
+}  // namespace nt
+
+using namespace nt;
+
+extern "C" int nt_layer_norm(const void* x, const void* residual, const void* gamma, const void* beta,
+                             void* out, int64_t rows, int64_t n, double eps, int dtype, void* stream) {
+  if (rows < 0 || n < 0) return fail(NT_ERR_INVALID_ARGUMENT, "layer_norm: negative extent");
+  if (rows == 0 || n == 0) return NT_OK;
+  if (!x || !out) return fail(NT_ERR_INVALID_ARGUMENT, "layer_norm: NULL pointer");
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case NT_F32: return launch_layer_norm<float>(x, residual, gamma, beta, out, rows, n, eps, s);
+    case NT_F16: return launch_layer_norm<_Float16>(x, residual, gamma, beta, out, rows, n, eps, s);
+    case NT_BF16: return launch_layer_norm<__bf16>(x, residual, gamma, beta, out, rows, n, eps, s);
+    default: return fail(NT_ERR_UNSUPPORTED, "layer_norm: dtype %d is not f32, f16 or bf16", dtype);
+  }
+}
+
+extern "C" int nt_add_packed(const void* a, const void* b, double alpha, void* out, int64_t numel,
+                             int64_t period, int dtype, void* stream) {
+  if (numel < 0 || period < 0) return fail(NT_ERR_INVALID_ARGUMENT, "add_packed: negative extent");
+  if (numel == 0) return NT_OK;
+  if (period == 0 || numel % period != 0) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "add_packed: numel %lld is not a multiple of the period %lld",
+                (long long)numel, (long long)period);
+  }
+  if (!a || !b || !out) return fail(NT_ERR_INVALID_ARGUMENT, "add_packed: NULL pointer");
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case NT_F32: return launch_add<float>(a, b, alpha, out, numel, period, s);
+    case NT_F16: return launch_add<_Float16>(a, b, alpha, out, numel, period, s);
+    case NT_BF16: return launch_add<__bf16>(a, b, alpha, out, numel, period, s);
+    default: return fail(NT_ERR_UNSUPPORTED, "add_packed: dtype %d is not f32, f16 or bf16", dtype);
+  }
+}

@@ -252,6 +252,16 @@ class NestedTensor:
             raise RuntimeError("NestedTensor should consistent of 2d Tensors of size L x *")
         return torch.nn.utils.rnn.pack_sequence(self.to_tensor_list(), enforce_sorted=False)
 
+    # --- packed element-wise add (BinaryOps.cpp:12-115) ---
+    def __add__(self, other):
+        return torch.add(self, other)
+
+    def __radd__(self, other):
+        return torch.add(self, other)
+
+    def add(self, other, *, alpha=1):
+        return torch.add(self, other, alpha=alpha)
+
     # --- dispatch ---
     @classmethod
     def __torch_function__(cls, func, types, args=(), kwargs=None):
@@ -283,6 +293,20 @@ def _nn_functional_linear(input, weight, bias=None):
     return NestedTensorImpl(out.reshape(-1), sizes)
 
 
+def _nn_functional_layer_norm(input, normalized_shape, weight=None, bias=None, eps=1e-5):
+    return ops.layer_norm(input, normalized_shape, weight, bias, eps)
+
+
+def _add(input, other, *, alpha=1, out=None):
+    if out is not None:
+        raise NotImplementedError("add on a NestedTensor does not take out=.")
+    if not isinstance(input, NestedTensorImpl):      # tensor + nested
+        if alpha != 1:
+            raise NotImplementedError("tensor + alpha * nested is not on the packed path.")
+        input, other = other, input
+    return ops.add(input, other, alpha)
+
+
 def _get_is_contiguous(impl, memory_format=torch.contiguous_format):
     return memory_format == torch.contiguous_format
 
@@ -304,4 +328,9 @@ _HANDLERS = {
     _ns.get_is_contiguous: _get_is_contiguous,
     _ns.make_contiguous: lambda impl: impl,
     _ns.to_tensor_list: lambda impl: list(NestedTensor(impl).unbind()),
+    torch.nn.functional.layer_norm: _nn_functional_layer_norm,
+    torch.add: _add,
+    torch.Tensor.add: _add,
+    torch.Tensor.__add__: _add,
+    torch.Tensor.__radd__: _add,
 }

@@ -427,3 +427,75 @@ def bt_min_mha(num_heads, head_dim, dropout_p, training, query, key, value, attr
     _check_mha_inputs(query, key, value)
     return mha_packed(num_heads, head_dim, query, query, query, attr_kernel, attr_bias, scaling,
                       out_proj_weight, None)
+
+
+# ---- row-wise ops on the packed buffer: the steps either side of attention ----
+
+def layer_norm(impl, normalized_shape, weight=None, bias=None, eps=1e-5, residual=None):
+    """NestedTensor_layer_norm (functions.cpp:65-112; device fast path
+    cuda/layernorm.cpp:14-76): normalise over the regular last dim, one launch
+    over the packed [T, n] view (nt_layer_norm).  `residual` (a nested tensor of
+    the same nested size) is added first, rounded to the storage type, as
+    ``layer_norm(nt + residual)`` does in two ops (BinaryOps.cpp:18-44)."""
+    normalized_shape = tuple(normalized_shape) if not isinstance(normalized_shape, int) \
+        else (normalized_shape,)
+    if len(normalized_shape) != 1:
+        raise RuntimeError("Currently only singleton tuples of integers supported for layer_norm.")
+    opt = impl.opt_sizes()
+    last = impl.dim() - 1
+    if opt[last] is None:
+        raise RuntimeError("Cannot normalize across irregular dimension %d" % last)
+    n = opt[last]
+    if n != normalized_shape[0]:
+        raise RuntimeError("Normalized shape [%d] does not match the size of the last dimension (%d) of input."
+                           % (normalized_shape[0], n))
+    if (weight is None) != (bias is None):
+        raise RuntimeError("Either both weight and bias are used or not.")
+    buf = impl.buffer
+    _C.require_device(buf, "layer_norm")
+    for t in (weight, bias):
+        if t is not None and (t.dtype != buf.dtype or t.device != buf.device or t.numel() != n):
+            raise RuntimeError("layer_norm: weight and bias must have %d elements of the input's dtype "
+                               "on the input's device" % n)
+    res_buf = None
+    if residual is not None:
+        if not torch.equal(residual.sizes, impl.sizes) or residual.buffer.dtype != buf.dtype:
+            raise RuntimeError("layer_norm: the residual must have the nested size and dtype of the input")
+        res_buf = residual.buffer
+    out = torch.empty_like(buf)
+    rows = buf.numel() // n if n > 0 else 0
+    weight = weight.contiguous() if weight is not None else None
+    bias = bias.contiguous() if bias is not None else None
+    with torch.cuda.device(buf.device):
+        _C.check(_C.lib.nt_layer_norm(_C.ptr(buf), _C.ptr(res_buf), _C.ptr(weight), _C.ptr(bias),
+                                      _C.ptr(out), rows, n, float(eps), _C.dtype_code(buf.dtype),
+                                      _C.current_stream(buf.device)))
+    return impl.with_buffer(out)
+
+
+def add(impl, other, alpha=1):
+    """NestedTensor_add_Tensor on the packed buffers (BinaryOps.cpp:12-115): the
+    two cases that need no per-constituent work, nested + nested of equal nested
+    size (:18-44) and nested with a regular last dim + 1-D tensor (:97-107)."""
+    buf = impl.buffer
+    _C.require_device(buf, "add")
+    if isinstance(other, NestedTensorImpl):
+        if other.sizes.shape != impl.sizes.shape or not torch.equal(other.sizes, impl.sizes):
+            raise NotImplementedError("add of nested tensors of different nested size is not on the packed path.")
+        b, period = other.buffer, buf.numel()
+    elif isinstance(other, torch.Tensor) and other.dim() == 1:
+        opt = impl.opt_sizes()
+        if opt[impl.dim() - 1] is None or opt[impl.dim() - 1] != other.size(0):
+            raise NotImplementedError("add of a 1-D tensor needs a regular last dim of the same size.")
+        b, period = other.contiguous(), other.size(0)
+    else:
+        raise NotImplementedError("add: only nested + nested (same nested size) and nested + 1-D tensor "
+                                  "are on the packed path.")
+    if b.dtype != buf.dtype or b.device != buf.device:
+        raise RuntimeError("add: both operands must have the same dtype and device")
+    out = torch.empty_like(buf)
+    if buf.numel() > 0:
+        with torch.cuda.device(buf.device):
+            _C.check(_C.lib.nt_add_packed(_C.ptr(buf), _C.ptr(b), float(alpha), _C.ptr(out), buf.numel(),
+                                          period, _C.dtype_code(buf.dtype), _C.current_stream(buf.device)))
+    return impl.with_buffer(out)

@@ -36,6 +36,12 @@ Pinning (what each part was checked against, see tests/test_oracle_*.py):
   attention with ``key_padding_mask`` (:1118-1140), plus an fp64 brute force.
 * bt_min_mha: equality with min_mha at 1e-5 for zero out-bias
   (test/test_nested_tensor_functional.py:1115).
+* layer_norm (written out in fp64, not a call of torch's): torch's
+  ``layer_norm`` per constituent, which is what the reference's test compares
+  with (test/test_nested_tensor_functional.py:894-917), and the closed forms
+  (zero mean, variance var/(var + eps), shift invariance).
+* add: ``torch.add`` on the packed buffers / per constituent
+  (test/test_nested_tensor_functional.py's add cases reduce to it).
 
 Two reference behaviours are restated here but deliberately not followed by
 the product: the uint8-vs-bool mask dtype of merge_tensor_mask
@@ -59,3 +65,4 @@ from .masking import (  # noqa: F401
     nested_tensor_from_padded_tensor,
 )
 from .mha import min_mha, bt_min_mha  # noqa: F401
+from .rowops import layer_norm, add  # noqa: F401

@@ -1,0 +1,122 @@
+"""Parity of the packed row-wise ops (layer norm, packed add) with the oracle.
+
+Tolerances: fp32 <= 1e-5 relative to the output scale, fp16 / bf16 <= 2e-2
+absolute (outputs are O(1)).  The size list is the reference's
+(test/test_nested_tensor_functional.py:935-939) plus the encoder widths of the
+BASELINE configurations."""
+
+import pytest
+import torch
+
+import nestedtensor_amd as nt
+import oracle
+from nestedtensor_amd import ops
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda", 0)
+
+
+def _tol(dtype):
+    return 1e-5 if dtype == torch.float32 else 2e-2
+
+
+def _close(got, exp, dtype):
+    got, exp = got.float().cpu(), exp.float()
+    assert got.shape == exp.shape and torch.isfinite(got).all()
+    err = (got - exp).abs().max().item()
+    if dtype == torch.float32:
+        assert err <= 1e-5 * max(1.0, exp.abs().max().item()), err
+    else:
+        assert err <= 2e-2, err
+
+
+def _tensors(shapes, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    return [(torch.randn(*s, generator=g) * 2 + 0.5).to(dtype) for s in shapes]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("size", [1024, 512, 256, 128, 2, 4, 32, 768, 2048, 4096, 100, 7])
+def test_layer_norm_module(size, dtype):
+    # reference test: two [2, size] constituents repeated; here ragged lengths too
+    ts = _tensors([(2, size), (2, size), (5, size), (1, size), (17, size)], dtype, size)
+    a = nt.nested_tensor(ts, device=DEV, dtype=dtype)
+    ln = torch.nn.LayerNorm(size).to(dtype)
+    with torch.no_grad():
+        ln.weight.copy_(torch.randn(size))
+        ln.bias.copy_(torch.randn(size))
+    got = ln.to(DEV)(a)
+    assert isinstance(got, nt.NestedTensor) and got.nested_size() == a.nested_size()
+    exp = oracle.layer_norm(oracle.ref_nested_tensor(ts, dtype=dtype), (size,), ln.weight.detach().cpu(),
+                            ln.bias.detach().cpu(), ln.eps)
+    _close(got._impl.buffer, exp.buffer, dtype)
+
+
+def test_layer_norm_no_affine_and_4d():
+    ts = _tensors([(3, 2, 64), (1, 5, 64)], torch.float32, 5)
+    a = nt.nested_tensor(ts, device=DEV)
+    got = torch.nn.functional.layer_norm(a, (64,))
+    exp = oracle.layer_norm(oracle.ref_nested_tensor(ts), 64)
+    _close(got._impl.buffer, exp.buffer, torch.float32)
+
+
+def test_layer_norm_errors():
+    a = nt.nested_tensor([torch.randn(3, 4), torch.randn(2, 5)], device=DEV)
+    with pytest.raises(RuntimeError, match="Cannot normalize across irregular dimension 2"):
+        torch.nn.functional.layer_norm(a, (4,))
+    a = nt.nested_tensor([torch.randn(3, 4), torch.randn(2, 4)], device=DEV)
+    with pytest.raises(RuntimeError, match=r"Normalized shape \[3\] does not match the size of the last dimension \(4\) of input."):
+        torch.nn.functional.layer_norm(a, (3,))
+    with pytest.raises(RuntimeError, match="Currently only singleton tuples of integers supported for layer_norm."):
+        torch.nn.functional.layer_norm(a, (3, 2, 4))
+    with pytest.raises(RuntimeError, match="Either both weight and bias are used or not."):
+        torch.nn.functional.layer_norm(a, (4,), torch.ones(4, device=DEV), None)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_add_nested_and_vector(dtype):
+    shapes = [(3, 40), (7, 40), (1, 40)]
+    ta, tb = _tensors(shapes, dtype, 1), _tensors(shapes, dtype, 2)
+    a, b = nt.nested_tensor(ta, device=DEV, dtype=dtype), nt.nested_tensor(tb, device=DEV, dtype=dtype)
+    ra, rb = oracle.ref_nested_tensor(ta, dtype=dtype), oracle.ref_nested_tensor(tb, dtype=dtype)
+    # one rounding of an fp32 sum: bit-exact against at::add
+    assert torch.equal((a + b)._impl.buffer.cpu(), oracle.add(ra, rb).buffer)
+    assert torch.equal(torch.add(a, b, alpha=2)._impl.buffer.cpu(), oracle.add(ra, rb, alpha=2).buffer)
+    v = torch.randn(40, generator=torch.Generator().manual_seed(3)).to(dtype)
+    assert torch.equal((a + v.to(DEV))._impl.buffer.cpu(), oracle.add(ra, v).buffer)
+    assert torch.equal((v.to(DEV) + a)._impl.buffer.cpu(), oracle.add(ra, v).buffer)
+    odd = nt.nested_tensor(_tensors([(3, 7), (2, 7)], dtype, 4), device=DEV, dtype=dtype)   # unaligned rows
+    ro = oracle.ref_nested_tensor(_tensors([(3, 7), (2, 7)], dtype, 4), dtype=dtype)
+    v7 = torch.arange(7.0).to(dtype)
+    assert torch.equal((odd + v7.to(DEV))._impl.buffer.cpu(), oracle.add(ro, v7).buffer)
+    with pytest.raises(NotImplementedError):
+        a + odd
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_residual_layer_norm_equals_two_ops(dtype):
+    # ops.layer_norm(x, residual=r) == layer_norm(x + r): the sum is rounded to the
+    # storage type first, so the fused launch is bit-identical to the two launches
+    E = 768
+    shapes = [(L, E) for L in (5, 131, 64, 1)]
+    tx, tr = _tensors(shapes, dtype, 7), _tensors(shapes, dtype, 8)
+    x, r = nt.nested_tensor(tx, device=DEV, dtype=dtype), nt.nested_tensor(tr, device=DEV, dtype=dtype)
+    g = torch.Generator().manual_seed(9)
+    w, b = torch.randn(E, generator=g).to(dtype).to(DEV), torch.randn(E, generator=g).to(dtype).to(DEV)
+    fused = ops.layer_norm(x._impl, (E,), w, b, 1e-5, residual=r._impl)
+    two = torch.nn.functional.layer_norm(x + r, (E,), w, b, 1e-5)
+    assert torch.equal(fused.buffer, two._impl.buffer)
+    exp = oracle.layer_norm(oracle.add(oracle.ref_nested_tensor(tx, dtype=dtype), oracle.ref_nested_tensor(tr, dtype=dtype)),
+                            (E,), w.cpu(), b.cpu(), 1e-5)
+    _close(fused.buffer, exp.buffer, dtype)
+
+
+def test_row_ops_at_encoder_size_properties():
+    # C3-sized buffer: rows normalised without affine have mean 0 and variance 1
+    g = torch.Generator().manual_seed(11)
+    lens = [int(v) for v in torch.randint(32, 513, (32,), generator=g)]
+    ts = [torch.randn(L, 768, generator=g).half() * 3 + 1 for L in lens]
+    a = nt.nested_tensor(ts, device=DEV, dtype=torch.float16)
+    y = torch.nn.functional.layer_norm(a, (768,))._impl.buffer.float().reshape(-1, 768)
+    assert y.mean(1).abs().max().item() < 2e-3
+    assert (y.var(1, unbiased=False) - 1).abs().max().item() < 5e-3

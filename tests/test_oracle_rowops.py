@@ -1,0 +1,63 @@
+"""Pins oracle.layer_norm / oracle.add (CPU only)."""
+import pytest
+import torch
+
+import oracle
+
+
+def _nt(shapes, dtype=torch.float32, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return oracle.ref_nested_tensor([torch.randn(*s, generator=g) * 3 + 1 for s in shapes], dtype=dtype)
+
+
+@pytest.mark.parametrize("size", [1024, 512, 256, 128, 2, 4, 32, 7])
+def test_layer_norm_matches_torch_per_constituent(size):
+    # the reference's own check (test/test_nested_tensor_functional.py:894-917):
+    # nn.LayerNorm applied to the nested tensor equals it applied per constituent
+    nt = _nt([(2, size), (2, size), (5, size), (1, size)], seed=size)
+    ln = torch.nn.LayerNorm(size)
+    with torch.no_grad():
+        ln.weight.copy_(torch.randn(size))
+        ln.bias.copy_(torch.randn(size))
+    got = oracle.layer_norm(nt, (size,), ln.weight.detach(), ln.bias.detach(), ln.eps)
+    for a, t in zip(got.unbind(), nt.unbind()):
+        exp = ln(t).detach()
+        assert (a - exp).abs().max() <= 2e-6 * max(1.0, exp.abs().max().item())
+
+
+def test_layer_norm_closed_forms():
+    nt = _nt([(3, 64), (9, 64)], seed=3)
+    eps = 1e-5
+    y = oracle.layer_norm(nt, 64, None, None, eps)
+    for a, t in zip(y.unbind(), nt.unbind()):
+        var = t.double().var(-1, unbiased=False)
+        assert a.double().mean(-1).abs().max() < 1e-6                                    # zero mean
+        assert (a.double().var(-1, unbiased=False) - var / (var + eps)).abs().max() < 1e-5  # var / (var + eps)
+    shifted = oracle.ref_nested_tensor([t.double() + 5.0 for t in nt.unbind()], dtype=torch.float64)
+    y64 = oracle.layer_norm(oracle.ref_nested_tensor(nt.unbind(), dtype=torch.float64), 64, None, None, eps)
+    ys = oracle.layer_norm(shifted, 64, None, None, eps)
+    for a, b in zip(y64.unbind(), ys.unbind()):
+        assert (a - b).abs().max() < 1e-9                                                  # shift invariance
+
+
+def test_layer_norm_errors():
+    nt = _nt([(3, 4), (2, 5)])
+    with pytest.raises(RuntimeError, match="Cannot normalize across irregular dimension 2"):
+        oracle.layer_norm(nt, 4)
+    nt = _nt([(3, 4), (2, 4)])
+    with pytest.raises(RuntimeError, match=r"Normalized shape \[3\] does not match the size of the last dimension \(4\) of input."):
+        oracle.layer_norm(nt, 3)
+    with pytest.raises(RuntimeError, match="Currently only singleton tuples of integers supported for layer_norm."):
+        oracle.layer_norm(nt, (3, 2, 4))
+    with pytest.raises(RuntimeError, match="Either both weight and bias are used or not."):
+        oracle.layer_norm(nt, 4, torch.ones(4), None)
+
+
+def test_add_matches_packed_buffer_add():
+    a = _nt([(3, 8), (5, 8)], seed=1)
+    b = _nt([(3, 8), (5, 8)], seed=2)
+    got = oracle.add(a, b, alpha=2)
+    assert torch.equal(got.buffer, a.buffer + 2 * b.buffer)          # BinaryOps.cpp:18-44
+    v = torch.arange(8.0)
+    got = oracle.add(a, v)
+    assert torch.equal(got.buffer, (a.buffer.reshape(-1, 8) + v).reshape(-1))   # BinaryOps.cpp:97-107
