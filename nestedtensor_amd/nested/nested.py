@@ -329,6 +329,9 @@ _HANDLERS = {
     _ns.make_contiguous: lambda impl: impl,
     _ns.to_tensor_list: lambda impl: list(NestedTensor(impl).unbind()),
     torch.nn.functional.layer_norm: _nn_functional_layer_norm,
+    torch.conv2d: ops.conv2d,
+    torch.nn.functional.max_pool2d: ops.max_pool2d,
+    torch.max_pool2d: ops.max_pool2d,
     torch.add: _add,
     torch.Tensor.add: _add,
     torch.Tensor.__add__: _add,

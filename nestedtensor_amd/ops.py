@@ -499,3 +499,60 @@ def add(impl, other, alpha=1):
             _C.check(_C.lib.nt_add_packed(_C.ptr(buf), _C.ptr(b), float(alpha), _C.ptr(out), buf.numel(),
                                           period, _C.dtype_code(buf.dtype), _C.current_stream(buf.device)))
     return impl.with_buffer(out)
+
+
+# ---- dense ops called through pad -> op -> un-pad (pooling.cpp:41-57, conv2d.cpp:77-92) ----
+
+def _pair(v):
+    if isinstance(v, int):
+        return (v, v)
+    v = tuple(int(x) for x in v)
+    return (v[0], v[0]) if len(v) == 1 else v
+
+
+def _dense_via_padding(impl, pad_value, dense_op, out_channels, k, stride, padding, dilation):
+    """to_padded_tensor -> one dense call over the whole batch -> from_padded_tensor
+    with the per-constituent output sizes
+    ``(s + 2 p - d (k - 1) - 1) // stride + 1`` (pooling.cpp:50-53, conv2d.cpp:80-84)."""
+    if impl.dim() != 4:
+        raise RuntimeError("Input must be 4 dimensional.")
+    _C.require_device(impl.buffer, "dense op on a NestedTensor")
+    data = to_padded_tensor(impl, pad_value)
+    result = dense_op(data).contiguous()
+    sizes = impl.sizes.clone()
+    if out_channels is not None:
+        sizes[:, 0] = out_channels
+    for j in (0, 1):
+        sizes[:, 1 + j] = (sizes[:, 1 + j] + 2 * padding[j] - dilation[j] * (k[j] - 1) - 1) // stride[j] + 1
+    if bool((sizes <= 0).any()):
+        raise RuntimeError("Output size is too small")
+    target = NestedTensorImpl(torch.empty(0, dtype=result.dtype, device=result.device), sizes)
+    return from_padded_tensor(result, target)
+
+
+def max_pool2d(impl, kernel_size, stride=None, padding=0, dilation=1, ceil_mode=False,
+               return_indices=False):
+    """NestedTensor_max_pool2d (pooling.cpp:34-75).  The reference takes the
+    padded route for fp16 only and pads with 0; here every dtype takes it and the
+    pad value is -inf, which makes the result equal to pooling each constituent on
+    its own (what the reference's tests assert) also for windows that reach past a
+    constituent's edge."""
+    if ceil_mode or return_indices:
+        raise NotImplementedError("max_pool2d on a NestedTensor: ceil_mode / return_indices are not supported.")
+    k = _pair(kernel_size)
+    s = _pair(stride) if stride not in (None, [], ()) else k
+    p, d = _pair(padding), _pair(dilation)
+    return _dense_via_padding(
+        impl, float("-inf"),
+        lambda x: torch.nn.functional.max_pool2d(x, k, s, p, d, False), None, k, s, p, d)
+
+
+def conv2d(impl, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
+    """NestedTensor_conv2d, padded route (conv2d.cpp:77-92; the reference takes it
+    for fp16).  Padding with 0 is exact: a convolution pads with zeros itself."""
+    if isinstance(padding, str):
+        raise NotImplementedError("conv2d on a NestedTensor: string padding is not supported.")
+    s, p, d = _pair(stride), _pair(padding), _pair(dilation)
+    k = (weight.size(2), weight.size(3))
+    return _dense_via_padding(
+        impl, 0.0, lambda x: torch.conv2d(x, weight, bias, s, p, d, groups), weight.size(0), k, s, p, d)

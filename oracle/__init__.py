@@ -40,6 +40,10 @@ Pinning (what each part was checked against, see tests/test_oracle_*.py):
   ``layer_norm`` per constituent, which is what the reference's test compares
   with (test/test_nested_tensor_functional.py:894-917), and the closed forms
   (zero mean, variance var/(var + eps), shift invariance).
+* max_pool2d / conv2d: the per-constituent mapping the reference's tests assert
+  (test/test_nested_tensor_functional.py:44-135, 251-266); the output sizes are
+  cross-checked against the closed form of pooling.cpp:50-53 / conv2d.cpp:80-84
+  in tests/test_oracle_rowops.py.
 * add: ``torch.add`` on the packed buffers / per constituent
   (test/test_nested_tensor_functional.py's add cases reduce to it).
 
@@ -66,3 +70,4 @@ from .masking import (  # noqa: F401
 )
 from .mha import min_mha, bt_min_mha  # noqa: F401
 from .rowops import layer_norm, add  # noqa: F401
+from .dense import max_pool2d, conv2d  # noqa: F401

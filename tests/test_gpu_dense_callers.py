@@ -1,0 +1,74 @@
+"""max_pool2d / conv2d on a NestedTensor through pad -> dense op -> un-pad
+(pooling.cpp:41-57, conv2d.cpp:77-92), against the per-constituent oracle.  The
+shapes are the reference's (test/test_nested_tensor_functional.py:81-135,
+251-266, 788-811, the 500x600 images scaled down where noted)."""
+
+import pytest
+import torch
+
+import nestedtensor_amd as nt
+import oracle
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda", 0)
+
+
+def _rand(shapes, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randn(*s, generator=g).to(dtype) for s in shapes]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("shapes", [[(3, 500, 600), (3, 128, 128)], [(3, 50, 60), (3, 50, 60)],
+                                    [(2, 7, 5), (2, 3, 9), (2, 8, 8)]])
+def test_max_pool2d_equals_per_constituent(shapes, dtype):
+    ts = _rand(shapes, dtype, 1)
+    ts = [t - 3.0 for t in ts]      # mostly negative: a 0-padded window would show
+    a = nt.nested_tensor(ts, device=DEV, dtype=dtype)
+    got = torch.nn.functional.max_pool2d(a, kernel_size=(3, 3), stride=(2, 2), padding=(1, 1),
+                                         dilation=(1, 1), ceil_mode=False)
+    exp = oracle.max_pool2d(oracle.ref_nested_tensor(ts, dtype=dtype), (3, 3), (2, 2), (1, 1), (1, 1))
+    assert got.nested_size() == nt.nested_tensor(list(exp.unbind())).nested_size()
+    assert torch.equal(got._impl.buffer.cpu(), exp.buffer)          # max is exact
+    pool = torch.nn.MaxPool2d(kernel_size=(3, 3), stride=2, padding=(1, 1), dilation=1, ceil_mode=False)
+    assert torch.equal(pool(a)._impl.buffer.cpu(), exp.buffer)
+
+
+CONV_CASES = [
+    # shapes, weight shape, stride, padding, dilation, groups
+    ([(2, 2, 3), (2, 4, 2), (2, 2, 2)], (3, 2, 1, 1), 1, 0, 1, 1),
+    ([(2, 4, 5), (2, 5, 3), (2, 3, 3)], (3, 2, 3, 3), 1, 0, 1, 1),
+    ([(32, 4, 5), (32, 5, 3), (32, 3, 3)], (32, 1, 3, 3), 1, 1, 1, 32),
+    ([(4, 3, 2), (4, 3, 3), (4, 2, 3)], (5, 4, 2, 2), 1, 1, 1, 1),
+    ([(8, 40, 33), (8, 17, 64)], (16, 8, 3, 3), 2, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv2d_equals_per_constituent(case, dtype):
+    shapes, wshape, stride, padding, dilation, groups = case
+    ts = _rand(shapes, dtype, 2)
+    g = torch.Generator().manual_seed(3)
+    w = (torch.randn(*wshape, generator=g) * 0.3).to(dtype)
+    b = torch.randn(wshape[0], generator=g).to(dtype)
+    a = nt.nested_tensor(ts, device=DEV, dtype=dtype)
+    got = torch.conv2d(a, w.to(DEV), b.to(DEV), stride=stride, padding=padding, dilation=dilation,
+                       groups=groups)
+    # oracle in fp32 on the host (no fp16 convolution there), rounded once
+    ref = oracle.conv2d(oracle.ref_nested_tensor([t.float() for t in ts], dtype=torch.float32), w.float(),
+                        b.float(), stride, padding, dilation, groups)
+    assert [tuple(x.shape) for x in got.unbind()] == [tuple(x.shape) for x in ref.unbind()]
+    err = (got._impl.buffer.float().cpu() - ref.buffer).abs().max().item()
+    scale = max(1.0, ref.buffer.abs().max().item())
+    assert err <= (1e-5 if dtype == torch.float32 else 2e-2) * scale, err
+    # and the same dense library applied per constituent on the device
+    for gi, t in zip(got.unbind(), ts):
+        ti = torch.conv2d(t.to(DEV).unsqueeze(0), w.to(DEV), b.to(DEV), stride, padding, dilation, groups).squeeze(0)
+        assert (gi.float() - ti.float()).abs().max().item() <= (1e-5 if dtype == torch.float32 else 2e-2) * scale
+
+
+def test_dense_callers_errors():
+    a = nt.nested_tensor([torch.randn(3, 4), torch.randn(2, 4)], device=DEV)
+    with pytest.raises(RuntimeError, match="Input must be 4 dimensional."):
+        torch.nn.functional.max_pool2d(a, 2)

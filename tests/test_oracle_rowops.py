@@ -61,3 +61,18 @@ def test_add_matches_packed_buffer_add():
     v = torch.arange(8.0)
     got = oracle.add(a, v)
     assert torch.equal(got.buffer, (a.buffer.reshape(-1, 8) + v).reshape(-1))   # BinaryOps.cpp:97-107
+
+
+def test_dense_ops_output_sizes_closed_form():
+    # pooling.cpp:50-53 / conv2d.cpp:80-84: (s + 2p - d(k-1) - 1) // stride + 1
+    nt = _nt([(3, 50, 60), (3, 28, 17), (3, 9, 33)])
+    k, s, p, d = (3, 3), (2, 2), (1, 1), (1, 1)
+    got = oracle.max_pool2d(nt, k, s, p, d)
+    for t, o in zip(nt.unbind(), got.unbind()):
+        exp = tuple((t.shape[1 + j] + 2 * p[j] - d[j] * (k[j] - 1) - 1) // s[j] + 1 for j in (0, 1))
+        assert tuple(o.shape) == (3,) + exp
+    w = torch.randn(5, 3, 2, 2)
+    got = oracle.conv2d(nt, w, None, (1, 2), (1, 0), (2, 1))
+    for t, o in zip(nt.unbind(), got.unbind()):
+        exp = ((t.shape[1] + 2 - 2 * 1 - 1) // 1 + 1, (t.shape[2] + 0 - 1 * 1 - 1) // 2 + 1)
+        assert tuple(o.shape) == (5,) + exp
