@@ -422,6 +422,40 @@ def bench_rows(args, torch, dev):
         rows[tag + "_packed_add_fp16"] = entry(ms_add, 3 * nb, None, rows=T_rw, width=E_rw)
         del buf, x_rw, r_rw
 
+    # ---- interop formats built from the offsets array ------------------------------
+    g = torch.Generator().manual_seed(1010 + 2)
+    lens_io = [int(v) for v in torch.randint(32, 513, (32,), generator=g)]
+    V_io, E_io = 30522, 768
+    ids_io = [torch.randint(V_io, (L,), generator=g) for L in lens_io]
+    table = torch.randn(V_io, E_io, generator=g).half().to(dev)
+    a_ids = nt.nested_tensor(ids_io, device=dev, dtype=torch.int64)
+    T_io = sum(lens_io)
+    ms_emb = _time_gpu(torch, lambda: torch.nn.functional.embedding(a_ids, table))
+    ms_bag = _time_gpu(torch, lambda: torch.nn.functional.embedding_bag(a_ids, table, mode="sum"))
+    x_io = torch.nn.functional.embedding(a_ids, table)
+    ms_ps = _time_gpu(torch, lambda: x_io.to_packed_sequence())
+    c_emb = c_ps = None
+    if cpu:
+        ref_ids = oracle.ref_nested_tensor(ids_io, dtype=torch.int64)
+        tcpu = table.cpu()
+        c_emb = _time_cpu(lambda: oracle.embedding(tcpu, ref_ids), 2)
+        ref_x = oracle.ref_nested_tensor([p.cpu() for p in x_io.unbind()], dtype=torch.float16)
+        c_ps = _time_cpu(lambda: oracle.to_packed_sequence(ref_x), 2)
+    rows["C3_embedding_fp16"] = entry(ms_emb, T_io * (8 + 2 * 2 * E_io), c_emb,
+                                      note="includes the device-to-host read of the out-of-range counter")
+    rows["C3_embedding_bag_sum_fp16"] = entry(ms_bag, T_io * (8 + 2 * E_io) + 32 * 2 * E_io)
+    rows["C3_to_packed_sequence_fp16"] = entry(ms_ps, T_io * (8 + 2 * 2 * E_io), c_ps)
+    big_T, big_E = 1 << 20, 1024
+    big_idx = torch.randint(V_io, (big_T,), device=dev)
+    big_tab = torch.randn(V_io, big_E, device=dev, dtype=torch.float16)
+    big_out = torch.empty(big_T, big_E, device=dev, dtype=torch.float16)
+    stream = _C.current_stream(dev)
+    ms_big = _time_gpu(torch, lambda: _C.check(_C.lib.nt_gather_rows(
+        _C.ptr(big_tab), V_io, big_E * 2, _C.ptr(big_idx), _C.ptr(big_out), big_T, None, stream)))
+    rows["large_gather_rows_fp16"] = entry(ms_big, big_T * (8 + 2 * 2 * big_E), None, rows=big_T, width=big_E,
+                                           note="2 GiB written; the 62 MB table is re-read from cache")
+    del big_idx, big_tab, big_out
+
     # ---- C4: bt_min_mha bf16, high raggedness ---------------------------------
     g = torch.Generator().manual_seed(1010 + 3)
     raw = torch.empty(128).exponential_(1.0 / 96.0, generator=g)

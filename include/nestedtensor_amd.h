@@ -214,6 +214,47 @@ int nt_layer_norm(const void* x, const void* residual, const void* gamma, const 
 int nt_add_packed(const void* a, const void* b, double alpha, void* out, int64_t numel,
                   int64_t period, int dtype, void* stream);
 
+/* ---- consumers of the offsets array (interop formats) ------------------- */
+
+/* dst row r = src row index[r]; rows of row_bytes bytes, src has src_rows rows.
+ * An index outside [0, src_rows) gives a zero row and, if oob_count is not NULL,
+ * increments *oob_count (device int32).  With src = an embedding table and index
+ * = the packed index buffer of a nested tensor this is the reference's packed
+ * embedding (NestedTensor_embedding, nestedtensor/csrc/functions.cpp:27-55: one
+ * at::embedding over the buffer); with the index built by
+ * nt_packed_sequence_index it re-orders token rows for a PackedSequence. */
+int nt_gather_rows(const void* src, int64_t src_rows, int64_t row_bytes, const int64_t* index,
+                   void* dst, int64_t n_rows, int32_t* oob_count, void* stream);
+
+/* Row order of torch.nn.utils.rnn.PackedSequence for the sequences of a nested
+ * tensor [B, L_i, *]: index_out[step_starts[t] + rank[b]] = offsets[b] + t for
+ * every token t of every sequence b.  offsets int64[B + 1] are token offsets,
+ * rank[b] is the position of sequence b in the order of decreasing length,
+ * step_starts[t] the number of rows of all time steps before t (exclusive prefix
+ * sum of batch_sizes; at least max L_i entries).  All device arrays.  Replaces
+ * the unbind + torch.nn.utils.rnn.pack_sequence of NestedTensor.to_packed_sequence
+ * (nestedtensor/nested/nested.py:484-488). */
+int nt_packed_sequence_index(const int64_t* offsets, const int64_t* rank, const int64_t* step_starts,
+                             int64_t B, int64_t total_rows, int64_t* index_out, void* stream);
+
+/* out[offsets[b] + j] = j for 0 <= j < offsets[b+1] - offsets[b]: the column
+ * indices of the CSR view of a nested tensor of 1-D constituents, whose
+ * crow_indices are offsets themselves (NestedTensor_to_sparse_csr,
+ * nestedtensor/csrc/nested_tensor_impl.h:326-349, which concatenates one
+ * torch::arange per constituent on the host).  max_len >= the longest row. */
+int nt_ragged_arange(const int64_t* offsets, int64_t B, int64_t max_len, int64_t* out, void* stream);
+
+/* out[b, :] = sum (mode 0), mean (1) or max (2) over t in [offsets[b], offsets[b+1])
+ * of weight[indices[t], :]; weight [num_embeddings, n] with row stride ldw, fp32
+ * accumulation in token order, empty bags give 0.  The bags are the constituents
+ * of a nested tensor of 1-D index tensors and offsets is its offsets array: the
+ * reference builds the same offsets in a host loop and calls torch.embedding_bag
+ * (nestedtensor/nested/nested.py:43-118).  Indices out of range are skipped and
+ * counted in *oob_count if it is not NULL. */
+int nt_embedding_bag(const void* weight, int64_t ldw, int64_t num_embeddings, const int64_t* indices,
+                     const int64_t* offsets, void* out, int64_t B, int64_t n, int mode, int dtype,
+                     int32_t* oob_count, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,229 @@
+// Consumers of the offsets array of a nested tensor (gfx950): row gather
+// (embedding on packed indices, time-major re-ordering for a PackedSequence),
+// per-constituent reduction of gathered rows (embedding_bag), and the column
+// indices of the CSR view.  All are HBM-bound integer / copy work; the reference
+// builds each of them on the host or with one ATen call per constituent
+// (nestedtensor/csrc/functions.cpp:14-63, nestedtensor/nested/nested.py:43-118,
+// 484-488, nestedtensor/csrc/nested_tensor_impl.h:326-349).
+#include "nt_common.h"
+
+namespace nt {
+
+// dst row r = src row index[r]; rows are row_bytes long, moved in pieces of UNIT
+// bytes (the largest power of two that divides row_bytes and both base
+// addresses).  An index outside [0, src_rows) yields a zero row and is counted.
+template <int UNIT>
+__global__ __launch_bounds__(256) void gather_rows_kernel(
+    const char* __restrict__ src, int64_t src_rows, int64_t row_bytes,
+    const int64_t* __restrict__ index, char* __restrict__ dst, int64_t n_rows,
+    int32_t* __restrict__ oob) {
+  const int64_t pieces_per_row = row_bytes / UNIT;
+  const int64_t total = n_rows * pieces_per_row;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; id < total; id += stride) {
+    const int64_t r = id / pieces_per_row;
+    const int64_t p = id - r * pieces_per_row;
+    const int64_t s = index[r];
+    const bool ok = s >= 0 && s < src_rows;
+    if (!ok && p == 0 && oob) atomicAdd(oob, 1);
+    char* d = dst + r * row_bytes + p * UNIT;
+    const char* q = src + (ok ? s : 0) * row_bytes + p * UNIT;
+    if (UNIT == 16) {
+      u32x4 v = *reinterpret_cast<const u32x4*>(q);
+      if (!ok) v = u32x4{0, 0, 0, 0};
+      store16_stream(d, v);
+    } else if (UNIT == 8) {
+      *reinterpret_cast<uint64_t*>(d) = ok ? *reinterpret_cast<const uint64_t*>(q) : 0ull;
+    } else if (UNIT == 4) {
+      *reinterpret_cast<uint32_t*>(d) = ok ? *reinterpret_cast<const uint32_t*>(q) : 0u;
+    } else if (UNIT == 2) {
+      *reinterpret_cast<uint16_t*>(d) = ok ? *reinterpret_cast<const uint16_t*>(q) : (uint16_t)0;
+    } else {
+      *d = ok ? *q : (char)0;
+    }
+  }
+}
+
+// b with offsets[b] <= i < offsets[b + 1] (offsets non-decreasing, offsets[B] > i)
+__device__ __forceinline__ int64_t find_segment(const int64_t* offsets, int64_t B, int64_t i) {
+  int64_t lo = 0, hi = B;   // answer in [lo, hi)
+  while (hi - lo > 1) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (offsets[mid] <= i) {
+      lo = mid;
+    } else {
+      hi = mid;
+    }
+  }
+  return lo;
+}
+
+// Time-major order of a PackedSequence: token t of the sequence at sorted
+// position r goes to row step_starts[t] + r.  index_out[that row] = source row.
+__global__ __launch_bounds__(256) void packed_sequence_index_kernel(
+    const int64_t* __restrict__ offsets, const int64_t* __restrict__ rank,
+    const int64_t* __restrict__ step_starts, int64_t B, int64_t T, int64_t* __restrict__ index_out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= T) return;
+  const int64_t b = find_segment(offsets, B, i);
+  const int64_t t = i - offsets[b];
+  index_out[step_starts[t] + rank[b]] = i;
+}
+
+// out[offsets[b] + j] = j
+__global__ __launch_bounds__(256) void ragged_arange_kernel(const int64_t* __restrict__ offsets,
+                                                            int64_t* __restrict__ out) {
+  const int64_t b = blockIdx.x;
+  const int64_t begin = offsets[b];
+  const int64_t len = offsets[b + 1] - begin;
+  const int64_t stride = (int64_t)gridDim.y * blockDim.x;
+  for (int64_t j = (int64_t)blockIdx.y * blockDim.x + threadIdx.x; j < len; j += stride) {
+    out[begin + j] = j;
+  }
+}
+
+enum { kBagSum = 0, kBagMean = 1, kBagMax = 2 };
+
+// out[b, c] = reduce over the bag's tokens t of weight[indices[t], c], tokens in
+// order (a thread owns a column, so sums are formed in token order like a
+// sequential host loop).  Empty bags give 0 in every mode.
+template <typename T>
+__global__ __launch_bounds__(64) void embedding_bag_kernel(
+    const T* __restrict__ weight, int64_t ldw, int64_t num_embeddings,
+    const int64_t* __restrict__ indices, const int64_t* __restrict__ offsets, T* __restrict__ out,
+    int64_t n, int mode, int32_t* __restrict__ oob) {
+  constexpr int kAhead = 8;   // rows in flight per lane
+  const int64_t b = blockIdx.x;
+  const int64_t c = (int64_t)blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= n) return;
+  const int64_t begin = offsets[b], end = offsets[b + 1];
+  float acc = 0.0f;
+  bool first = true;
+  for (int64_t t0 = begin; t0 < end; t0 += kAhead) {
+    float v[kAhead];
+    bool use[kAhead];
+#pragma unroll
+    for (int j = 0; j < kAhead; ++j) {
+      const int64_t t = t0 + j;
+      const int64_t row = t < end ? indices[t] : 0;
+      const bool ok = row >= 0 && row < num_embeddings;
+      if (t < end && !ok && c == 0 && oob) atomicAdd(oob, 1);
+      use[j] = t < end && ok;
+      v[j] = (float)weight[(use[j] ? row : 0) * ldw + c];
+    }
+#pragma unroll
+    for (int j = 0; j < kAhead; ++j) {
+      if (use[j]) {
+        if (mode == kBagMax) {
+          acc = first ? v[j] : (v[j] > acc ? v[j] : acc);
+        } else {
+          acc += v[j];
+        }
+        first = false;
+      }
+    }
+  }
+  if (mode == kBagMean && end > begin) acc = acc / (float)(end - begin);
+  out[b * n + c] = (T)acc;
+}
+
+static int pick_unit3(const void* a, const void* b, int64_t row_bytes) {
+  const uintptr_t x = (uintptr_t)a | (uintptr_t)b | (uintptr_t)row_bytes;
+  if ((x & 15) == 0) return 16;
+  if ((x & 7) == 0) return 8;
+  if ((x & 3) == 0) return 4;
+  if ((x & 1) == 0) return 2;
+  return 1;
+}
+
+template <int UNIT>
+static void launch_gather(const void* src, int64_t src_rows, int64_t row_bytes, const int64_t* index,
+                          void* dst, int64_t n_rows, int32_t* oob, hipStream_t stream) {
+  const int64_t total = n_rows * (row_bytes / UNIT);
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > (1 << 22)) blocks = 1 << 22;   // grid-stride beyond that
+  hipLaunchKernelGGL((gather_rows_kernel<UNIT>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                     static_cast<const char*>(src), src_rows, row_bytes, index,
+                     static_cast<char*>(dst), n_rows, oob);
+}
+
+}  // namespace nt
+
+using namespace nt;
+
+extern "C" int nt_gather_rows(const void* src, int64_t src_rows, int64_t row_bytes,
+                              const int64_t* index, void* dst, int64_t n_rows, int32_t* oob_count,
+                              void* stream) {
+  if (src_rows < 0 || row_bytes < 0 || n_rows < 0) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "gather_rows: negative extent");
+  }
+  if (n_rows == 0 || row_bytes == 0) return NT_OK;
+  if (!src || !index || !dst) return fail(NT_ERR_INVALID_ARGUMENT, "gather_rows: NULL pointer");
+  hipStream_t s = (hipStream_t)stream;
+  switch (pick_unit3(src, dst, row_bytes)) {
+    case 16: launch_gather<16>(src, src_rows, row_bytes, index, dst, n_rows, oob_count, s); break;
+    case 8: launch_gather<8>(src, src_rows, row_bytes, index, dst, n_rows, oob_count, s); break;
+    case 4: launch_gather<4>(src, src_rows, row_bytes, index, dst, n_rows, oob_count, s); break;
+    case 2: launch_gather<2>(src, src_rows, row_bytes, index, dst, n_rows, oob_count, s); break;
+    default: launch_gather<1>(src, src_rows, row_bytes, index, dst, n_rows, oob_count, s); break;
+  }
+  return check_launch("gather_rows_kernel");
+}
+
+extern "C" int nt_packed_sequence_index(const int64_t* offsets, const int64_t* rank,
+                                        const int64_t* step_starts, int64_t B, int64_t total_rows,
+                                        int64_t* index_out, void* stream) {
+  if (B < 0 || total_rows < 0) return fail(NT_ERR_INVALID_ARGUMENT, "packed_sequence_index: negative extent");
+  if (total_rows == 0) return NT_OK;
+  if (B == 0 || !offsets || !rank || !step_starts || !index_out) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "packed_sequence_index: NULL pointer or no sequences");
+  }
+  const int64_t blocks = (total_rows + 255) / 256;
+  if (blocks > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "packed_sequence_index: too many rows");
+  hipLaunchKernelGGL(packed_sequence_index_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                     (hipStream_t)stream, offsets, rank, step_starts, B, total_rows, index_out);
+  return check_launch("packed_sequence_index_kernel");
+}
+
+extern "C" int nt_ragged_arange(const int64_t* offsets, int64_t B, int64_t max_len, int64_t* out,
+                                void* stream) {
+  if (B < 0 || max_len < 0) return fail(NT_ERR_INVALID_ARGUMENT, "ragged_arange: negative extent");
+  if (B == 0 || max_len == 0) return NT_OK;
+  if (!offsets || !out) return fail(NT_ERR_INVALID_ARGUMENT, "ragged_arange: NULL pointer");
+  if (B > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "ragged_arange: too many rows");
+  int64_t tiles = (max_len + 1023) / 1024;   // a block covers >= 4 elements per thread before looping
+  if (tiles > 65535) tiles = 65535;
+  hipLaunchKernelGGL(ragged_arange_kernel, dim3((unsigned)B, (unsigned)tiles), dim3(256), 0,
+                     (hipStream_t)stream, offsets, out);
+  return check_launch("ragged_arange_kernel");
+}
+
+extern "C" int nt_embedding_bag(const void* weight, int64_t ldw, int64_t num_embeddings,
+                                const int64_t* indices, const int64_t* offsets, void* out, int64_t B,
+                                int64_t n, int mode, int dtype, int32_t* oob_count, void* stream) {
+  if (B < 0 || n < 0 || num_embeddings < 0 || ldw < n) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "embedding_bag: bad shape");
+  }
+  if (mode < 0 || mode > 2) return fail(NT_ERR_INVALID_ARGUMENT, "embedding_bag: mode %d", mode);
+  if (B == 0 || n == 0) return NT_OK;
+  if (!weight || !offsets || !out) return fail(NT_ERR_INVALID_ARGUMENT, "embedding_bag: NULL pointer");
+  if (num_embeddings == 0) return fail(NT_ERR_INVALID_ARGUMENT, "embedding_bag: empty table");
+  if (B > 0x7fffffffLL || (n + 63) / 64 > 65535) {
+    return fail(NT_ERR_UNSUPPORTED, "embedding_bag: too many bags or columns");
+  }
+  dim3 grid((unsigned)B, (unsigned)((n + 63) / 64));
+  hipStream_t s = (hipStream_t)stream;
+#define NT_BAG_CASE(TYPE)                                                                       \
+  hipLaunchKernelGGL((embedding_bag_kernel<TYPE>), grid, dim3(64), 0, s,                        \
+                     static_cast<const TYPE*>(weight), ldw, num_embeddings, indices, offsets,   \
+                     static_cast<TYPE*>(out), n, mode, oob_count);                              \
+  break;
+  switch (dtype) {
+    case NT_F32: NT_BAG_CASE(float)
+    case NT_F16: NT_BAG_CASE(_Float16)
+    case NT_BF16: NT_BAG_CASE(__bf16)
+    default: return fail(NT_ERR_UNSUPPORTED, "embedding_bag: dtype %d is not f32, f16 or bf16", dtype);
+  }
+#undef NT_BAG_CASE
+  return check_launch("embedding_bag_kernel");
+}

@@ -250,7 +250,10 @@ class NestedTensor:
     def to_packed_sequence(self):
         if not self.dim() == 3 and self.nested_dim() == 1:
             raise RuntimeError("NestedTensor should consistent of 2d Tensors of size L x *")
-        return torch.nn.utils.rnn.pack_sequence(self.to_tensor_list(), enforce_sorted=False)
+        return ops.to_packed_sequence(self._impl)
+
+    def to_sparse_csr_tensor(self):
+        return ops.to_sparse_csr(self._impl)
 
     # --- packed element-wise add (BinaryOps.cpp:12-115) ---
     def __add__(self, other):
@@ -329,6 +332,9 @@ _HANDLERS = {
     _ns.make_contiguous: lambda impl: impl,
     _ns.to_tensor_list: lambda impl: list(NestedTensor(impl).unbind()),
     torch.nn.functional.layer_norm: _nn_functional_layer_norm,
+    torch.nn.functional.embedding: lambda input, weight, *a, **k: ops.embedding(weight, input, *a, **k),
+    torch.embedding: lambda weight, indices, *a, **k: ops.embedding(weight, indices),
+    torch.nn.functional.embedding_bag: ops.embedding_bag,
     torch.conv2d: ops.conv2d,
     torch.nn.functional.max_pool2d: ops.max_pool2d,
     torch.max_pool2d: ops.max_pool2d,

@@ -556,3 +556,156 @@ def conv2d(impl, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
     k = (weight.size(2), weight.size(3))
     return _dense_via_padding(
         impl, 0.0, lambda x: torch.conv2d(x, weight, bias, s, p, d, groups), weight.size(0), k, s, p, d)
+
+
+# ---- consumers of the offsets array: interop formats ----------------------------
+
+def _raise_if_oob(oob, what):
+    n = int(oob.item())
+    if n:
+        raise IndexError("%s: %d index value(s) out of range" % (what, n))
+
+
+def embedding(weight, indices, padding_idx=None, max_norm=None, norm_type=2.0,
+              scale_grad_by_freq=False, sparse=False):
+    """NestedTensor_embedding (functions.cpp:14-63): one gather over the packed
+    index buffer (nt_gather_rows); the result gets a trailing regular dim of
+    weight.size(1).  padding_idx, scale_grad_by_freq and sparse only shape
+    gradients and are accepted for the call signature; max_norm would modify the
+    table and is refused."""
+    if max_norm is not None:
+        raise NotImplementedError("embedding on a NestedTensor: max_norm is not supported.")
+    if not isinstance(indices, NestedTensorImpl) or isinstance(weight, NestedTensorImpl):
+        raise NotImplementedError("embedding: expected a dense weight and NestedTensor indices.")
+    if weight.dim() != 2:
+        raise RuntimeError("'weight' must be 2-D")
+    idx = indices.buffer
+    _C.require_device(idx, "embedding")
+    if idx.dtype not in (torch.int64, torch.int32):
+        raise RuntimeError("Expected tensor for argument #1 'indices' to have one of the following scalar "
+                           "types: Long, Int; but got %s instead" % idx.dtype)
+    if weight.device != idx.device:
+        raise RuntimeError("embedding: weight and indices must be on the same device")
+    weight = weight.contiguous()
+    idx64 = idx.to(torch.int64)
+    V, E = weight.shape
+    out = torch.empty(idx.numel() * E, dtype=weight.dtype, device=weight.device)
+    oob = torch.zeros(1, dtype=torch.int32, device=weight.device)
+    with torch.cuda.device(weight.device):
+        _C.check(_C.lib.nt_gather_rows(_C.ptr(weight), V, E * weight.element_size(), _C.ptr(idx64),
+                                       _C.ptr(out), idx.numel(), _C.ptr(oob),
+                                       _C.current_stream(weight.device)))
+    _raise_if_oob(oob, "embedding")
+    if indices.sizes.dim() == 0:
+        sizes = indices.sizes
+    else:
+        sizes = torch.cat([indices.sizes, torch.full((indices.B, 1), E, dtype=torch.int64)], 1)
+    return NestedTensorImpl(out, sizes)
+
+
+def embedding_bag(input, weight, offsets=None, max_norm=None, norm_type=2, scale_grad_by_freq=False,
+                  mode="mean", sparse=False, per_sample_weights=None, include_last_offset=False,
+                  padding_idx=None):
+    """_nn_functional_embedding_bag (nested/nested.py:43-118): the bags are the
+    constituents of a nested tensor of 1-D index tensors; its device offsets array
+    is the offsets argument the reference rebuilds in a host loop.  Returns a
+    dense [B, E] tensor."""
+    if max_norm is not None:
+        raise NotImplementedError("NestedTensor embedding_bag: max_norm is not supported")
+    if per_sample_weights is not None:
+        raise NotImplementedError("NestedTensor embedding_bag: per_sample_weights is not supported")
+    if not isinstance(input, NestedTensorImpl):
+        raise NotImplementedError("embedding_bag: expected NestedTensor indices.")
+    if input.dim() == 2:
+        if offsets is not None:
+            raise ValueError("if input is 2D, then offsets has to be None, as input is treated is a "
+                             "mini-batch of fixed length sequences. However, found offsets of type %s"
+                             % type(offsets))
+    else:
+        raise ValueError("input has to be 2D NestedTensor, but got NestedTensor of dimension %d"
+                         % input.dim())
+    modes = {"sum": 0, "mean": 1, "max": 2}
+    if mode not in modes:
+        raise ValueError("mode has to be one of sum, mean or max")
+    if mode == "max" and scale_grad_by_freq:
+        raise ValueError("max mode does not support scaling the gradient by the frequency")
+    if mode == "max" and sparse:
+        raise ValueError("max mode does not support sparse weights")
+    if padding_idx is not None:
+        raise NotImplementedError("padding_idx is not supported for NestedTensor embedding_bag")
+    idx = input.buffer
+    _C.require_device(idx, "embedding_bag")
+    if weight.dim() != 2 or weight.device != idx.device:
+        raise RuntimeError("embedding_bag: weight must be 2-D on the device of the indices")
+    weight = weight.contiguous()
+    idx64 = idx.to(torch.int64)
+    V, E = weight.shape
+    B = input.B
+    out = torch.empty((B, E), dtype=weight.dtype, device=weight.device)
+    oob = torch.zeros(1, dtype=torch.int32, device=weight.device)
+    with torch.cuda.device(weight.device):
+        _C.check(_C.lib.nt_embedding_bag(_C.ptr(weight), E, V, _C.ptr(idx64), _C.ptr(input.offsets_dev()),
+                                         _C.ptr(out), B, E, modes[mode], _C.dtype_code(weight.dtype),
+                                         _C.ptr(oob), _C.current_stream(weight.device)))
+    _raise_if_oob(oob, "embedding_bag")
+    return out
+
+
+def to_sparse_csr(impl):
+    """NestedTensor_to_sparse_csr (nested_tensor_impl.h:326-349): crow_indices are
+    the offsets array, col_indices one arange per constituent (nt_ragged_arange),
+    values the packed buffer."""
+    if impl.dim() != 2:
+        raise RuntimeError("Given tensor must be of dimension 2, got dimension %d" % impl.dim())
+    buf = impl.buffer
+    _C.require_device(buf, "to_sparse_csr")
+    crow = impl.offsets_dev()
+    col = torch.empty(buf.numel(), dtype=torch.int64, device=buf.device)
+    mx = impl.max_sizes()
+    with torch.cuda.device(buf.device):
+        _C.check(_C.lib.nt_ragged_arange(_C.ptr(crow), impl.B, mx[0] if mx else 0, _C.ptr(col),
+                                         _C.current_stream(buf.device)))
+    return torch.sparse_csr_tensor(crow, col, buf, size=(impl.B, mx[0] if mx else 0))
+
+
+def to_packed_sequence(impl):
+    """NestedTensor.to_packed_sequence (nested/nested.py:484-488) without the
+    unbind: the time-major row order of torch.nn.utils.rnn.pack_sequence(...,
+    enforce_sorted=False) is built on the device (nt_packed_sequence_index) and
+    the token rows are moved by one gather (nt_gather_rows)."""
+    if impl.dim() < 3:
+        raise RuntimeError("NestedTensor should consistent of 2d Tensors of size L x *")
+    buf = impl.buffer
+    _C.require_device(buf, "to_packed_sequence")
+    opt = impl.opt_sizes()
+    if any(v is None for v in opt[2:]):
+        raise RuntimeError("to_packed_sequence: the trailing dims of the constituents must be regular")
+    if impl.has_empty_constituent():
+        raise RuntimeError("Length of all samples has to be greater than 0, but found an element in "
+                           "'lengths' that is <= 0")
+    lengths = impl.sizes[:, 0].contiguous()
+    # as torch.nn.utils.rnn.pack_padded_sequence(enforce_sorted=False) orders them
+    sorted_lengths, sorted_indices = torch.sort(lengths, descending=True)
+    B, Lmax = impl.B, int(sorted_lengths[0])
+    unsorted_indices = torch.empty_like(sorted_indices)
+    unsorted_indices[sorted_indices] = torch.arange(B)
+    # batch_sizes[t] = number of sequences longer than t
+    batch_sizes = (lengths.unsqueeze(0) > torch.arange(Lmax).unsqueeze(1)).sum(1)
+    step_starts = torch.cumsum(batch_sizes, 0) - batch_sizes
+    dev = buf.device
+    trailing = [int(v) for v in opt[2:]]
+    row_elems = 1
+    for v in trailing:
+        row_elems *= v
+    T = int(lengths.sum())
+    index = torch.empty(T, dtype=torch.int64, device=dev)
+    data = torch.empty([T] + trailing, dtype=buf.dtype, device=dev)
+    rank_dev, starts_dev = unsorted_indices.to(dev), step_starts.to(dev)
+    with torch.cuda.device(dev):
+        stream = _C.current_stream(dev)
+        _C.check(_C.lib.nt_packed_sequence_index(_C.ptr(impl.row_offsets_dev()), _C.ptr(rank_dev),
+                                                 _C.ptr(starts_dev), B, T, _C.ptr(index), stream))
+        _C.check(_C.lib.nt_gather_rows(_C.ptr(buf), T, row_elems * buf.element_size(), _C.ptr(index),
+                                       _C.ptr(data), T, None, stream))
+    return torch.nn.utils.rnn.PackedSequence(data, batch_sizes, sorted_indices.to(dev),
+                                             unsorted_indices.to(dev))

@@ -44,6 +44,10 @@ Pinning (what each part was checked against, see tests/test_oracle_*.py):
   (test/test_nested_tensor_functional.py:44-135, 251-266); the output sizes are
   cross-checked against the closed form of pooling.cpp:50-53 / conv2d.cpp:80-84
   in tests/test_oracle_rowops.py.
+* embedding / embedding_bag / to_sparse_csr / to_packed_sequence: closed forms
+  that avoid the library call being restated (indexing, Python loops, the CSR
+  ``to_dense`` check of test/test_nested_tensor_class.py:741-752, the
+  ``pad_packed_sequence`` round trip); tests/test_oracle_interop.py.
 * add: ``torch.add`` on the packed buffers / per constituent
   (test/test_nested_tensor_functional.py's add cases reduce to it).
 
@@ -71,3 +75,4 @@ from .masking import (  # noqa: F401
 from .mha import min_mha, bt_min_mha  # noqa: F401
 from .rowops import layer_norm, add  # noqa: F401
 from .dense import max_pool2d, conv2d  # noqa: F401
+from .interop import embedding, embedding_bag, to_sparse_csr, to_packed_sequence  # noqa: F401

@@ -1,0 +1,53 @@
+"""Oracle for the interop formats built from the offsets array.
+TEST INFRASTRUCTURE ONLY (see oracle/__init__.py).
+
+Follows nestedtensor/csrc/functions.cpp:14-63 (embedding: at::embedding over the
+packed index buffer, result gains a trailing regular dim),
+nestedtensor/nested/nested.py:43-118 (embedding_bag: offsets from a host loop over
+nested_size, then torch.embedding_bag), nestedtensor/csrc/nested_tensor_impl.h:326-349
+(to_sparse_csr: crow = [0, cumsum(lengths)], col = cat of aranges, values = buffer)
+and nestedtensor/nested/nested.py:484-488 (to_packed_sequence: pack_sequence of the
+constituents, enforce_sorted=False).
+
+Pinned in tests/test_oracle_interop.py by closed forms that do not go through the
+same library calls: ``weight[idx]`` indexing, explicit Python loops for the bag
+reductions, ``csr.to_dense() == to_padded_tensor(0)`` (the reference's own check,
+test/test_nested_tensor_class.py:741-752) and the
+``pad_packed_sequence(to_packed_sequence(nt)) == to_padded_tensor(0)`` round trip.
+"""
+
+import torch
+
+from .nt import RefNestedTensor
+
+
+def embedding(weight, indices):
+    outs = [torch.embedding(weight, t) for t in indices.unbind()]
+    return RefNestedTensor(outs, weight.dtype)
+
+
+def embedding_bag(indices, weight, mode="mean"):
+    if indices.dim() != 2:
+        raise ValueError("input has to be 2D NestedTensor, but got NestedTensor of dimension %d" % indices.dim())
+    sizes = [int(s[0]) for s in indices._shapes]
+    offsets = torch.zeros(len(sizes), dtype=torch.int64)       # nested.py:76-79
+    for i in range(1, len(sizes)):
+        offsets[i] = offsets[i - 1] + sizes[i - 1]
+    mode_enum = {"sum": 0, "mean": 1, "max": 2}[mode]
+    ret, _, _, _ = torch.embedding_bag(weight, indices.buffer, offsets, False, mode_enum, False, None, False)
+    return ret
+
+
+def to_sparse_csr(nt):
+    if nt.dim() != 2:
+        raise RuntimeError("Given tensor must be of dimension 2, got dimension %d" % nt.dim())
+    lengths = nt.sizes.reshape(-1)
+    crow = torch.cat([torch.tensor([0]), torch.cumsum(lengths, 0)])
+    col = torch.cat([torch.arange(int(v)) for v in lengths]) if len(lengths) else torch.zeros(0, dtype=torch.int64)
+    return torch.sparse_csr_tensor(crow, col, nt.buffer)
+
+
+def to_packed_sequence(nt):
+    if not nt.dim() == 3:
+        raise RuntimeError("NestedTensor should consistent of 2d Tensors of size L x *")
+    return torch.nn.utils.rnn.pack_sequence(nt.unbind(), enforce_sorted=False)

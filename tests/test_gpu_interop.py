@@ -1,0 +1,109 @@
+"""Parity of the interop formats (embedding, embedding_bag, CSR, PackedSequence)
+built on the device from the offsets array, against the oracle.  Copies and
+integer work are bit-exact; bag sums are fp32 in token order (1e-5 relative)."""
+
+import pytest
+import torch
+
+import nestedtensor_amd as nt
+import oracle
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda", 0)
+
+
+def _idx(lens, V, seed):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(V, (L,), generator=g) for L in lens]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("E", [8, 768, 7])
+def test_embedding(E, dtype):
+    V = 1000
+    ids = _idx([5, 1, 131, 64], V, 1)
+    w = torch.randn(V, E, generator=torch.Generator().manual_seed(2)).to(dtype)
+    a = nt.nested_tensor(ids, device=DEV, dtype=torch.int64)
+    emb = torch.nn.Embedding(V, E).to(dtype)
+    with torch.no_grad():
+        emb.weight.copy_(w)
+    got = emb.to(DEV)(a)
+    exp = oracle.embedding(w, oracle.ref_nested_tensor(ids, dtype=torch.int64))
+    assert got.nested_size() == nt.nested_tensor(list(exp.unbind())).nested_size()
+    assert torch.equal(got._impl.buffer.cpu(), exp.buffer)
+    got2 = torch.nn.functional.embedding(a, w.to(DEV))
+    assert torch.equal(got2._impl.buffer.cpu(), exp.buffer)
+
+
+def test_embedding_out_of_range_raises():
+    a = nt.nested_tensor([torch.tensor([1, 2, 50]), torch.tensor([3])], device=DEV, dtype=torch.int64)
+    with pytest.raises(IndexError):
+        torch.nn.functional.embedding(a, torch.randn(10, 4, device=DEV))
+
+
+@pytest.mark.parametrize("mode", ["sum", "mean", "max"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_embedding_bag(mode, dtype):
+    V, E = 100, 8
+    for lens in ([5, 5], [5, 1, 12, 300], [3] * 70):       # first: the reference's case
+        ids = _idx(lens, V, 3)
+        w = torch.randn(V, E, generator=torch.Generator().manual_seed(4)).to(dtype)
+        a = nt.nested_tensor(ids, device=DEV, dtype=torch.int64)
+        bag = torch.nn.EmbeddingBag(V, E, mode=mode).to(dtype)
+        with torch.no_grad():
+            bag.weight.copy_(w)
+        got = bag.to(DEV)(a)
+        exp = oracle.embedding_bag(oracle.ref_nested_tensor(ids, dtype=torch.int64), w.float(), mode)
+        assert got.shape == (len(lens), E) and got.dtype == dtype
+        tol = 1e-5 if dtype == torch.float32 else 2e-2
+        assert (got.float().cpu() - exp).abs().max().item() <= tol * max(1.0, exp.abs().max().item())
+
+
+def test_embedding_bag_errors():
+    a = nt.nested_tensor([torch.tensor([[1, 2]]), torch.tensor([[3, 4]])], device=DEV, dtype=torch.int64)
+    with pytest.raises(ValueError, match="input has to be 2D NestedTensor"):
+        torch.nn.functional.embedding_bag(a, torch.randn(10, 4, device=DEV))
+    a = nt.nested_tensor([torch.tensor([1, 2]), torch.tensor([3])], device=DEV, dtype=torch.int64)
+    with pytest.raises(ValueError, match="if input is 2D, then offsets has to be None"):
+        torch.nn.functional.embedding_bag(a, torch.randn(10, 4, device=DEV), offsets=torch.tensor([0, 2]))
+    with pytest.raises(ValueError, match="mode has to be one of sum, mean or max"):
+        torch.nn.functional.embedding_bag(a, torch.randn(10, 4, device=DEV), mode="prod")
+
+
+def test_to_sparse_csr():
+    # test/test_nested_tensor_class.py:741-752
+    a, b, c = torch.arange(3) + 1, torch.arange(4) + 1, torch.arange(2) + 1
+    x = nt.nested_tensor([a, b, c], device=DEV, dtype=torch.int64)
+    st = x.to_sparse_csr_tensor()
+    assert torch.equal(st.to_dense(), x.to_padded_tensor(padding=0))
+    ref = oracle.to_sparse_csr(oracle.ref_nested_tensor([a, b, c], dtype=torch.int64))
+    assert torch.equal(st.crow_indices().cpu(), ref.crow_indices())
+    assert torch.equal(st.col_indices().cpu(), ref.col_indices())
+    assert torch.equal(st.values().cpu(), ref.values())
+    y = nt.nested_tensor([a.unsqueeze(1), b.unsqueeze(1)], device=DEV, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="Given tensor must be of dimension 2, got dimension 3"):
+        y.to_sparse_csr_tensor()
+    # long rows: more than one block per row
+    g = torch.Generator().manual_seed(5)
+    ts = [torch.randn(L, generator=g) for L in (5000, 1, 70000)]
+    z = nt.nested_tensor(ts, device=DEV)
+    ref = oracle.to_sparse_csr(oracle.ref_nested_tensor(ts))
+    st = z.to_sparse_csr_tensor()
+    assert torch.equal(st.col_indices().cpu(), ref.col_indices())
+    assert torch.equal(st.crow_indices().cpu(), ref.crow_indices())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_to_packed_sequence(dtype):
+    g = torch.Generator().manual_seed(6)
+    for lens, E in (((4, 7, 1, 7, 2), 3), ((33, 512, 32, 100, 512, 77), 768)):
+        ts = [torch.randn(L, E, generator=g).to(dtype) for L in lens]
+        a = nt.nested_tensor(ts, device=DEV, dtype=dtype)
+        ps = a.to_packed_sequence()
+        ref = oracle.to_packed_sequence(oracle.ref_nested_tensor(ts, dtype=dtype))
+        assert torch.equal(ps.data.cpu(), ref.data)
+        assert torch.equal(ps.batch_sizes, ref.batch_sizes)
+        assert torch.equal(ps.sorted_indices.cpu(), ref.sorted_indices)
+        assert torch.equal(ps.unsorted_indices.cpu(), ref.unsorted_indices)
+        padded, lengths = torch.nn.utils.rnn.pad_packed_sequence(ps, batch_first=True)
+        assert torch.equal(padded, a.to_padded_tensor(0))

@@ -1,0 +1,59 @@
+"""Pins the interop oracle functions (CPU only)."""
+import pytest
+import torch
+
+import oracle
+
+
+def _idx_nt(lens, V, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return oracle.ref_nested_tensor([torch.randint(V, (L,), generator=g) for L in lens], dtype=torch.int64)
+
+
+def test_embedding_is_row_indexing():
+    w = torch.randn(50, 6, generator=torch.Generator().manual_seed(1))
+    nt = _idx_nt([5, 1, 9], 50)
+    got = oracle.embedding(w, nt)
+    for o, i in zip(got.unbind(), nt.unbind()):
+        assert torch.equal(o, w[i])
+    assert got.opt_sizes() == [3, None, 6]
+
+
+@pytest.mark.parametrize("mode", ["sum", "mean", "max"])
+def test_embedding_bag_against_loops(mode):
+    w = torch.randn(100, 8, generator=torch.Generator().manual_seed(2))
+    nt = _idx_nt([5, 5, 1, 12], 100, seed=3)            # reference case: two bags of 5 (functional.py:189-190)
+    got = oracle.embedding_bag(nt, w, mode)
+    for b, idx in enumerate(nt.unbind()):
+        rows = [w[int(i)] for i in idx]
+        if mode == "max":
+            exp = torch.stack(rows).max(0).values
+        else:
+            exp = rows[0].clone()
+            for r in rows[1:]:
+                exp = exp + r
+            if mode == "mean":
+                exp = exp / len(rows)
+        assert (got[b] - exp).abs().max() <= 1e-6 * max(1.0, exp.abs().max().item())
+
+
+def test_to_sparse_csr_to_dense_is_padded():
+    # test/test_nested_tensor_class.py:741-752
+    a, b, c = torch.arange(3) + 1, torch.arange(4) + 1, torch.arange(2) + 1
+    nt = oracle.ref_nested_tensor([a, b, c], dtype=torch.int64)
+    st = oracle.to_sparse_csr(nt)
+    assert torch.equal(st.to_dense(), oracle.to_padded_tensor(nt, 0))
+    nt = oracle.ref_nested_tensor([a.unsqueeze(1), b.unsqueeze(1)], dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="Given tensor must be of dimension 2, got dimension 3"):
+        oracle.to_sparse_csr(nt)
+
+
+def test_to_packed_sequence_round_trip():
+    g = torch.Generator().manual_seed(4)
+    ts = [torch.randn(L, 3, generator=g) for L in (4, 7, 1, 7, 2)]
+    nt = oracle.ref_nested_tensor(ts)
+    ps = oracle.to_packed_sequence(nt)
+    padded, lengths = torch.nn.utils.rnn.pad_packed_sequence(ps, batch_first=True)
+    assert torch.equal(padded, oracle.to_padded_tensor(nt, 0))
+    assert lengths.tolist() == [4, 7, 1, 7, 2]
+    assert ps.batch_sizes.tolist() == [5, 4, 3, 3, 2, 2, 2]
