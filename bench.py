@@ -456,6 +456,21 @@ def bench_rows(args, torch, dev):
                                            note="2 GiB written; the 62 MB table is re-read from cache")
     del big_idx, big_tab, big_out
 
+    # ---- channels-last ragged images: per-constituent transpose -----------------------
+    g = torch.Generator().manual_seed(1010 + 1)
+    hw_t = torch.randint(480, 1025, (16, 2), generator=g)
+    sizes_t = torch.tensor([[64, int(h), int(w)] for h, w in hw_t], dtype=torch.int64)
+    buf_t = torch.randn(int(sizes_t.prod(1).sum()), device=dev, dtype=torch.float16)
+    from nestedtensor_amd.impl import NestedTensorImpl as _Impl
+    img = _Impl(buf_t, sizes_t)
+    nhwc = _ops.transpose_nchw_nhwc(img)
+    ms_t0 = _time_gpu(torch, lambda: _ops.transpose_nchw_nhwc(img))
+    ms_t1 = _time_gpu(torch, lambda: _ops.transpose_nhwc_nchw(nhwc))
+    assert torch.equal(_ops.transpose_nhwc_nchw(nhwc).buffer, buf_t)
+    rows["C2x64ch_transpose_nchw_nhwc_fp16"] = entry(ms_t0, 2 * 2 * buf_t.numel())
+    rows["C2x64ch_transpose_nhwc_nchw_fp16"] = entry(ms_t1, 2 * 2 * buf_t.numel())
+    del buf_t, img, nhwc
+
     # ---- C4: bt_min_mha bf16, high raggedness ---------------------------------
     g = torch.Generator().manual_seed(1010 + 3)
     raw = torch.empty(128).exponential_(1.0 / 96.0, generator=g)

@@ -255,6 +255,19 @@ int nt_embedding_bag(const void* weight, int64_t ldw, int64_t num_embeddings, co
                      const int64_t* offsets, void* out, int64_t B, int64_t n, int mode, int dtype,
                      int32_t* oob_count, void* stream);
 
+/* Per-constituent 2-D transpose on the packed buffer: constituent b, a row-major
+ * [rows[b], cols[b]] matrix at element offset offsets[b], is written as its
+ * [cols[b], rows[b]] transpose at the same offset of out.  rows = C, cols =
+ * H_b * W_b is the reference's transpose_nchw_nhwc, the two exchanged its
+ * transpose_nhwc_nchw (nestedtensor/csrc/transpose.cpp:87-204 with the
+ * launchers of nestedtensor/csrc/cuda/transpose.h:11-31).  tile_offsets
+ * int64[B + 1]: tile_offsets[b] = sum over c < b of ceil(rows[c] / 64) *
+ * ceil(cols[c] / 64) (nt_offsets_from_sizes over a [B, 2] array of the two tile
+ * counts builds it); total_tiles = tile_offsets[B].  All arrays on the device. */
+int nt_transpose_ragged(const void* in, void* out, const int64_t* offsets, const int64_t* rows,
+                        const int64_t* cols, const int64_t* tile_offsets, int64_t B,
+                        int64_t total_tiles, int elem_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

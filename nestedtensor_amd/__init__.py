@@ -17,6 +17,8 @@ from .nested.masking import nested_tensor_from_padded_tensor
 from .nested.masking import from_padded_tensor
 
 from .nested.nested import NestedTensor
+from .nested.nested import transpose_nchw_nhwc
+from .nested.nested import transpose_nhwc_nchw
 
 from . import nested
 from . import nn

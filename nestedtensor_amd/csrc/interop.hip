@@ -227,3 +227,106 @@ extern "C" int nt_embedding_bag(const void* weight, int64_t ldw, int64_t num_emb
 #undef NT_BAG_CASE
   return check_launch("embedding_bag_kernel");
 }
+
+// ---------------------------------------------------------------------------
+// Per-constituent 2-D transpose on the packed buffer: constituent b is a
+// row-major [rows[b], cols[b]] matrix at element offset offsets[b]; the result
+// holds its [cols[b], rows[b]] transpose at the same offset.  With rows = C and
+// cols = H_b * W_b this is NCHW -> NHWC of a batch of ragged images, and the
+// other way round with the two exchanged (the reference's
+// transpose_nchw_nhwc / transpose_nhwc_nchw, nestedtensor/csrc/transpose.cpp:87-204,
+// kernels nestedtensor/csrc/cuda/transpose.cu).  One workgroup per 64 x 64 tile,
+// through LDS, so that both the reads and the writes are contiguous per
+// wavefront; tile_offsets[b] = number of tiles of all constituents before b, and
+// a workgroup finds its constituent by binary search.
+namespace nt {
+
+constexpr int kTrTile = 64;
+
+template <typename U>
+__global__ __launch_bounds__(256) void transpose_ragged_kernel(
+    const U* __restrict__ in, U* __restrict__ out, const int64_t* __restrict__ offsets,
+    const int64_t* __restrict__ rows, const int64_t* __restrict__ cols,
+    const int64_t* __restrict__ tile_offsets, int64_t B) {
+  // a lane moves V consecutive elements (8 bytes) per access on both sides
+  constexpr int V = 8 / (int)sizeof(U);
+  constexpr int kLanesPerRow = kTrTile / V;
+  constexpr int kRowsPerPass = 256 / kLanesPerRow;
+  constexpr int kStride = kTrTile + V;      // keeps every row of the tile 8-byte aligned
+  __shared__ __align__(8) U tile[kTrTile][kStride];
+  const int64_t id = blockIdx.x;
+  const int64_t b = find_segment(tile_offsets, B, id);
+  const int64_t R = rows[b], C = cols[b];
+  const int64_t tiles_c = (C + kTrTile - 1) / kTrTile;
+  const int64_t local = id - tile_offsets[b];
+  const int64_t r0 = (local / tiles_c) * kTrTile;
+  const int64_t c0 = (local % tiles_c) * kTrTile;
+  const U* src = in + offsets[b];
+  U* dst = out + offsets[b];
+  const int lv = (threadIdx.x % kLanesPerRow) * V;   // first of this lane's V elements
+  const int lr = threadIdx.x / kLanesPerRow;
+  for (int r = lr; r < kTrTile; r += kRowsPerPass) {
+    if (r0 + r < R) {
+      const U* p = src + (r0 + r) * C + c0 + lv;
+      if (c0 + lv + V <= C) {
+        uint64_t bits;
+        __builtin_memcpy(&bits, p, 8);                // any alignment
+        *reinterpret_cast<uint64_t*>(&tile[r][lv]) = bits;
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+          if (c0 + lv + j < C) tile[r][lv + j] = p[j];
+      }
+    }
+  }
+  __syncthreads();
+  for (int c = lr; c < kTrTile; c += kRowsPerPass) {
+    if (c0 + c < C) {
+      U v[V];
+#pragma unroll
+      for (int j = 0; j < V; ++j) v[j] = tile[lv + j][c];
+      U* q = dst + (c0 + c) * R + r0 + lv;
+      if (r0 + lv + V <= R) {
+        uint64_t bits;
+        __builtin_memcpy(&bits, v, 8);
+        __builtin_memcpy(q, &bits, 8);
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+          if (r0 + lv + j < R) q[j] = v[j];
+      }
+    }
+  }
+}
+
+template <typename U>
+static void launch_transpose(const void* in, void* out, const int64_t* offsets, const int64_t* rows,
+                             const int64_t* cols, const int64_t* tile_offsets, int64_t B,
+                             int64_t total_tiles, hipStream_t stream) {
+  hipLaunchKernelGGL((transpose_ragged_kernel<U>), dim3((unsigned)total_tiles), dim3(256), 0, stream,
+                     static_cast<const U*>(in), static_cast<U*>(out), offsets, rows, cols,
+                     tile_offsets, B);
+}
+
+}  // namespace nt
+
+extern "C" int nt_transpose_ragged(const void* in, void* out, const int64_t* offsets,
+                                   const int64_t* rows, const int64_t* cols,
+                                   const int64_t* tile_offsets, int64_t B, int64_t total_tiles,
+                                   int elem_bytes, void* stream) {
+  if (B < 0 || total_tiles < 0) return nt::fail(NT_ERR_INVALID_ARGUMENT, "transpose_ragged: negative extent");
+  if (B == 0 || total_tiles == 0) return NT_OK;
+  if (!in || !out || !offsets || !rows || !cols || !tile_offsets) {
+    return nt::fail(NT_ERR_INVALID_ARGUMENT, "transpose_ragged: NULL pointer");
+  }
+  if (total_tiles > 0x7fffffffLL) return nt::fail(NT_ERR_UNSUPPORTED, "transpose_ragged: too many tiles");
+  hipStream_t s = (hipStream_t)stream;
+  switch (elem_bytes) {
+    case 1: nt::launch_transpose<uint8_t>(in, out, offsets, rows, cols, tile_offsets, B, total_tiles, s); break;
+    case 2: nt::launch_transpose<uint16_t>(in, out, offsets, rows, cols, tile_offsets, B, total_tiles, s); break;
+    case 4: nt::launch_transpose<uint32_t>(in, out, offsets, rows, cols, tile_offsets, B, total_tiles, s); break;
+    case 8: nt::launch_transpose<uint64_t>(in, out, offsets, rows, cols, tile_offsets, B, total_tiles, s); break;
+    default: return nt::fail(NT_ERR_UNSUPPORTED, "transpose_ragged: element size %d", elem_bytes);
+  }
+  return nt::check_launch("transpose_ragged_kernel");
+}

@@ -253,7 +253,7 @@ class NestedTensor:
         return ops.to_packed_sequence(self._impl)
 
     def to_sparse_csr_tensor(self):
-        return ops.to_sparse_csr(self._impl)
+        return torch.ops.nestedtensor.to_sparse_csr(self)
 
     # --- packed element-wise add (BinaryOps.cpp:12-115) ---
     def __add__(self, other):
@@ -296,6 +296,16 @@ def _nn_functional_linear(input, weight, bias=None):
     return NestedTensorImpl(out.reshape(-1), sizes)
 
 
+def transpose_nchw_nhwc(tensor):
+    """nested/nested.py:176-178."""
+    return torch.ops.nestedtensor.transpose_nchw_nhwc(tensor)
+
+
+def transpose_nhwc_nchw(tensor):
+    """nested/nested.py:181-183."""
+    return torch.ops.nestedtensor.transpose_nhwc_nchw(tensor)
+
+
 def _nn_functional_layer_norm(input, normalized_shape, weight=None, bias=None, eps=1e-5):
     return ops.layer_norm(input, normalized_shape, weight, bias, eps)
 
@@ -331,6 +341,9 @@ _HANDLERS = {
     _ns.get_is_contiguous: _get_is_contiguous,
     _ns.make_contiguous: lambda impl: impl,
     _ns.to_tensor_list: lambda impl: list(NestedTensor(impl).unbind()),
+    _ns.transpose_nchw_nhwc: ops.transpose_nchw_nhwc,
+    _ns.transpose_nhwc_nchw: ops.transpose_nhwc_nchw,
+    _ns.to_sparse_csr: ops.to_sparse_csr,
     torch.nn.functional.layer_norm: _nn_functional_layer_norm,
     torch.nn.functional.embedding: lambda input, weight, *a, **k: ops.embedding(weight, input, *a, **k),
     torch.embedding: lambda weight, indices, *a, **k: ops.embedding(weight, indices),

@@ -46,6 +46,9 @@ _SCHEMAS = [
     "get_is_contiguous(Tensor self, MemoryFormat memory_format) -> bool",
     "make_contiguous(Tensor self) -> Tensor",
     "to_tensor_list(Tensor tensor) -> Tensor[]",
+    "transpose_nhwc_nchw(Tensor self) -> Tensor",
+    "transpose_nchw_nhwc(Tensor self) -> Tensor",
+    "to_sparse_csr(Tensor tensor) -> Tensor",
 ]
 for _s in _SCHEMAS:
     _lib.define(_s)
@@ -709,3 +712,51 @@ def to_packed_sequence(impl):
                                        _C.ptr(data), T, None, stream))
     return torch.nn.utils.rnn.PackedSequence(data, batch_sizes, sorted_indices.to(dev),
                                              unsorted_indices.to(dev))
+
+
+# ---- channels-last ragged images: per-constituent transposes ------------------------
+
+def _transpose_constituents(impl, rows, cols, new_sizes):
+    """Every constituent, seen as a row-major [rows[b], cols[b]] matrix, is
+    transposed in place of its slot of the packed buffer (nt_transpose_ragged)."""
+    buf = impl.buffer
+    _C.require_device(buf, "transpose")
+    B = impl.B
+    tiles = ((rows + 63) // 64) * ((cols + 63) // 64)
+    meta = torch.zeros((3, B + 1), dtype=torch.int64)
+    meta[0, :B], meta[1, :B] = rows, cols
+    meta[2, 1:] = torch.cumsum(tiles, 0)
+    total_tiles = int(meta[2, B])
+    meta_dev = meta.to(buf.device)
+    out = torch.empty_like(buf)
+    if total_tiles:
+        with torch.cuda.device(buf.device):
+            _C.check(_C.lib.nt_transpose_ragged(
+                _C.ptr(buf), _C.ptr(out), _C.ptr(impl.offsets_dev()), _C.ptr(meta_dev[0]),
+                _C.ptr(meta_dev[1]), _C.ptr(meta_dev[2]), B, total_tiles, buf.element_size(),
+                _C.current_stream(buf.device)))
+    return NestedTensorImpl(out, new_sizes)
+
+
+def transpose_nchw_nhwc(impl):
+    """transpose_nchw_nhwc (transpose.cpp:122-146): constituents [C, H_i, W_i]
+    with a regular C become [H_i, W_i, C]."""
+    if impl.dim() != 4:
+        raise RuntimeError("transpose_nchw_nhwc needs 4d input.")
+    if impl.opt_sizes()[1] is None:
+        raise RuntimeError("Expected first dimension to be regular.")
+    s = impl.sizes
+    return _transpose_constituents(impl, s[:, 0], s[:, 1] * s[:, 2],
+                                   torch.stack([s[:, 1], s[:, 2], s[:, 0]], 1).contiguous())
+
+
+def transpose_nhwc_nchw(impl):
+    """transpose_nhwc_nchw (transpose.cpp:183-204): constituents [H_i, W_i, C]
+    with a regular C become [C, H_i, W_i]."""
+    if impl.dim() != 4:
+        raise RuntimeError("transpose_nhwc_nchw needs 4d input.")
+    if impl.opt_sizes()[3] is None:
+        raise RuntimeError("Expected last dimension to be regular.")
+    s = impl.sizes
+    return _transpose_constituents(impl, s[:, 0] * s[:, 1], s[:, 2],
+                                   torch.stack([s[:, 2], s[:, 0], s[:, 1]], 1).contiguous())

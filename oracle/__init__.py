@@ -75,4 +75,5 @@ from .masking import (  # noqa: F401
 from .mha import min_mha, bt_min_mha  # noqa: F401
 from .rowops import layer_norm, add  # noqa: F401
 from .dense import max_pool2d, conv2d  # noqa: F401
-from .interop import embedding, embedding_bag, to_sparse_csr, to_packed_sequence  # noqa: F401
+from .interop import (  # noqa: F401
+    embedding, embedding_bag, to_sparse_csr, to_packed_sequence, transpose_nchw_nhwc, transpose_nhwc_nchw)

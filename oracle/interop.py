@@ -51,3 +51,23 @@ def to_packed_sequence(nt):
     if not nt.dim() == 3:
         raise RuntimeError("NestedTensor should consistent of 2d Tensors of size L x *")
     return torch.nn.utils.rnn.pack_sequence(nt.unbind(), enforce_sorted=False)
+
+
+def transpose_nchw_nhwc(nt):
+    """transpose.cpp:122-146: every constituent permuted (1, 2, 0) and made
+    contiguous, which is what the reference's test compares with
+    (test/test_nested_tensor_class.py:820-840)."""
+    if nt.dim() != 4:
+        raise RuntimeError("transpose_nchw_nhwc needs 4d input.")
+    if nt.opt_sizes()[1] is None:
+        raise RuntimeError("Expected first dimension to be regular.")
+    return RefNestedTensor([t.permute(1, 2, 0).contiguous() for t in nt.unbind()], nt.dtype)
+
+
+def transpose_nhwc_nchw(nt):
+    """transpose.cpp:183-204: the inverse, permute (2, 0, 1)."""
+    if nt.dim() != 4:
+        raise RuntimeError("transpose_nhwc_nchw needs 4d input.")
+    if nt.opt_sizes()[3] is None:
+        raise RuntimeError("Expected last dimension to be regular.")
+    return RefNestedTensor([t.permute(2, 0, 1).contiguous() for t in nt.unbind()], nt.dtype)

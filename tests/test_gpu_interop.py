@@ -107,3 +107,30 @@ def test_to_packed_sequence(dtype):
         assert torch.equal(ps.unsorted_indices.cpu(), ref.unsorted_indices)
         padded, lengths = torch.nn.utils.rnn.pad_packed_sequence(ps, batch_first=True)
         assert torch.equal(padded, a.to_padded_tensor(0))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.int64, torch.uint8])
+def test_transpose_nchw_nhwc_round_trip(dtype):
+    # test/test_nested_tensor_class.py:820-840: 20 images [32, H, W], H, W in [20, 100]
+    import random
+    random.seed(1010)
+    shapes = [(32, random.randint(20, 100), random.randint(20, 100)) for _ in range(20)] + [(32, 1, 1), (32, 129, 3)]
+    g = torch.Generator().manual_seed(7)
+    ts = [(torch.randn(*s, generator=g) * 50).to(dtype) for s in shapes]
+    a = nt.nested_tensor(ts, device=DEV, dtype=dtype)
+    ref = oracle.ref_nested_tensor(ts, dtype=dtype)
+    a0 = nt.transpose_nchw_nhwc(a)
+    e0 = oracle.transpose_nchw_nhwc(ref)
+    assert a0.nested_size() == nt.nested_tensor(list(e0.unbind())).nested_size()
+    assert torch.equal(a0._impl.buffer.cpu(), e0.buffer)
+    a2 = nt.transpose_nhwc_nchw(a0)
+    assert a2.nested_size() == a.nested_size()
+    assert torch.equal(a2._impl.buffer, a._impl.buffer)
+
+
+def test_transpose_errors_and_irregular_channels():
+    a = nt.nested_tensor([torch.randn(2, 3, 3), torch.randn(3, 3, 3)], device=DEV)
+    with pytest.raises(RuntimeError, match="Expected first dimension to be regular."):
+        nt.transpose_nchw_nhwc(a)
+    with pytest.raises(RuntimeError, match="transpose_nchw_nhwc needs 4d input."):
+        nt.transpose_nchw_nhwc(nt.nested_tensor([torch.randn(2, 3)], device=DEV))

@@ -57,3 +57,18 @@ def test_to_packed_sequence_round_trip():
     assert torch.equal(padded, oracle.to_padded_tensor(nt, 0))
     assert lengths.tolist() == [4, 7, 1, 7, 2]
     assert ps.batch_sizes.tolist() == [5, 4, 3, 3, 2, 2, 2]
+
+
+def test_transposes_are_inverse_permutations():
+    g = torch.Generator().manual_seed(5)
+    ts = [torch.randn(4, h, w, generator=g) for h, w in ((3, 5), (7, 2), (1, 1))]
+    nt = oracle.ref_nested_tensor(ts)
+    a = oracle.transpose_nchw_nhwc(nt)
+    for t, o in zip(ts, a.unbind()):
+        assert o.shape == (t.shape[1], t.shape[2], 4)
+        for c in range(4):
+            assert torch.equal(o[:, :, c], t[c])           # element [h, w, c] == [c, h, w]
+    back = oracle.transpose_nhwc_nchw(a)
+    assert torch.equal(back.buffer, nt.buffer)
+    with pytest.raises(RuntimeError, match="Expected first dimension to be regular."):
+        oracle.transpose_nchw_nhwc(oracle.ref_nested_tensor([torch.randn(2, 3, 3), torch.randn(3, 3, 3)]))
