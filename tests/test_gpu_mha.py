@@ -274,3 +274,37 @@ def test_linear_qkv_tile_shapes():
         assert (qk.float().cpu() - exp[:, :2 * E]).abs().max().item() <= 2e-2
         assert (vt[:, :T].float().cpu() - exp[:, 2 * E:].t()).abs().max().item() <= 2e-2
         assert vt[:, T:].abs().max().item() == 0      # nothing written past the last token
+
+
+def test_min_mha_under_hip_graph_replays():
+    # the three launches of a layer captured in a graph: every replay, with new
+    # input contents and eager work in between, must equal the eager result
+    E, H = 256, 4
+    xs, W_in, b_in, W_out, b_out = make_case(E, [37, 200, 64, 129], 21, torch.float16, bias_std=0.1)
+    a = nt.nested_tensor(xs, device=DEV, dtype=torch.float16)
+    dW_in, db_in, dW_out, db_out = (t.to(DEV) for t in (W_in, b_in, W_out, b_out))
+
+    def layer():
+        return torch.ops.nestedtensor.min_mha(H, 64, 0.0, False, a, a, a, dW_in, db_in, 0.125, dW_out, db_out)
+
+    for _ in range(3):          # warm up: schedule upload, kernel attributes, allocator
+        eager = layer()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layer()
+        with torch.cuda.graph(graph, stream=side):
+            out = layer()
+    torch.cuda.current_stream().wait_stream(side)
+    g = torch.Generator().manual_seed(22)
+    for rep in range(4):
+        new = torch.randn(a._impl.buffer.shape, generator=g).half().to(DEV)
+        a._impl.buffer.copy_(new)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out._impl.buffer.clone()
+        exp = layer()._impl.buffer
+        torch.cuda.synchronize()
+        assert torch.equal(got, exp), "replay %d differs from the eager layer" % rep
