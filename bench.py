@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-One step = one pass over BASELINE configuration C5: 4096 fp16 constituents
+One step = one pass over the headline configuration C5: 4096 fp16 constituents
 [L_i, 4096], L_i uniform in [1, 2048] (1.7e10 elements, 34 GB packed), padded to
 the chunk maximum in chunks of 512 constituents (nt_add_padding) and un-padded
 again (nt_remove_padding).  All data is generated on the device and is resident
@@ -338,7 +338,7 @@ def _time_cpu(fn, runs=2):
 
 
 def bench_rows(args, torch, dev):
-    """The other rows of the hot path, each on the BASELINE configuration that
+    """The other rows of the hot path, each on the benchmark configuration that
     exercises it, through the package's Python surface (so allocation of the
     result and, for dense -> nested, the device-to-host copy of the row counts
     are inside the timed region).  GB/s = algorithmic bytes / time."""
@@ -518,7 +518,7 @@ def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported "
-              "(the path shards by constituent ranges, see DESIGN.md)." % args.gpus, file=sys.stderr)
+              "(the path shards by constituent ranges; nothing here uses a second GPU)." % args.gpus, file=sys.stderr)
         sys.exit(2)
     import torch
     if not torch.cuda.is_available():

@@ -1,8 +1,8 @@
 """Parity of the HIP nested multi-head attention path with the CPU oracle.
 
-Tolerances (BASELINE north_star): fp32 <= 1e-5 relative to the output scale
+Tolerances of the benchmark definition: fp32 <= 1e-5 relative to the output scale
 (max |a-b| / max |b|), fp16 / bf16 <= 2e-2 absolute.  The shape list is the
-reference's (test/test_nested_tensor_functional.py:1142-1160) plus the BASELINE
+reference's (test/test_nested_tensor_functional.py:1142-1160) plus the benchmark
 configurations C3 (BERT-base, fp16) and C4 (bf16, high raggedness)."""
 
 import random

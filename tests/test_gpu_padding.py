@@ -315,7 +315,7 @@ def test_from_padded_tensor_length_based(dims, dtype):
     bits_equal(back2._impl.buffer, ref.buffer)
 
 
-# ---- BASELINE configurations -----------------------------------------------------
+# ---- benchmark configurations -----------------------------------------------------
 
 def test_config_c1_round_trip_bit_exact():
     g = torch.Generator().manual_seed(1010 + 0)

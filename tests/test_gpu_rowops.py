@@ -3,7 +3,7 @@
 Tolerances: fp32 <= 1e-5 relative to the output scale, fp16 / bf16 <= 2e-2
 absolute (outputs are O(1)).  The size list is the reference's
 (test/test_nested_tensor_functional.py:935-939) plus the encoder widths of the
-BASELINE configurations."""
+benchmark configurations C3 and C4."""
 
 import pytest
 import torch
