@@ -33,6 +33,15 @@ typedef float float2v __attribute__((ext_vector_type(2)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
+// max over the two lanes l and l ^ 32 without the LDS round trip of a shuffle:
+// v_permlane32_swap exchanges the upper half of one register with the lower half
+// of another, which leaves (lo, lo) in one and (hi, hi) in the other.
+__device__ __forceinline__ float max_across_halves(float v) {
+  const unsigned b = __builtin_bit_cast(unsigned, v);
+  const auto r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+  return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+}
+
 template <typename T> struct AttnT;
 template <> struct AttnT<_Float16> {
   typedef half8 Frag;
@@ -198,7 +207,7 @@ __global__ __launch_bounds__(256) void varlen_attention_kernel(
           }
           m_tile = fmaxf(m_tile, s_acc[kb][e]);
         }
-      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
+      m_tile = max_across_halves(m_tile);
       const float m_new = fmaxf(m_run, m_tile);   // finite: every tile holds >= 1 valid key
       const float alpha = exp2f((m_run - m_new) * scale_log2e);
       const float m_scaled = m_new * scale_log2e;
@@ -451,7 +460,7 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int e = 0; e < 16; ++e) m_tile = fmaxf(m_tile, sa[kb][e]);
-    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
+    m_tile = max_across_halves(m_tile);
     const float m_new = fmaxf(m_run, m_tile);   // finite: every tile holds a valid key
     // raw v_exp_f32: arguments are <= 0, results in [0, 1]
     const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
