@@ -405,25 +405,42 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
       vm[j] = nv >= 2 * j + 2 ? 0xffffffffu : (nv == 2 * j + 1 ? 0x0000ffffu : 0u);
     }
   }
+  // Row 64 of a V^T buffer: 1 for every valid key.  Multiplied with P^T by the
+  // matrix pipe it yields the softmax denominators, and because it is zero past L
+  // (like the V^T columns) the keys of a partial tile need no masking of their
+  // scores.  Full tiles share the all-ones row written here once; the last tile
+  // writes its own masked row.
+  if (r0 == 0) {
+    const uint64_t ones = ((uint64_t)AT::kOnePair << 32) | AT::kOnePair;
+#pragma unroll
+    for (int b2 = 0; b2 < 2; ++b2) {
+      char* row = &lds_v[b2][kHd * kVRow + v_lo];
+      *reinterpret_cast<uint64_t*>(row) = ones;
+      *reinterpret_cast<uint64_t*>(row + 16) = ones;
+    }
+  }
   auto lstore_v = [&](int buf, int t) {
-    const bool last = t >= ntiles - 1;   // uniform
-    const uint32_t m0 = last ? vm[0] : 0xffffffffu, m1 = last ? vm[1] : 0xffffffffu;
-    const uint32_t m2 = last ? vm[2] : 0xffffffffu, m3 = last ? vm[3] : 0xffffffffu;
+    if (t < ntiles - 1) {   // uniform: a full tile, nothing to mask
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        char* row = &lds_v[buf][(r0 + i * 32) * kVRow + v_lo];
+        *reinterpret_cast<uint64_t*>(row) = ((uint64_t)rv[i].y << 32) | rv[i].x;
+        *reinterpret_cast<uint64_t*>(row + 16) = ((uint64_t)rv[i].w << 32) | rv[i].z;
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       char* row = &lds_v[buf][(r0 + i * 32) * kVRow + v_lo];
-      const uint64_t lo = ((uint64_t)(rv[i].y & m1) << 32) | (rv[i].x & m0);
-      const uint64_t hi = ((uint64_t)(rv[i].w & m3) << 32) | (rv[i].z & m2);
+      const uint64_t lo = ((uint64_t)(rv[i].y & vm[1]) << 32) | (rv[i].x & vm[0]);
+      const uint64_t hi = ((uint64_t)(rv[i].w & vm[3]) << 32) | (rv[i].z & vm[2]);
       *reinterpret_cast<uint64_t*>(row) = lo;
       *reinterpret_cast<uint64_t*>(row + 16) = hi;
     }
     if (r0 == 0) {
-      // row 64: 1 for every valid key.  Multiplied with P^T by the matrix pipe it
-      // yields the softmax denominators, and because it is zero past L (like the
-      // V^T rows) the keys of a partial tile need no masking of their scores.
       char* row = &lds_v[buf][kHd * kVRow + v_lo];
-      const uint64_t lo = ((uint64_t)(AT::kOnePair & m1) << 32) | (AT::kOnePair & m0);
-      const uint64_t hi = ((uint64_t)(AT::kOnePair & m3) << 32) | (AT::kOnePair & m2);
+      const uint64_t lo = ((uint64_t)(AT::kOnePair & vm[1]) << 32) | (AT::kOnePair & vm[0]);
+      const uint64_t hi = ((uint64_t)(AT::kOnePair & vm[3]) << 32) | (AT::kOnePair & vm[2]);
       *reinterpret_cast<uint64_t*>(row) = lo;
       *reinterpret_cast<uint64_t*>(row + 16) = hi;
     }
