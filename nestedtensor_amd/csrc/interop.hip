@@ -127,6 +127,94 @@ __global__ __launch_bounds__(64) void embedding_bag_kernel(
   out[b * n + c] = (T)acc;
 }
 
+// Rows of whole, aligned 16-byte pieces: a lane owns 8 (16-bit) or 4 (32-bit)
+// consecutive columns, the four wavefronts of a workgroup take every fourth token
+// of the bag with kAhead rows in flight each, and the partial results are combined
+// through LDS (so sums are formed in a different order than a sequential loop).
+template <typename T>
+__global__ __launch_bounds__(256) void embedding_bag_vec_kernel(
+    const T* __restrict__ weight, int64_t ldw, int64_t num_embeddings,
+    const int64_t* __restrict__ indices, const int64_t* __restrict__ offsets, T* __restrict__ out,
+    int64_t n, int mode, int32_t* __restrict__ oob) {
+  constexpr int kPer = 16 / sizeof(T);
+  constexpr int kAhead = 8;
+  __shared__ float part[4][kWave][kPer];
+  __shared__ int any_row[4];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int64_t b = blockIdx.x;
+  const int64_t c0 = ((int64_t)blockIdx.y * kWave + lane) * kPer;   // first column of this lane
+  const bool col_ok = c0 < n;                                       // n is a multiple of kPer
+  const int64_t begin = offsets[b], end = offsets[b + 1];
+  float acc[kPer];
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) acc[j] = 0.0f;
+  bool first = true;
+  for (int64_t t0 = begin + wave * kAhead; t0 < end; t0 += 4 * kAhead) {
+    u32x4 raw[kAhead];
+    bool use[kAhead];
+#pragma unroll
+    for (int j = 0; j < kAhead; ++j) {
+      const int64_t t = t0 + j;
+      const int64_t row = t < end ? indices[t] : 0;
+      const bool ok = row >= 0 && row < num_embeddings;
+      if (t < end && !ok && lane == 0 && blockIdx.y == 0 && oob) atomicAdd(oob, 1);
+      use[j] = t < end && ok;
+      raw[j] = *reinterpret_cast<const u32x4*>(weight + (use[j] ? row : 0) * ldw + (col_ok ? c0 : 0));
+    }
+#pragma unroll
+    for (int j = 0; j < kAhead; ++j) {
+      if (use[j]) {
+        T v[kPer];
+        __builtin_memcpy(v, &raw[j], 16);
+#pragma unroll
+        for (int e = 0; e < kPer; ++e) {
+          const float f = (float)v[e];
+          if (mode == kBagMax) {
+            acc[e] = first ? f : (f > acc[e] ? f : acc[e]);
+          } else {
+            acc[e] += f;
+          }
+        }
+        first = false;
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < kPer; ++e) part[wave][lane][e] = acc[e];
+  if (lane == 0) any_row[wave] = first ? 0 : 1;
+  __syncthreads();
+  if (wave != 0 || !col_ok) return;
+  float res[kPer];
+  bool have = false;
+#pragma unroll
+  for (int e = 0; e < kPer; ++e) res[e] = 0.0f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    if (!any_row[w]) continue;   // uniform
+#pragma unroll
+    for (int e = 0; e < kPer; ++e) {
+      const float f = part[w][lane][e];
+      if (mode == kBagMax) {
+        res[e] = have ? (f > res[e] ? f : res[e]) : f;
+      } else {
+        res[e] += f;
+      }
+    }
+    have = true;
+  }
+  T o[kPer];
+#pragma unroll
+  for (int e = 0; e < kPer; ++e) {
+    float f = res[e];
+    if (mode == kBagMean && end > begin) f = f / (float)(end - begin);
+    o[e] = (T)f;
+  }
+  u32x4 bits;
+  __builtin_memcpy(&bits, o, 16);
+  *reinterpret_cast<u32x4*>(out + b * n + c0) = bits;
+}
+
 static int pick_unit3(const void* a, const void* b, int64_t row_bytes) {
   const uintptr_t x = (uintptr_t)a | (uintptr_t)b | (uintptr_t)row_bytes;
   if ((x & 15) == 0) return 16;
@@ -211,12 +299,21 @@ extern "C" int nt_embedding_bag(const void* weight, int64_t ldw, int64_t num_emb
   if (B > 0x7fffffffLL || (n + 63) / 64 > 65535) {
     return fail(NT_ERR_UNSUPPORTED, "embedding_bag: too many bags or columns");
   }
-  dim3 grid((unsigned)B, (unsigned)((n + 63) / 64));
   hipStream_t s = (hipStream_t)stream;
-#define NT_BAG_CASE(TYPE)                                                                       \
-  hipLaunchKernelGGL((embedding_bag_kernel<TYPE>), grid, dim3(64), 0, s,                        \
-                     static_cast<const TYPE*>(weight), ldw, num_embeddings, indices, offsets,   \
-                     static_cast<TYPE*>(out), n, mode, oob_count);                              \
+  const int64_t elem = dtype == NT_F32 ? 4 : 2;
+  const int64_t per = 16 / elem;
+  const bool vec = n % per == 0 && ldw % per == 0 && (uintptr_t)weight % 16 == 0 && (uintptr_t)out % 16 == 0;
+  dim3 grid((unsigned)B, (unsigned)(vec ? (n / per + 63) / 64 : (n + 63) / 64));
+#define NT_BAG_CASE(TYPE)                                                                         \
+  if (vec) {                                                                                      \
+    hipLaunchKernelGGL((embedding_bag_vec_kernel<TYPE>), grid, dim3(256), 0, s,                   \
+                       static_cast<const TYPE*>(weight), ldw, num_embeddings, indices, offsets,   \
+                       static_cast<TYPE*>(out), n, mode, oob_count);                              \
+  } else {                                                                                        \
+    hipLaunchKernelGGL((embedding_bag_kernel<TYPE>), grid, dim3(64), 0, s,                        \
+                       static_cast<const TYPE*>(weight), ldw, num_embeddings, indices, offsets,   \
+                       static_cast<TYPE*>(out), n, mode, oob_count);                              \
+  }                                                                                               \
   break;
   switch (dtype) {
     case NT_F32: NT_BAG_CASE(float)

@@ -43,8 +43,9 @@ def test_embedding_out_of_range_raises():
 
 @pytest.mark.parametrize("mode", ["sum", "mean", "max"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
-def test_embedding_bag(mode, dtype):
-    V, E = 100, 8
+@pytest.mark.parametrize("E", [8, 7, 776])     # 16-byte column pieces, the scalar path, two column blocks
+def test_embedding_bag(mode, dtype, E):
+    V = 100
     for lens in ([5, 5], [5, 1, 12, 300], [3] * 70):       # first: the reference's case
         ids = _idx(lens, V, 3)
         w = torch.randn(V, E, generator=torch.Generator().manual_seed(4)).to(dtype)
