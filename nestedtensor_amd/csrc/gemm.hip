@@ -7,11 +7,13 @@
 // fragment is one 16-byte run of a row.  A workgroup owns a BM x BN tile of C,
 // its wavefronts a WAVES_M x WAVES_N grid of (WM*32) x (WN*32) sub-tiles made of
 // 32x32 MFMA blocks (fp32 accumulate; f16 / bf16: v_mfma_f32_32x32x16_*, fp32:
-// v_mfma_f32_32x32x2_f32).  K is walked in tiles of BKB bytes per row,
-// double-buffered in LDS; LDS rows are padded by 16 bytes so that the 128-bit
-// fragment reads of 16 consecutive lanes fall into distinct banks.  Global
-// loads run ahead of the MFMAs through registers, because one K tile of MFMA
-// work is far shorter than the L2 / HBM latency.
+// v_mfma_f32_32x32x2_f32).  K is walked in tiles of 128 bytes per row.  When K
+// is a whole number of tiles the K tiles go from global memory straight into LDS
+// (global_load_lds_dwordx4: no staging registers, no ds_write), two to three
+// tiles resident, in an unpadded layout whose 16-byte pieces are XOR-swizzled so
+// that the 128-bit fragment reads of 16 consecutive lanes fall into distinct
+// banks; any other K takes a register-staged loop with padded LDS rows and
+// element-wise tails.
 //
 // Three tile shapes are compiled (256x128, 256x192, 256x256, eight wavefronts
 // each); the launcher picks per problem the one with the least rounds x tile
@@ -28,9 +30,6 @@
 #include "nt_common.h"
 
 // Compile-time tuning knobs.
-#ifndef NT_GEMM_WAVES_PER_EU
-#define NT_GEMM_WAVES_PER_EU 2           // wavefronts per SIMD the kernels are compiled for
-#endif
 #ifndef NT_GEMM_FORCE_CFG
 #define NT_GEMM_FORCE_CFG (-1)           // 0, 1, 2: always that tile shape (experiments)
 #endif
@@ -67,11 +66,11 @@ template <> struct Mma<float> {
   }
 };
 
-template <int WAVES_M_, int WAVES_N_, int WM_, int WN_, int BKB_, int PF_>
+template <int WAVES_M_, int WAVES_N_, int WM_, int WN_, int BKB_>
 struct GemmCfg {
-  static constexpr int kPF = PF_;                     // K tiles in flight in registers
   static constexpr int kWavesM = WAVES_M_, kWavesN = WAVES_N_, kWM = WM_, kWN = WN_;
   static constexpr int kThreads = 64 * WAVES_M_ * WAVES_N_;
+  static constexpr int kWavesPerSimd = kThreads >= 512 ? 2 : 1;   // the kernel is compiled for this occupancy
   static constexpr int kBM = WAVES_M_ * WM_ * 32;
   static constexpr int kBN = WAVES_N_ * WN_ * 32;
   static constexpr int kRowBytes = BKB_;              // K-tile bytes per row
@@ -82,6 +81,12 @@ struct GemmCfg {
   static constexpr int kPerB = kBN * kChunksPerRow / kThreads;   // W pieces per thread
   static constexpr int kPerThread = kPerA + kPerB;
   static constexpr int kBufBytes = (kBM + kBN) * kLdsRow;
+  // direct global -> LDS loads: unpadded rows, as many K tiles resident as fit (at most 4)
+  static constexpr int kDmaTileBytes = (kBM + kBN) * BKB_;
+  static constexpr int kDmaBufs = (160 * 1024 - 2048) / kDmaTileBytes > 4 ? 4 : (160 * 1024 - 2048) / kDmaTileBytes;
+  // tile buffers (kernels for a ragged K use two padded, register-staged buffers)
+  static constexpr int kLdsBytes =
+      kDmaBufs * kDmaTileBytes > 2 * kBufBytes ? kDmaBufs * kDmaTileBytes : 2 * kBufBytes;
   static_assert((kBM * kChunksPerRow) % kThreads == 0 && (kBN * kChunksPerRow) % kThreads == 0,
                 "tile pieces must divide among the threads");
 };
@@ -153,7 +158,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
   constexpr int kBK = Cfg::kRowBytes / sizeof(T);
   constexpr int kSteps = kBK / MM::kK;
   constexpr int kFragBytes = (MM::kK / 2) * sizeof(T);
-  constexpr int WM = Cfg::kWM, WN = Cfg::kWN, PF = Cfg::kPF;
+  constexpr int WM = Cfg::kWM, WN = Cfg::kWN;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -172,98 +177,105 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   const int64_t nk = (a.K + kBK - 1) / kBK;
-  u32x4 stage[PF][Cfg::kPerThread];
 
   // bias of the tile's columns as fp32, behind the tile buffers (visible after
   // the first barrier below)
   if (tid < Cfg::kBN) {
     const int64_t col = n0 + tid;
-    reinterpret_cast<float*>(lds + 2 * Cfg::kBufBytes)[tid] =
+    reinterpret_cast<float*>(lds + Cfg::kLdsBytes)[tid] =
         (a.bias && col < a.N) ? (float)a.bias[col] : 0.0f;
   }
 
   if (ALIGNED_K) {
-    // Straight-line K loop (loads past the last K tile re-read it and are never
-    // consumed).  Every k-step issues, in this order: the LDS fragment reads of the
-    // NEXT k-step, its own MFMAs, and its share of the LDS stores of K tile kt + 1
-    // and of the global loads of K tile kt + 2.  The matrix pipe runs the MFMAs
-    // asynchronously, so the LDS and memory instructions behind them execute in
-    // their shadow; issued as one block after the barrier they would run while
-    // no wavefront of the workgroup has MFMAs in flight.
+    // K tiles travel global -> LDS directly (global_load_lds_dwordx4): no staging
+    // registers, no ds_write instructions.  A wavefront-level load writes its 64
+    // 16-byte pieces to 1 KiB of consecutive LDS, i.e. eight unpadded 128-byte rows,
+    // so bank conflicts of the fragment reads are avoided by WHICH piece of the row a
+    // lane fetches: slot p of row r holds piece p ^ ((r >> 1) & 7).  The compiler
+    // does not see these loads (inline asm), so their completion is awaited by hand
+    // before the barrier that publishes the tile.
+    static_assert(Cfg::kRowBytes == 128 && Cfg::kBM % 8 == 0, "1 KiB blocks of eight rows");
     constexpr int kN = Cfg::kPerThread;
-    auto gload_one = [&](int slot, int i, int64_t kt_in) {
-      const int64_t kt = kt_in >= nk ? nk - 1 : kt_in;
-      const bool is_a = i < Cfg::kPerA;
-      const int c = tid + (is_a ? i : i - Cfg::kPerA) * Cfg::kThreads;
-      const int row = c / Cfg::kChunksPerRow;
-      const int64_t k = kt * kBK + (c % Cfg::kChunksPerRow) * kPer;
-      stage[slot][i] = is_a ? load_chunk<T, true>(a.A, a.lda, m0 + row, a.M, k, a.K)
-                            : load_chunk<T, true>(a.W, a.K, n0 + row, a.N, k, a.K);
-    };
-    auto lstore_one = [&](int slot, int i, int buf) {
-      const bool is_a = i < Cfg::kPerA;
-      const int c = tid + (is_a ? i : i - Cfg::kPerA) * Cfg::kThreads;
-      const int row = (is_a ? 0 : Cfg::kBM) + c / Cfg::kChunksPerRow;
-      store16(lds + buf * Cfg::kBufBytes + row * Cfg::kLdsRow + (c % Cfg::kChunksPerRow) * 16,
-              stage[slot][i]);
-    };
-    auto read_frags = [&](Frag* fa, Frag* fb, int buf, int s) {
-      const char* a_base = lds + buf * Cfg::kBufBytes + (wm * WM * 32 + l32) * Cfg::kLdsRow;
-      const char* b_base =
-          lds + buf * Cfg::kBufBytes + (Cfg::kBM + wn * WN * 32 + l32) * Cfg::kLdsRow;
-      const int koff = s * MM::kK * (int)sizeof(T) + g * kFragBytes;
+    constexpr int kWaves = Cfg::kThreads / 64;
+    const char* gptr[kN];
 #pragma unroll
-      for (int i = 0; i < WM; ++i)
-        fa[i] = *reinterpret_cast<const Frag*>(a_base + i * 32 * Cfg::kLdsRow + koff);
-#pragma unroll
-      for (int j = 0; j < WN; ++j)
-        fb[j] = *reinterpret_cast<const Frag*>(b_base + j * 32 * Cfg::kLdsRow + koff);
-    };
-
-    // K tile j waits in register slot j % PF; tile 0 goes to LDS right away
-#pragma unroll
-    for (int i = 0; i < kN; ++i) gload_one(0, i, 0);
-#pragma unroll
-    for (int i = 0; i < kN; ++i) lstore_one(0, i, 0);
-#pragma unroll
-    for (int j = 1; j <= PF; ++j)
-#pragma unroll
-      for (int i = 0; i < kN; ++i) gload_one(j % PF, i, j);
-    __syncthreads();
-    for (int64_t kt0 = 0; kt0 < nk; kt0 += PF) {
-#pragma unroll
-      for (int j = 0; j < PF; ++j) {
-        const int64_t kt = kt0 + j;
-        if (PF > 1 && kt >= nk) break;                       // uniform: last, partial group
-        const int buf = (j + (int)(kt0 & 1) * (PF & 1)) & 1;   // == kt & 1
-        const int slot = (j + 1) % PF;                         // == (kt + 1) % PF
-        Frag fa[2][WM], fb[2][WN];
-        read_frags(fa[0], fb[0], buf, 0);
-#pragma unroll
-        for (int s = 0; s < kSteps; ++s) {
-          if (s + 1 < kSteps) read_frags(fa[(s + 1) & 1], fb[(s + 1) & 1], buf, s + 1);
-#pragma unroll
-          for (int i = 0; i < WM; ++i)
-#pragma unroll
-            for (int jj = 0; jj < WN; ++jj) {
-              if (VT_OUT) {
-                acc[i][jj] = MM::run(fa[s & 1][i], fb[s & 1][jj], acc[i][jj]);
-              } else {
-                acc[i][jj] = MM::run(fb[s & 1][jj], fa[s & 1][i], acc[i][jj]);
-              }
-            }
-#pragma unroll
-          for (int i = s * kN / kSteps; i < (s + 1) * kN / kSteps; ++i) {
-            lstore_one(slot, i, buf ^ 1);
-            gload_one(slot, i, kt + 1 + PF);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        __syncthreads();
+    for (int i = 0; i < kN; ++i) {
+      const int blk = i * kWaves + wave;
+      const int r = blk * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ ((r >> 1) & 7);
+      if (blk * 8 < Cfg::kBM) {          // uniform per (wave, i)
+        int64_t row = m0 + r;
+        row = row < a.M ? row : a.M - 1;
+        gptr[i] = reinterpret_cast<const char*>(a.A + row * a.lda + c * kPer);
+      } else {
+        int64_t row = n0 + r - Cfg::kBM;
+        row = row < a.N ? row : a.N - 1;
+        gptr[i] = reinterpret_cast<const char*>(a.W + row * a.K + c * kPer);
       }
     }
+    const unsigned lds_base = (unsigned)reinterpret_cast<uintptr_t>(lds);
+    constexpr int kNB = Cfg::kDmaBufs;
+    static_assert(kNB >= 2 && (kNB - 2) * kN <= 63, "vmcnt is a 6-bit counter");
+    auto dma_tile = [&](int buf, int64_t kt_in) {
+      const int64_t kt = kt_in >= nk ? nk - 1 : kt_in;    // past the end: re-read, never used
+#pragma unroll
+      for (int i = 0; i < kN; ++i) {
+        const unsigned dst = __builtin_amdgcn_readfirstlane(
+            lds_base + (unsigned)(buf * Cfg::kDmaTileBytes + (i * kWaves + wave) * 1024));
+        const char* src = gptr[i] + kt * Cfg::kRowBytes;
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                     :: "v"(src), "s"(dst) : "memory");
+      }
+    };
+    const int sw = (l32 >> 1) & 7;
+    auto read_frags = [&](Frag* fa, Frag* fb, int buf, int s) {
+      const char* a_base = lds + buf * Cfg::kDmaTileBytes + (wm * WM * 32 + l32) * 128;
+      const char* b_base = lds + buf * Cfg::kDmaTileBytes + (Cfg::kBM + wn * WN * 32 + l32) * 128;
+      const int off = s * MM::kK * (int)sizeof(T) + g * kFragBytes;   // byte offset in the row
+      const int koff = ((((off >> 4) ^ sw)) << 4) | (off & 15);
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+        fa[i] = *reinterpret_cast<const Frag*>(a_base + i * 32 * 128 + koff);
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+        fb[j] = *reinterpret_cast<const Frag*>(b_base + j * 32 * 128 + koff);
+    };
+    // K tiles kt + 1 .. kt + kNB - 1 are resident or in flight while tile kt is
+    // multiplied; the loads of the newest kNB - 2 tiles may still be outstanding
+    // when the barrier publishes tile kt + 1 (loads complete in order).
+#pragma unroll
+    for (int j = 0; j < kNB - 1; ++j) dma_tile(j, j);
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"((kNB - 2) * kN) : "memory");
+    __syncthreads();
+    int buf = 0;
+    for (int64_t kt = 0; kt < nk; ++kt) {
+      const int buf_new = buf == 0 ? kNB - 1 : buf - 1;    // == (kt + kNB - 1) % kNB, free since the last barrier
+      dma_tile(buf_new, kt + kNB - 1);
+      Frag fa[2][WM], fb[2][WN];
+      read_frags(fa[0], fb[0], buf, 0);
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s) {
+        if (s + 1 < kSteps) read_frags(fa[(s + 1) & 1], fb[(s + 1) & 1], buf, s + 1);
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+          for (int jj = 0; jj < WN; ++jj) {
+            if (VT_OUT) {
+              acc[i][jj] = MM::run(fa[s & 1][i], fb[s & 1][jj], acc[i][jj]);
+            } else {
+              acc[i][jj] = MM::run(fb[s & 1][jj], fa[s & 1][i], acc[i][jj]);
+            }
+          }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      asm volatile("s_waitcnt vmcnt(%0)" :: "n"((kNB - 2) * kN) : "memory");
+      __syncthreads();
+      buf = buf + 1 == kNB ? 0 : buf + 1;
+    }
   } else {
-    // Any K: element-wise tails, one K tile in registers ahead of the MFMAs.
+    // Any K: element-wise tails, one K tile in registers ahead of the MFMAs, two
+    // padded LDS buffers.
+    u32x4 stage[1][Cfg::kPerThread];
     auto gload = [&](int64_t kt) {
 #pragma unroll
       for (int i = 0; i < Cfg::kPerA; ++i) {
@@ -329,9 +341,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
   constexpr int kStripW = VT_OUT ? WM : WN;                    // 32-wide blocks per strip row
   constexpr int kStripRow = kStripW * 32 * (int)sizeof(T) + 16;
   constexpr int kCpr = kStripW * 32 * (int)sizeof(T) / 16;    // 16-byte pieces per strip row
-  static_assert((Cfg::kThreads / 64) * 32 * kStripRow <= 2 * Cfg::kBufBytes, "strips must fit");
+  static_assert((Cfg::kThreads / 64) * 32 * kStripRow <= Cfg::kLdsBytes, "strips must fit");
   char* strip = lds + wave * (32 * kStripRow);
-  const float* lds_bias = reinterpret_cast<const float*>(lds + 2 * Cfg::kBufBytes);
+  const float* lds_bias = reinterpret_cast<const float*>(lds + Cfg::kLdsBytes);
   typedef T Quad __attribute__((ext_vector_type(4)));
 
   if (!VT_OUT) {
@@ -431,7 +443,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
 // its default it schedules for maximum occupancy, keeps three fragments live
 // and waits for LDS in front of every MFMA.
 template <typename T, class Cfg, int EPI, bool ALIGNED_K>
-__global__ __launch_bounds__(Cfg::kThreads, NT_GEMM_WAVES_PER_EU) void linear_kernel(GemmArgs<T> a) {
+__global__ __launch_bounds__(Cfg::kThreads, Cfg::kWavesPerSimd) void linear_kernel(GemmArgs<T> a) {
   extern __shared__ __align__(16) char lds[];
   const int64_t tiles_m = (a.M + Cfg::kBM - 1) / Cfg::kBM;
   const int64_t per_xcd = (tiles_m + 7) / 8;
@@ -455,7 +467,7 @@ static int launch_kernel(const GemmArgs<T>& a, hipStream_t stream) {
   const int64_t tiles_n = (a.N + Cfg::kBN - 1) / Cfg::kBN;
   const int64_t wgs = ((tiles_m + 7) / 8) * 8 * tiles_n;
   if (wgs > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "linear: too many tiles");
-  const int lds_bytes = 2 * Cfg::kBufBytes + Cfg::kBN * (int)sizeof(float);
+  const int lds_bytes = Cfg::kLdsBytes + Cfg::kBN * (int)sizeof(float);
   static bool attr_set = false;
   if (!attr_set && lds_bytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(
@@ -477,10 +489,10 @@ static int launch_cfg(const GemmArgs<T>& a, hipStream_t stream) {
   return launch_kernel<T, Cfg, EPI, false>(a, stream);
 }
 
-// WAVES_M, WAVES_N, WM, WN, K-tile bytes, K tiles in flight in registers
-typedef GemmCfg<4, 2, 2, 2, 128, 1> Cfg128;   // 256 x 128
-typedef GemmCfg<4, 2, 2, 3, 128, 1> Cfg192;   // 256 x 192
-typedef GemmCfg<4, 2, 2, 4, 128, 1> Cfg256;   // 256 x 256
+// WAVES_M, WAVES_N, WM, WN, K-tile bytes per row
+typedef GemmCfg<4, 2, 2, 2, 128> Cfg128;   // 256 x 128
+typedef GemmCfg<4, 2, 2, 3, 128> Cfg192;   // 256 x 192
+typedef GemmCfg<4, 2, 2, 4, 128> Cfg256;   // 256 x 256
 
 // Tile shape with the least (rounds over the CUs) x (tile area / efficiency).
 // The efficiencies are the measured steady-state MFMA rates of the shapes
