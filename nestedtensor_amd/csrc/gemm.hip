@@ -193,7 +193,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
     // so bank conflicts of the fragment reads are avoided by WHICH piece of the row a
     // lane fetches: slot p of row r holds piece p ^ ((r >> 1) & 7).  The compiler
     // does not see these loads (inline asm), so their completion is awaited by hand
-    // before the barrier that publishes the tile.
+    // before the barrier that publishes the tile.  The asm writes M0 (the LDS
+    // destination); nothing else in these kernels uses M0 (no dynamic register
+    // indexing, no LDS-direct builtin), which is why it is not saved.
     static_assert(Cfg::kRowBytes == 128 && Cfg::kBM % 8 == 0, "1 KiB blocks of eight rows");
     constexpr int kN = Cfg::kPerThread;
     constexpr int kWaves = Cfg::kThreads / 64;
