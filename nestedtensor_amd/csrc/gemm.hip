@@ -496,9 +496,13 @@ typedef GemmCfg<4, 2, 2, 2, 128> Cfg128;   // 256 x 128
 typedef GemmCfg<4, 2, 2, 3, 128> Cfg192;   // 256 x 192
 typedef GemmCfg<4, 2, 2, 4, 128> Cfg256;   // 256 x 256
 
-// Tile shape with the least (rounds over the CUs) x (tile area / efficiency).
-// The efficiencies are the measured steady-state MFMA rates of the shapes
-// relative to 256x128 (less LDS traffic per MFMA with wider wavefront tiles).
+// Tile shape with the least estimated time.  A tile costs its area divided by the
+// measured steady-state rate of its shape relative to 256x128 (wider wavefront
+// tiles read less LDS and L2 per MFMA).  The number of tiles a CU runs one after
+// the other is taken as the mean of the whole rounds (all tiles start together
+// and take equally long) and of tiles / CUs (a partly filled last round runs
+// faster, it shares the memory path with fewer workgroups); fitted on the
+// projection shapes of the two attention benchmarks and on large square problems.
 static int pick_cfg(int64_t M, int64_t N, int64_t n_split, int* which) {
   static int num_cus = 0;
   if (num_cus == 0) {
@@ -511,15 +515,16 @@ static int pick_cfg(int64_t M, int64_t N, int64_t n_split, int* which) {
     num_cus = prop.multiProcessorCount;
   }
   const int bn[3] = {Cfg128::kBN, Cfg192::kBN, Cfg256::kBN};
-  const double eff[3] = {1.0, 1.08, 1.15};
+  const double eff[3] = {1.0, 1.08, 1.17};
   int best = -1;
   double best_cost = 0.0;
   for (int c = 0; c < 3; ++c) {
     if (n_split % bn[c] != 0) continue;          // a tile must not straddle the K | V boundary
     if (NT_GEMM_FORCE_CFG >= 0 && c != NT_GEMM_FORCE_CFG) continue;
     const int64_t tiles = ((M + 255) / 256) * ((N + bn[c] - 1) / bn[c]);
-    const int64_t rounds = (tiles + num_cus - 1) / num_cus;
-    const double cost = (double)rounds * bn[c] / eff[c];
+    const double whole = (double)((tiles + num_cus - 1) / num_cus);
+    const double fluid = (double)tiles / num_cus;
+    const double cost = 0.5 * (whole + fluid) * bn[c] / eff[c];
     if (best < 0 || cost < best_cost) {
       best = c;
       best_cost = cost;
