@@ -557,6 +557,17 @@ def conv2d(impl, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
         raise NotImplementedError("conv2d on a NestedTensor: string padding is not supported.")
     s, p, d = _pair(stride), _pair(padding), _pair(dilation)
     k = (weight.size(2), weight.size(3))
+    if (impl.dim() == 4 and bias is None and k == (1, 1) and s == (1, 1) and p == (0, 0) and d == (1, 1)
+            and groups == 1 and impl.opt_sizes()[1] is not None and impl.buffer.is_cuda
+            and weight.dtype == impl.buffer.dtype and weight.size(1) == impl.opt_sizes()[1]):
+        # 1x1 convolution = one GEMM over all pixels of all images (conv2d.cpp:33-75):
+        # NCHW -> NHWC on the packed buffer, [pixels, C_in] x W^T, and back
+        nhwc = transpose_nchw_nhwc(impl)
+        c_in, c_out = weight.size(1), weight.size(0)
+        y = linear(nhwc.buffer.reshape(-1, c_in), weight.reshape(c_out, c_in), None)
+        sizes = nhwc.sizes.clone()
+        sizes[:, 2] = c_out
+        return transpose_nhwc_nchw(NestedTensorImpl(y.reshape(-1), sizes))
     return _dense_via_padding(
         impl, 0.0, lambda x: torch.conv2d(x, weight, bias, s, p, d, groups), weight.size(0), k, s, p, d)
 

@@ -72,3 +72,20 @@ def test_dense_callers_errors():
     a = nt.nested_tensor([torch.randn(3, 4), torch.randn(2, 4)], device=DEV)
     with pytest.raises(RuntimeError, match="Input must be 4 dimensional."):
         torch.nn.functional.max_pool2d(a, 2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_conv2d_1x1_runs_as_one_gemm(dtype):
+    # conv2d.cpp:33-75: no bias, 1x1, unit stride -> transpose, packed GEMM, transpose back;
+    # shapes of the reference's 1x1 test plus an image-sized case
+    for shapes, c_out in (([(2, 2, 3), (2, 4, 2), (2, 2, 2)], 3), ([(64, 37, 50), (64, 128, 9), (64, 1, 1)], 96)):
+        ts = _rand(shapes, dtype, 5)
+        c_in = shapes[0][0]
+        w = (torch.randn(c_out, c_in, 1, 1, generator=torch.Generator().manual_seed(6)) * 0.3).to(dtype)
+        a = nt.nested_tensor(ts, device=DEV, dtype=dtype)
+        got = torch.conv2d(a, w.to(DEV))
+        ref = oracle.conv2d(oracle.ref_nested_tensor([t.float() for t in ts], dtype=torch.float32), w.float())
+        assert [tuple(x.shape) for x in got.unbind()] == [tuple(x.shape) for x in ref.unbind()]
+        err = (got._impl.buffer.float().cpu() - ref.buffer).abs().max().item()
+        scale = max(1.0, ref.buffer.abs().max().item())
+        assert err <= (1e-5 if dtype == torch.float32 else 2e-2) * scale, err
