@@ -492,7 +492,19 @@ def bench_rows(args, torch, dev):
     assert torch.equal(_ops.transpose_nhwc_nchw(nhwc).buffer, buf_t)
     rows["C2x64ch_transpose_nchw_nhwc_fp16"] = entry(ms_t0, 2 * 2 * buf_t.numel())
     rows["C2x64ch_transpose_nhwc_nchw_fp16"] = entry(ms_t1, 2 * 2 * buf_t.numel())
-    del buf_t, img, nhwc
+    # 1x1 convolution 64 -> 256 channels: row-major input (transpose, GEMM, transpose)
+    # against the channels-last storage of the same images (the GEMM alone)
+    w11 = (torch.randn(256, 64, 1, 1, device=dev) * 0.1).half()
+    img_cl = _ops.contiguous(img, torch.channels_last)
+    pix = buf_t.numel() // 64
+    ms_c0 = _time_gpu(torch, lambda: _ops.conv2d(img, w11), iters=10)
+    ms_c1 = _time_gpu(torch, lambda: _ops.conv2d(img_cl, w11), iters=10)
+    conv_bytes = 2 * pix * (64 + 256)
+    for key, ms_c in (("C2x64ch_conv2d_1x1_to_256ch_fp16", ms_c0),
+                      ("C2x64ch_conv2d_1x1_to_256ch_channels_last_fp16", ms_c1)):
+        rows[key] = entry(ms_c, conv_bytes, None, pixels=pix)
+        rows[key]["tflops"] = 2.0 * pix * 64 * 256 / (ms_c * 1e-3) / 1e12
+    del buf_t, img, nhwc, img_cl, w11
 
     # ---- C4: bt_min_mha bf16, high raggedness ---------------------------------
     g = torch.Generator().manual_seed(1010 + 3)

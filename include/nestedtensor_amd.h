@@ -260,13 +260,20 @@ int nt_embedding_bag(const void* weight, int64_t ldw, int64_t num_embeddings, co
  * [cols[b], rows[b]] transpose at the same offset of out.  rows = C, cols =
  * H_b * W_b is the reference's transpose_nchw_nhwc, the two exchanged its
  * transpose_nhwc_nchw (nestedtensor/csrc/transpose.cpp:87-204 with the
- * launchers of nestedtensor/csrc/cuda/transpose.h:11-31).  tile_offsets
- * int64[B + 1]: tile_offsets[b] = sum over c < b of ceil(rows[c] / 64) *
- * ceil(cols[c] / 64) (nt_offsets_from_sizes over a [B, 2] array of the two tile
- * counts builds it); total_tiles = tile_offsets[B].  All arrays on the device. */
+ * launchers of nestedtensor/csrc/cuda/transpose.h:11-31).  A workgroup moves one
+ * tile_rows x tile_cols tile of one constituent; the caller chooses the shape
+ * among 64x64, 64x128, 128x64, 128x128, 64x256, 256x64 with tile_rows *
+ * tile_cols * elem_bytes <= 32768 (taller tiles write longer contiguous pieces
+ * of the output rows), or, with S = 2048 / elem_bytes, the strips 16 x S when
+ * every rows[b] <= 16 and S x 16 when every cols[b] <= 16 (a constituent that
+ * breaks that promise is left unwritten).  tile_offsets int64[B + 1]: tile_offsets[b] = sum over c < b of
+ * ceil(rows[c] / tile_rows) * ceil(cols[c] / tile_cols) (nt_offsets_from_sizes
+ * over a [B, 2] array of the two tile counts builds it); total_tiles =
+ * tile_offsets[B].  All arrays on the device. */
 int nt_transpose_ragged(const void* in, void* out, const int64_t* offsets, const int64_t* rows,
                         const int64_t* cols, const int64_t* tile_offsets, int64_t B,
-                        int64_t total_tiles, int elem_bytes, void* stream);
+                        int64_t total_tiles, int tile_rows, int tile_cols, int elem_bytes,
+                        void* stream);
 
 #ifdef __cplusplus
 }

@@ -332,52 +332,67 @@ extern "C" int nt_embedding_bag(const void* weight, int64_t ldw, int64_t num_emb
 // cols = H_b * W_b this is NCHW -> NHWC of a batch of ragged images, and the
 // other way round with the two exchanged (the reference's
 // transpose_nchw_nhwc / transpose_nhwc_nchw, nestedtensor/csrc/transpose.cpp:87-204,
-// kernels nestedtensor/csrc/cuda/transpose.cu).  One workgroup per 64 x 64 tile,
+// kernels nestedtensor/csrc/cuda/transpose.cu).  One workgroup per TR x TC tile,
 // through LDS, so that both the reads and the writes are contiguous per
 // wavefront; tile_offsets[b] = number of tiles of all constituents before b, and
-// a workgroup finds its constituent by binary search.
+// a workgroup finds its constituent by binary search.  The caller picks the tile
+// shape: 64 x 64 in general, and a tile that is longer along the long side of a
+// narrow matrix (the [C, H*W] / [H*W, C] matrices of images have C of 64 or so),
+// so that the strided side moves 256 or 512 contiguous bytes per row of the tile
+// instead of 128.
 namespace nt {
 
-constexpr int kTrTile = 64;
+constexpr int kTrMaxTileBytes = 32 * 1024;
 
-template <typename U>
+template <typename U, int TR, int TC>
 __global__ __launch_bounds__(256) void transpose_ragged_kernel(
     const U* __restrict__ in, U* __restrict__ out, const int64_t* __restrict__ offsets,
     const int64_t* __restrict__ rows, const int64_t* __restrict__ cols,
     const int64_t* __restrict__ tile_offsets, int64_t B) {
   // a lane moves V consecutive elements (8 bytes) per access on both sides
   constexpr int V = 8 / (int)sizeof(U);
-  constexpr int kLanesPerRow = kTrTile / V;
-  constexpr int kRowsPerPass = 256 / kLanesPerRow;
-  constexpr int kStride = kTrTile + V;      // keeps every row of the tile 8-byte aligned
-  __shared__ __align__(8) U tile[kTrTile][kStride];
-  const int64_t id = blockIdx.x;
+  constexpr int kLanesIn = TC / V, kRowsPerPassIn = 256 / kLanesIn;
+  constexpr int kLanesOut = TR / V, kRowsPerPassOut = 256 / kLanesOut;
+  constexpr int kStride = TC + V;      // keeps every row of the tile 8-byte aligned
+  static_assert(kLanesIn <= 256 && kLanesOut <= 256, "tile too wide for 256 lanes");
+  __shared__ __align__(8) U tile[TR][kStride];
+  // Workgroups are dealt to the 8 XCDs in turn; give each XCD a contiguous run of
+  // tiles, so that neighbouring pieces of an output row meet in one L2.
+  int64_t id = blockIdx.x;
+  {
+    const int64_t per_xcd = gridDim.x / 8;
+    if (id < per_xcd * 8) id = (id % 8) * per_xcd + id / 8;
+  }
   const int64_t b = find_segment(tile_offsets, B, id);
   const int64_t R = rows[b], C = cols[b];
-  const int64_t tiles_c = (C + kTrTile - 1) / kTrTile;
+  const int64_t tiles_c = (C + TC - 1) / TC;
   const int64_t local = id - tile_offsets[b];
-  const int64_t r0 = (local / tiles_c) * kTrTile;
-  const int64_t c0 = (local % tiles_c) * kTrTile;
+  const int64_t r0 = (local / tiles_c) * TR;
+  const int64_t c0 = (local % tiles_c) * TC;
   const U* src = in + offsets[b];
   U* dst = out + offsets[b];
-  const int lv = (threadIdx.x % kLanesPerRow) * V;   // first of this lane's V elements
-  const int lr = threadIdx.x / kLanesPerRow;
-  for (int r = lr; r < kTrTile; r += kRowsPerPass) {
-    if (r0 + r < R) {
-      const U* p = src + (r0 + r) * C + c0 + lv;
-      if (c0 + lv + V <= C) {
-        uint64_t bits;
-        __builtin_memcpy(&bits, p, 8);                // any alignment
-        *reinterpret_cast<uint64_t*>(&tile[r][lv]) = bits;
-      } else {
+  {
+    const int lv = (threadIdx.x % kLanesIn) * V;   // first of this lane's V elements
+    const int lr = threadIdx.x / kLanesIn;
+    for (int r = lr; r < TR; r += kRowsPerPassIn) {
+      if (r0 + r < R) {
+        const U* p = src + (r0 + r) * C + c0 + lv;
+        if (c0 + lv + V <= C) {
+          uint64_t bits;
+          __builtin_memcpy(&bits, p, 8);                // any alignment
+          *reinterpret_cast<uint64_t*>(&tile[r][lv]) = bits;
+        } else {
 #pragma unroll
-        for (int j = 0; j < V; ++j)
-          if (c0 + lv + j < C) tile[r][lv + j] = p[j];
+          for (int j = 0; j < V; ++j)
+            if (c0 + lv + j < C) tile[r][lv + j] = p[j];
+        }
       }
     }
   }
   __syncthreads();
-  for (int c = lr; c < kTrTile; c += kRowsPerPass) {
+  const int lv = (threadIdx.x % kLanesOut) * V;
+  const int lr = threadIdx.x / kLanesOut;
+  for (int c = lr; c < TC; c += kRowsPerPassOut) {
     if (c0 + c < C) {
       U v[V];
 #pragma unroll
@@ -396,13 +411,124 @@ __global__ __launch_bounds__(256) void transpose_ragged_kernel(
   }
 }
 
+// Matrices with at most kTrNarrow rows (or columns): images of a few channels.  A
+// 64-wide tile would leave most of its lanes idle, so a workgroup takes a strip
+// of 256 * V columns (rows) of the long side instead, with V = 8 / sizeof(U), and
+// all the rows (columns) of the narrow side: the strip is contiguous in the
+// output (input) and is moved with 8-byte accesses; on the other side every lane
+// moves 8 contiguous bytes per row of the narrow side.  NARROW_ROWS: the input
+// has few rows (NCHW -> NHWC of few channels); otherwise it has few columns.
+constexpr int kTrNarrow = 16;
+
+template <typename U, bool NARROW_ROWS>
+__global__ __launch_bounds__(256) void transpose_narrow_kernel(
+    const U* __restrict__ in, U* __restrict__ out, const int64_t* __restrict__ offsets,
+    const int64_t* __restrict__ rows, const int64_t* __restrict__ cols,
+    const int64_t* __restrict__ tile_offsets, int64_t B) {
+  constexpr int V = 8 / (int)sizeof(U);
+  constexpr int kStrip = 256 * V;
+  __shared__ __align__(8) U tile[kStrip * kTrNarrow];
+  const int64_t id = blockIdx.x;
+  const int64_t b = find_segment(tile_offsets, B, id);
+  const int64_t R = rows[b], C = cols[b];
+  const int64_t s0 = (id - tile_offsets[b]) * kStrip;      // first index of the strip on the long side
+  const U* src = in + offsets[b];
+  U* dst = out + offsets[b];
+  if ((NARROW_ROWS ? R : C) > kTrNarrow) return;   // not a strip matrix: the tile would not hold it
+  const int narrow = (int)(NARROW_ROWS ? R : C);
+  const int64_t long_n = NARROW_ROWS ? C : R;
+  const int len = (int)(long_n - s0 < kStrip ? long_n - s0 : kStrip);   // strip length
+  const int lv = threadIdx.x * V;
+  // the contiguous side: len * narrow elements from s0 * narrow on
+  const int n_lin = len * narrow;
+  if (!NARROW_ROWS) {
+    const U* p = src + s0 * narrow;
+    for (int k = lv; k < n_lin; k += kStrip) {
+      if (k + V <= n_lin) {
+        uint64_t bits;
+        __builtin_memcpy(&bits, p + k, 8);
+        *reinterpret_cast<uint64_t*>(&tile[k]) = bits;
+      } else {
+        for (int j = 0; k + j < n_lin; ++j) tile[k + j] = p[k + j];
+      }
+    }
+  } else {
+    for (int r = 0; r < narrow; ++r) {
+      const U* p = src + r * C + s0 + lv;
+      if (lv + V <= len) {
+        U v[V];
+        __builtin_memcpy(v, p, 8);
+#pragma unroll
+        for (int j = 0; j < V; ++j) tile[(lv + j) * narrow + r] = v[j];
+      } else {
+        for (int j = 0; lv + j < len; ++j) tile[(lv + j) * narrow + r] = p[j];
+      }
+    }
+  }
+  __syncthreads();
+  if (NARROW_ROWS) {
+    U* q = dst + s0 * narrow;
+    for (int k = lv; k < n_lin; k += kStrip) {
+      if (k + V <= n_lin) {
+        const uint64_t bits = *reinterpret_cast<const uint64_t*>(&tile[k]);
+        __builtin_memcpy(q + k, &bits, 8);
+      } else {
+        for (int j = 0; k + j < n_lin; ++j) q[k + j] = tile[k + j];
+      }
+    }
+  } else {
+    for (int c = 0; c < narrow; ++c) {
+      U* q = dst + c * R + s0 + lv;
+      if (lv + V <= len) {
+        U v[V];
+#pragma unroll
+        for (int j = 0; j < V; ++j) v[j] = tile[(lv + j) * narrow + c];
+        __builtin_memcpy(q, v, 8);
+      } else {
+        for (int j = 0; lv + j < len; ++j) q[j] = tile[(lv + j) * narrow + c];
+      }
+    }
+  }
+}
+
 template <typename U>
-static void launch_transpose(const void* in, void* out, const int64_t* offsets, const int64_t* rows,
-                             const int64_t* cols, const int64_t* tile_offsets, int64_t B,
-                             int64_t total_tiles, hipStream_t stream) {
-  hipLaunchKernelGGL((transpose_ragged_kernel<U>), dim3((unsigned)total_tiles), dim3(256), 0, stream,
-                     static_cast<const U*>(in), static_cast<U*>(out), offsets, rows, cols,
-                     tile_offsets, B);
+static int launch_transpose(const void* in, void* out, const int64_t* offsets, const int64_t* rows,
+                            const int64_t* cols, const int64_t* tile_offsets, int64_t B,
+                            int64_t total_tiles, int tile_rows, int tile_cols, hipStream_t stream) {
+#define NT_TR_CASE(TR, TC)                                                                         \
+  if (tile_rows == TR && tile_cols == TC) {                                                        \
+    if constexpr ((size_t)TR * TC * sizeof(U) <= (size_t)kTrMaxTileBytes) {                        \
+      hipLaunchKernelGGL((transpose_ragged_kernel<U, TR, TC>), dim3((unsigned)total_tiles),        \
+                         dim3(256), 0, stream, static_cast<const U*>(in), static_cast<U*>(out),    \
+                         offsets, rows, cols, tile_offsets, B);                                    \
+      return check_launch("transpose_ragged_kernel");                                              \
+    }                                                                                              \
+  }
+  constexpr int kStrip = 256 * 8 / (int)sizeof(U);
+  if ((tile_rows == kTrNarrow && tile_cols == kStrip) || (tile_rows == kStrip && tile_cols == kTrNarrow)) {
+    // the strip kernels; the caller guarantees rows[b] <= 16 (cols[b] <= 16) for every b
+    if (tile_rows == kTrNarrow) {
+      hipLaunchKernelGGL((transpose_narrow_kernel<U, true>), dim3((unsigned)total_tiles), dim3(256), 0,
+                         stream, static_cast<const U*>(in), static_cast<U*>(out), offsets, rows, cols,
+                         tile_offsets, B);
+    } else {
+      hipLaunchKernelGGL((transpose_narrow_kernel<U, false>), dim3((unsigned)total_tiles), dim3(256), 0,
+                         stream, static_cast<const U*>(in), static_cast<U*>(out), offsets, rows, cols,
+                         tile_offsets, B);
+    }
+    return check_launch("transpose_narrow_kernel");
+  }
+  NT_TR_CASE(64, 64)
+  NT_TR_CASE(64, 128)
+  NT_TR_CASE(128, 64)
+  NT_TR_CASE(128, 128)
+  NT_TR_CASE(64, 256)
+  NT_TR_CASE(256, 64)
+#undef NT_TR_CASE
+  return fail(NT_ERR_UNSUPPORTED,
+              "transpose_ragged: tile %d x %d of %d-byte elements is not one of 64x64, 64x128, 128x64, "
+              "128x128, 64x256, 256x64 within %d bytes, nor the 16 x %d / %d x 16 strip", tile_rows,
+              tile_cols, (int)sizeof(U), kTrMaxTileBytes, kStrip, kStrip);
 }
 
 }  // namespace nt
@@ -410,7 +536,7 @@ static void launch_transpose(const void* in, void* out, const int64_t* offsets, 
 extern "C" int nt_transpose_ragged(const void* in, void* out, const int64_t* offsets,
                                    const int64_t* rows, const int64_t* cols,
                                    const int64_t* tile_offsets, int64_t B, int64_t total_tiles,
-                                   int elem_bytes, void* stream) {
+                                   int tile_rows, int tile_cols, int elem_bytes, void* stream) {
   if (B < 0 || total_tiles < 0) return nt::fail(NT_ERR_INVALID_ARGUMENT, "transpose_ragged: negative extent");
   if (B == 0 || total_tiles == 0) return NT_OK;
   if (!in || !out || !offsets || !rows || !cols || !tile_offsets) {
@@ -419,11 +545,12 @@ extern "C" int nt_transpose_ragged(const void* in, void* out, const int64_t* off
   if (total_tiles > 0x7fffffffLL) return nt::fail(NT_ERR_UNSUPPORTED, "transpose_ragged: too many tiles");
   hipStream_t s = (hipStream_t)stream;
   switch (elem_bytes) {
-    case 1: nt::launch_transpose<uint8_t>(in, out, offsets, rows, cols, tile_offsets, B, total_tiles, s); break;
-    case 2: nt::launch_transpose<uint16_t>(in, out, offsets, rows, cols, tile_offsets, B, total_tiles, s); break;
-    case 4: nt::launch_transpose<uint32_t>(in, out, offsets, rows, cols, tile_offsets, B, total_tiles, s); break;
-    case 8: nt::launch_transpose<uint64_t>(in, out, offsets, rows, cols, tile_offsets, B, total_tiles, s); break;
+#define NT_TR_ARGS in, out, offsets, rows, cols, tile_offsets, B, total_tiles, tile_rows, tile_cols, s
+    case 1: return nt::launch_transpose<uint8_t>(NT_TR_ARGS);
+    case 2: return nt::launch_transpose<uint16_t>(NT_TR_ARGS);
+    case 4: return nt::launch_transpose<uint32_t>(NT_TR_ARGS);
+    case 8: return nt::launch_transpose<uint64_t>(NT_TR_ARGS);
+#undef NT_TR_ARGS
     default: return nt::fail(NT_ERR_UNSUPPORTED, "transpose_ragged: element size %d", elem_bytes);
   }
-  return nt::check_launch("transpose_ragged_kernel");
 }

@@ -7,8 +7,15 @@ buffer, a host int64 table ``sizes[B, D]`` and the per-dimension "regular or
 not" summary ``opt_sizes``.  What is new here is the device side of the
 metadata: ``sizes`` mirrored in HBM and int64 element ``offsets[B + 1]`` built
 by the device prefix scan (nt_offsets_from_sizes), both cached on the impl and
-created on first use on the buffer's stream.  Only nested_dim 1 and the
-contiguous layout exist (EfficientSizeNode.h:86-88).
+created on first use on the buffer's stream.  Only nested_dim 1 exists
+(EfficientSizeNode.h:86-88).
+
+Two storage layouts exist, as in the reference (Packed.h:100-163): every
+constituent row-major contiguous, or, for constituents [C, H, W], every
+constituent stored as [H, W, C] ("channels last", the nested stride is then
+(1, W * C, C)).  The second is a flag on the impl, not a stride table: these
+are the only two layouts the reference's kernels accept, and the constituent
+extents, hence the element offsets, are the same in both.
 """
 
 import torch
@@ -18,16 +25,20 @@ from . import _C
 
 class NestedTensorImpl:
     __slots__ = ("buffer", "sizes", "_opt_sizes", "_sizes_dev", "_offsets_dev",
-                 "_row_offsets_dev", "_max_sizes", "_attn_schedule")
+                 "_row_offsets_dev", "_max_sizes", "_attn_schedule", "channels_last")
 
-    def __init__(self, buffer, sizes):
+    def __init__(self, buffer, sizes, channels_last=False):
         """buffer: 1-D contiguous tensor; sizes: CPU int64 [B, D], or 0-d for an
-        empty nested tensor (EfficientSizeNode.h:8-12)."""
+        empty nested tensor (EfficientSizeNode.h:8-12).  channels_last: the
+        buffer holds each [C, H, W] constituent as [H, W, C]."""
         if buffer.dim() != 1:
             raise RuntimeError("Given buffer must be vector, i.e. dim 1 Tensor.")
         if not buffer.is_contiguous():
             raise RuntimeError("Given buffer must be contiguous.")
         assert sizes.dtype == torch.int64 and sizes.device.type == "cpu"
+        if channels_last and not (sizes.dim() == 2 and sizes.size(1) == 3):
+            raise RuntimeError("ChannelsLast memory format requires 4 dim input.")
+        self.channels_last = bool(channels_last)
         self.buffer = buffer
         self.sizes = sizes
         self._opt_sizes = None
@@ -86,6 +97,21 @@ class NestedTensorImpl:
     def shapes(self):
         return [tuple(int(v) for v in row) for row in self.sizes] if self.sizes.dim() > 0 else []
 
+    def strides(self):
+        """Per-constituent element strides: row-major (Packed.h:10-19), or
+        (1, W * C, C) for the channels-last layout (nested_tensor_impl.cpp:188-192)."""
+        out = []
+        for s in self.shapes():
+            if self.channels_last:
+                out.append((1, s[2] * s[0], s[0]))
+                continue
+            st, acc = [], 1
+            for v in reversed(s):
+                st.append(acc)
+                acc *= v
+            out.append(tuple(reversed(st)))
+        return out
+
     # ---- device metadata ---------------------------------------------------
     def sizes_dev(self):
         if self._sizes_dev is None:
@@ -127,10 +153,12 @@ class NestedTensorImpl:
             self._attn_schedule = items.to(torch.int32).contiguous().to(self.buffer.device)
         return self._attn_schedule
 
-    def with_buffer(self, buffer):
-        """Same nested size over another buffer; shares the cached metadata when
-        the device matches."""
-        out = NestedTensorImpl(buffer, self.sizes)
+    def with_buffer(self, buffer, channels_last=None):
+        """Same nested size over another buffer (in the same layout unless
+        channels_last says otherwise); shares the cached metadata when the
+        device matches."""
+        out = NestedTensorImpl(buffer, self.sizes,
+                               self.channels_last if channels_last is None else channels_last)
         out._opt_sizes = self._opt_sizes
         out._max_sizes = self._max_sizes
         if buffer.device == self.buffer.device:

@@ -46,7 +46,9 @@ def nested_tensor_impl(data, dtype, device, requires_grad, pin_memory, channels_
             "This version of nestedtensor currently does not support autograd. Please open an "
             "issue on https://github.com/pytorch/nestedtensor if you need this.")
     if channels_last:
-        raise RuntimeError("channels_last nested tensors are not part of this build.")
+        # creation.cpp:217-219: pack row-major, then change the layout
+        impl = nested_tensor_impl(data, dtype, device, requires_grad, pin_memory, False)
+        return ops.contiguous(impl, torch.channels_last)
     if isinstance(data, nested.NestedTensor):
         data = data.unbind()   # a NestedTensor is a sequence of its constituents
     if torch.is_tensor(data) or not isinstance(data, (list, tuple)):

@@ -485,8 +485,15 @@ def add(impl, other, alpha=1):
     if isinstance(other, NestedTensorImpl):
         if other.sizes.shape != impl.sizes.shape or not torch.equal(other.sizes, impl.sizes):
             raise NotImplementedError("add of nested tensors of different nested size is not on the packed path.")
+        if not (impl.channels_last and other.channels_last):
+            # two channels-last operands add buffer to buffer and stay channels-last
+            # (BinaryOps.cpp:25-32); any other mix goes through the row-major layout (:33-43)
+            impl, other = contiguous(impl), contiguous(other)
+            buf = impl.buffer
         b, period = other.buffer, buf.numel()
     elif isinstance(other, torch.Tensor) and other.dim() == 1:
+        impl = contiguous(impl)
+        buf = impl.buffer
         opt = impl.opt_sizes()
         if opt[impl.dim() - 1] is None or opt[impl.dim() - 1] != other.size(0):
             raise NotImplementedError("add of a 1-D tensor needs a regular last dim of the same size.")
@@ -520,6 +527,8 @@ def _dense_via_padding(impl, pad_value, dense_op, out_channels, k, stride, paddi
     if impl.dim() != 4:
         raise RuntimeError("Input must be 4 dimensional.")
     _C.require_device(impl.buffer, "dense op on a NestedTensor")
+    was_channels_last = impl.channels_last
+    impl = contiguous(impl)
     data = to_padded_tensor(impl, pad_value)
     result = dense_op(data).contiguous()
     sizes = impl.sizes.clone()
@@ -530,7 +539,9 @@ def _dense_via_padding(impl, pad_value, dense_op, out_channels, k, stride, paddi
     if bool((sizes <= 0).any()):
         raise RuntimeError("Output size is too small")
     target = NestedTensorImpl(torch.empty(0, dtype=result.dtype, device=result.device), sizes)
-    return from_padded_tensor(result, target)
+    out = from_padded_tensor(result, target)
+    # a channels-last input gives a channels-last result (pooling.cpp:54-56, conv2d.cpp:88-90)
+    return contiguous(out, torch.channels_last) if was_channels_last else out
 
 
 def max_pool2d(impl, kernel_size, stride=None, padding=0, dilation=1, ceil_mode=False,
@@ -560,10 +571,18 @@ def conv2d(impl, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
     if (impl.dim() == 4 and bias is None and k == (1, 1) and s == (1, 1) and p == (0, 0) and d == (1, 1)
             and groups == 1 and impl.opt_sizes()[1] is not None and impl.buffer.is_cuda
             and weight.dtype == impl.buffer.dtype and weight.size(1) == impl.opt_sizes()[1]):
-        # 1x1 convolution = one GEMM over all pixels of all images (conv2d.cpp:33-75):
-        # NCHW -> NHWC on the packed buffer, [pixels, C_in] x W^T, and back
-        nhwc = transpose_nchw_nhwc(impl)
+        # 1x1 convolution = one GEMM over all pixels of all images (conv2d.cpp:33-75)
         c_in, c_out = weight.size(1), weight.size(0)
+        if impl.channels_last:
+            # the buffer already is the [pixels, C_in] matrix, and the product is
+            # the channels-last result (conv2d.cpp:43-60): no transposes
+            y = linear(impl.buffer.reshape(-1, c_in), weight.reshape(c_out, c_in), None)
+            sizes = impl.sizes.clone()
+            sizes[:, 0] = c_out
+            res = NestedTensorImpl(y.reshape(-1), sizes, channels_last=True)
+            return res
+        # NCHW -> NHWC on the packed buffer, [pixels, C_in] x W^T, and back (conv2d.cpp:61-73)
+        nhwc = transpose_nchw_nhwc(impl)
         y = linear(nhwc.buffer.reshape(-1, c_in), weight.reshape(c_out, c_in), None)
         sizes = nhwc.sizes.clone()
         sizes[:, 2] = c_out
@@ -727,13 +746,27 @@ def to_packed_sequence(impl):
 
 # ---- channels-last ragged images: per-constituent transposes ------------------------
 
+def _transpose_tile(max_rows, max_cols, elem_bytes):
+    """Tile shape for nt_transpose_ragged: the strip kernels (a workgroup per 2048
+    bytes of the long side) when the other side is at most 16, images of a few
+    channels; 64 x 64 otherwise.  The larger tiles the library also accepts keep
+    fewer workgroups in flight and measured slower on every image shape tried."""
+    strip = 2048 // elem_bytes
+    if max_rows <= 16 and max_cols > 64:
+        return 16, strip
+    if max_cols <= 16 and max_rows > 64:
+        return strip, 16
+    return 64, 64
+
+
 def _transpose_constituents(impl, rows, cols, new_sizes):
     """Every constituent, seen as a row-major [rows[b], cols[b]] matrix, is
     transposed in place of its slot of the packed buffer (nt_transpose_ragged)."""
     buf = impl.buffer
     _C.require_device(buf, "transpose")
     B = impl.B
-    tiles = ((rows + 63) // 64) * ((cols + 63) // 64)
+    tr, tc = _transpose_tile(int(rows.max()) if B else 0, int(cols.max()) if B else 0, buf.element_size())
+    tiles = ((rows + tr - 1) // tr) * ((cols + tc - 1) // tc)
     meta = torch.zeros((3, B + 1), dtype=torch.int64)
     meta[0, :B], meta[1, :B] = rows, cols
     meta[2, 1:] = torch.cumsum(tiles, 0)
@@ -744,14 +777,17 @@ def _transpose_constituents(impl, rows, cols, new_sizes):
         with torch.cuda.device(buf.device):
             _C.check(_C.lib.nt_transpose_ragged(
                 _C.ptr(buf), _C.ptr(out), _C.ptr(impl.offsets_dev()), _C.ptr(meta_dev[0]),
-                _C.ptr(meta_dev[1]), _C.ptr(meta_dev[2]), B, total_tiles, buf.element_size(),
+                _C.ptr(meta_dev[1]), _C.ptr(meta_dev[2]), B, total_tiles, tr, tc, buf.element_size(),
                 _C.current_stream(buf.device)))
-    return NestedTensorImpl(out, new_sizes)
+    res = NestedTensorImpl(out, new_sizes)
+    res._offsets_dev = impl._offsets_dev      # the constituents keep their extents
+    return res
 
 
 def transpose_nchw_nhwc(impl):
     """transpose_nchw_nhwc (transpose.cpp:122-146): constituents [C, H_i, W_i]
     with a regular C become [H_i, W_i, C]."""
+    impl = contiguous(impl)
     if impl.dim() != 4:
         raise RuntimeError("transpose_nchw_nhwc needs 4d input.")
     if impl.opt_sizes()[1] is None:
@@ -764,6 +800,7 @@ def transpose_nchw_nhwc(impl):
 def transpose_nhwc_nchw(impl):
     """transpose_nhwc_nchw (transpose.cpp:183-204): constituents [H_i, W_i, C]
     with a regular C become [C, H_i, W_i]."""
+    impl = contiguous(impl)
     if impl.dim() != 4:
         raise RuntimeError("transpose_nhwc_nchw needs 4d input.")
     if impl.opt_sizes()[3] is None:
@@ -771,3 +808,42 @@ def transpose_nhwc_nchw(impl):
     s = impl.sizes
     return _transpose_constituents(impl, s[:, 0] * s[:, 1], s[:, 2],
                                    torch.stack([s[:, 2], s[:, 0], s[:, 1]], 1).contiguous())
+
+
+def is_contiguous(impl, memory_format=torch.contiguous_format):
+    """get_is_contiguous (nested_tensor_impl.h:151-160)."""
+    if memory_format in (torch.contiguous_format, 0):
+        return not impl.channels_last
+    if memory_format in (torch.channels_last, 2):
+        # an empty buffer is contiguous in both senses (Packed.h:131-133)
+        return impl.channels_last or (impl.buffer.numel() == 0 and not impl.channels_last)
+    raise RuntimeError("is_contiguous does not support memory format " + str(memory_format))
+
+
+def contiguous(impl, memory_format=torch.contiguous_format):
+    """NestedTensor_contiguous (nested_tensor_impl.cpp:157-198): the same nested
+    tensor with its buffer in the requested layout.  Going to channels-last is
+    the NCHW -> NHWC transpose of every constituent with the nested size kept
+    (:182-194); coming back views the buffer as [H_i, W_i, C] constituents and
+    transposes them the other way (:165-179)."""
+    if memory_format == torch.preserve_format:
+        raise RuntimeError("preserve memory format is unsupported by the contiguous operator")
+    if memory_format == torch.contiguous_format:
+        if not impl.channels_last:
+            return impl
+        s = impl.sizes
+        as_nhwc = NestedTensorImpl(impl.buffer, torch.stack([s[:, 1], s[:, 2], s[:, 0]], 1).contiguous())
+        as_nhwc._offsets_dev = impl._offsets_dev
+        out = transpose_nhwc_nchw(as_nhwc)
+        return impl.with_buffer(out.buffer, channels_last=False)
+    if memory_format == torch.channels_last:
+        if impl.channels_last:
+            return impl
+        if impl.dim() != 4:
+            raise RuntimeError("ChannelsLast memory format requires 4 dim input.")
+        if impl.buffer.numel() == 0:
+            return impl.with_buffer(impl.buffer, channels_last=True)
+        out = transpose_nchw_nhwc(impl)
+        return impl.with_buffer(out.buffer, channels_last=True)
+    raise RuntimeError("Given memory format " + str(memory_format) +
+                       " not supported by NestedTensor_contiguous.")

@@ -48,6 +48,9 @@ Pinning (what each part was checked against, see tests/test_oracle_*.py):
   that avoid the library call being restated (indexing, Python loops, the CSR
   ``to_dense`` check of test/test_nested_tensor_class.py:741-752, the
   ``pad_packed_sequence`` round trip); tests/test_oracle_interop.py.
+* to_channels_last / from_channels_last: torch's own
+  ``contiguous(memory_format=torch.channels_last)`` per constituent, values and
+  strides (test/test_nested_tensor_class.py:844-866), and the round trip.
 * add: ``torch.add`` on the packed buffers / per constituent
   (test/test_nested_tensor_functional.py's add cases reduce to it).
 
@@ -76,4 +79,5 @@ from .mha import min_mha, bt_min_mha  # noqa: F401
 from .rowops import layer_norm, add  # noqa: F401
 from .dense import max_pool2d, conv2d  # noqa: F401
 from .interop import (  # noqa: F401
-    embedding, embedding_bag, to_sparse_csr, to_packed_sequence, transpose_nchw_nhwc, transpose_nhwc_nchw)
+    embedding, embedding_bag, to_sparse_csr, to_packed_sequence, transpose_nchw_nhwc, transpose_nhwc_nchw,
+    to_channels_last, from_channels_last)

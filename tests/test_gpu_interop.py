@@ -135,3 +135,61 @@ def test_transpose_errors_and_irregular_channels():
         nt.transpose_nchw_nhwc(a)
     with pytest.raises(RuntimeError, match="transpose_nchw_nhwc needs 4d input."):
         nt.transpose_nchw_nhwc(nt.nested_tensor([torch.randn(2, 3)], device=DEV))
+
+
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.float16, torch.float32, torch.int64])
+def test_transpose_ragged_every_tile_shape(dtype):
+    """nt_transpose_ragged through the C ABI with each tile shape it accepts, on
+    matrices whose extents are not multiples of any of them (one is a single
+    row, one a single column)."""
+    from nestedtensor_amd import _C
+    from nestedtensor_amd.impl import device_offsets
+    shapes = [(1, 300), (300, 1), (64, 257), (130, 67), (255, 129), (7, 5)]
+    g = torch.Generator().manual_seed(21)
+    mats = [torch.randint(0, 200, s, generator=g).to(dtype) for s in shapes]
+    buf = torch.cat([m.reshape(-1) for m in mats]).to(DEV)
+    exp = torch.cat([m.t().contiguous().reshape(-1) for m in mats])
+    B = len(shapes)
+    rows = torch.tensor([s[0] for s in shapes], dtype=torch.int64)
+    cols = torch.tensor([s[1] for s in shapes], dtype=torch.int64)
+    offsets = device_offsets(torch.stack([rows, cols], 1).contiguous().to(DEV), B, 2)
+    eb = buf.element_size()
+    stream = _C.current_stream(DEV)
+    rows_d, cols_d = rows.to(DEV), cols.to(DEV)
+    for tr, tc in ((64, 64), (64, 128), (128, 64), (128, 128), (64, 256), (256, 64)):
+        tiles = ((rows + tr - 1) // tr) * ((cols + tc - 1) // tc)
+        toff = torch.zeros(B + 1, dtype=torch.int64)
+        toff[1:] = torch.cumsum(tiles, 0)
+        toff_d = toff.to(DEV)
+        out = torch.full_like(buf, 201 if dtype != torch.uint8 else 255)
+        rc = _C.lib.nt_transpose_ragged(_C.ptr(buf), _C.ptr(out), _C.ptr(offsets), _C.ptr(rows_d),
+                                        _C.ptr(cols_d), _C.ptr(toff_d), B, int(toff[B]), tr, tc, eb, stream)
+        if tr * tc * eb > 32768:
+            assert rc != 0 and b"tile" in _C.lib.nt_last_error()
+            continue
+        assert rc == 0, _C.lib.nt_last_error()
+        assert torch.equal(out.cpu(), exp), (tr, tc)
+    rc = _C.lib.nt_transpose_ragged(_C.ptr(buf), _C.ptr(out), _C.ptr(offsets), _C.ptr(rows_d),
+                                    _C.ptr(cols_d), _C.ptr(toff_d), B, 1, 32, 64, eb, stream)
+    assert rc != 0
+
+
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.float16, torch.float32, torch.int64])
+@pytest.mark.parametrize("narrow", [1, 3, 4, 7, 16])
+def test_transpose_ragged_strips(dtype, narrow):
+    """Images of a few channels take the strip kernels in both directions; the
+    long sides straddle one, two and many strips."""
+    strip = 2048 // torch.empty(0, dtype=dtype).element_size()
+    longs = [1, 65, strip - 1, strip, strip + 1, 2 * strip + 13, 5 * strip + 7]
+    g = torch.Generator().manual_seed(22)
+    for shapes in ([(narrow, n, 1) for n in longs], ):
+        ts = [torch.randint(0, 200, s, generator=g).to(dtype) for s in shapes]
+        a = nt.nested_tensor(ts, device=DEV, dtype=dtype)
+        from nestedtensor_amd import ops
+        assert ops._transpose_tile(narrow, max(longs), a.element_size()) == (16, strip)
+        assert ops._transpose_tile(max(longs), narrow, a.element_size()) == (strip, 16)
+        fwd = nt.transpose_nchw_nhwc(a)
+        exp = oracle.transpose_nchw_nhwc(oracle.ref_nested_tensor(ts, dtype=dtype))
+        assert torch.equal(fwd._impl.buffer.cpu(), exp.buffer)
+        back = nt.transpose_nhwc_nchw(fwd)
+        assert torch.equal(back._impl.buffer, a._impl.buffer)

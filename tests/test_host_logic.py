@@ -214,3 +214,35 @@ def test_mask_collapse_closed_form_matches_oracle():
             except RuntimeError as e:
                 got = str(e)
             assert got == exp, (parts and [p.shape for p in parts], md, got, exp)
+
+
+def test_channels_last_metadata_and_views():
+    """A channels-last impl over a host buffer: strides, is_contiguous and the
+    constituent views need no device work (nested_tensor_impl.cpp:182-194,
+    Packed.h:125-163)."""
+    from nestedtensor_amd.impl import NestedTensorImpl
+    from nestedtensor_amd.nested.nested import NestedTensor
+    import oracle
+    ts = [torch.randn(4, 3, 5), torch.randn(4, 2, 7)]
+    ref = oracle.ref_nested_tensor(ts)
+    buffer, strides = oracle.to_channels_last(ref)
+    a = NestedTensor(NestedTensorImpl(buffer, ref.sizes, channels_last=True))
+    assert a.is_contiguous(memory_format=torch.channels_last)
+    assert not a.is_contiguous()
+    assert a.nested_size() == nt.nested_tensor(ts).nested_size()
+    assert list(a.nested_stride()) == strides
+    assert a.nested_stride(1) == (1, 1) and a.nested_stride(3) == (4, 4)
+    for got, t in zip(a.unbind(), ts):
+        want = t.unsqueeze(0).contiguous(memory_format=torch.channels_last).squeeze(0)
+        assert got.stride() == want.stride() and torch.equal(got, t)
+    b = nt.nested_tensor(ts)
+    assert b.is_contiguous() and not b.is_contiguous(memory_format=torch.channels_last)
+    assert b.contiguous() is b and a.contiguous(memory_format=torch.channels_last) is a
+    with pytest.raises(RuntimeError, match="not supported"):
+        b.is_contiguous(memory_format=torch.channels_last_3d)
+    with pytest.raises(RuntimeError, match="requires 4 dim input"):
+        NestedTensorImpl(torch.zeros(6), torch.tensor([[2, 3]]), channels_last=True)
+    with pytest.raises(RuntimeError, match="runs on the HIP device only"):
+        b.contiguous(memory_format=torch.channels_last)
+    with pytest.raises(RuntimeError, match="requires 4 dim input"):
+        nt.nested_tensor([torch.randn(2, 3)]).contiguous(memory_format=torch.channels_last)

@@ -72,3 +72,39 @@ def test_transposes_are_inverse_permutations():
     assert torch.equal(back.buffer, nt.buffer)
     with pytest.raises(RuntimeError, match="Expected first dimension to be regular."):
         oracle.transpose_nchw_nhwc(oracle.ref_nested_tensor([torch.randn(2, 3, 3), torch.randn(3, 3, 3)]))
+
+
+def _images(seed=1010, n=7, c=30):
+    # shapes of the reference's case (test/test_nested_tensor_class.py:852-856)
+    import random
+    rnd = random.Random(seed)
+    shapes = [(c, rnd.randint(20, 40), rnd.randint(20, 40)) for _ in range(n)]
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randn(*s, generator=g) for s in shapes]
+
+
+def test_channels_last_storage_is_torch_channels_last_per_constituent():
+    ts = _images()
+    nt = oracle.ref_nested_tensor(ts)
+    buffer, strides = oracle.to_channels_last(nt)
+    off = 0
+    for t, st in zip(ts, strides):
+        want = t.unsqueeze(0).contiguous(memory_format=torch.channels_last).squeeze(0)
+        assert tuple(want.stride()) == st
+        got = torch.as_strided(buffer, t.shape, st, off)
+        assert torch.equal(got, t) and torch.equal(got, want)
+        # the storage order itself: [H, W, C] row-major
+        assert torch.equal(buffer[off:off + t.numel()], t.permute(1, 2, 0).reshape(-1))
+        off += t.numel()
+    assert off == buffer.numel()
+
+
+def test_channels_last_round_trip():
+    ts = _images(seed=3, n=4, c=5)
+    nt = oracle.ref_nested_tensor(ts)
+    buffer, _ = oracle.to_channels_last(nt)
+    back = oracle.from_channels_last(buffer, nt._shapes, nt.dtype)
+    assert torch.equal(back.buffer, nt.buffer)
+    assert [tuple(t.shape) for t in back.unbind()] == [tuple(t.shape) for t in ts]
+    with pytest.raises(RuntimeError, match="requires 4 dim input"):
+        oracle.to_channels_last(oracle.ref_nested_tensor([torch.randn(3, 4), torch.randn(2, 4)]))
