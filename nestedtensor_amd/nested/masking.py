@@ -259,12 +259,8 @@ def _from_rows(tensor, mask_dims, count_rows, byte_mask):
     if bool((extents.prod(1) != total).any()):
         raise RuntimeError("stack expects each tensor to be equal size: the mask does not select "
                            "a rectangular block in every constituent.")
-    shapes = []
-    for b in range(B):
-        if int(total[b]) == 0:
-            shapes.append(list(inner_mask_shape[:-1]) + [0])
-        else:
-            shapes.append([int(v) for v in extents[b]] + rest)
+    empty_shape = list(inner_mask_shape[:-1]) + [0]
+    shapes = [e + rest if t else empty_shape for t, e in zip(total.tolist(), extents.tolist())]
     if leading:
         # Every constituent keeps a leading box: this is the length-based un-pad
         # (nt_remove_padding) with the nested size just derived.
