@@ -379,9 +379,10 @@ def bench_rows(args, torch, dev):
         cp = oracle.to_padded_tensor(ref, -1e30)
         c_pad = _time_cpu(lambda: oracle.to_padded_tensor(ref, 0), 3)
         c_back = _time_cpu(lambda: oracle.from_padded_tensor(cp, ref), 3)
+        c_val = _time_cpu(lambda: oracle.nt_from_tensor_mask_vectorised(cp, cp != -1e30), 3)
     rows["C1_to_padded_tensor"] = entry(ms_pad, 4 * (nvalid + npadded), c_pad)
     rows["C1_nested_tensor_from_padded_tensor"] = entry(
-        ms_back, 4 * (npadded + 2 * nvalid), None,
+        ms_back, 4 * (npadded + 2 * nvalid), c_val if cpu else None,
         note="value-based; includes the device-to-host copy of the row counts")
     rows["C1_from_padded_tensor_length_based"] = entry(ms_len, 4 * 2 * nvalid, c_back)
 
@@ -401,19 +402,21 @@ def bench_rows(args, torch, dev):
     ms_pack = _time_gpu(torch, lambda: nt.nested_tensor(dev_imgs, device=dev), iters=10)
     back2 = nt.nested_tensor_from_tensor_mask(data, mask)
     assert torch.equal(back2._impl.buffer, a2._impl.buffer)
-    c_tm = c_fm = None
+    c_tm = c_fm = c_m = c_pack = None
     if cpu:
         ref2 = oracle.ref_nested_tensor(imgs)
         c_tm = _time_cpu(lambda: oracle.to_tensor_mask(ref2), 1)
         dcpu, mcpu = data.cpu(), mask.cpu()
         c_fm = _time_cpu(lambda: oracle.nt_from_tensor_mask_vectorised(dcpu, mcpu), 1)
+        c_m = _time_cpu(lambda: oracle.to_mask(ref2, 4), 1)
+        c_pack = _time_cpu(lambda: oracle.ref_nested_tensor(imgs), 1)
     rows["C2_to_tensor_mask"] = entry(ms_tm, 4 * (nvalid2 + npadded2) + npadded2, c_tm)
-    rows["C2_to_mask"] = entry(ms_m, npadded2)
+    rows["C2_to_mask"] = entry(ms_m, npadded2, c_m)
     rows["C2_nested_tensor_from_tensor_mask"] = entry(
         ms_fm, npadded2 + 2 * 4 * nvalid2, c_fm,
         note="includes the device-to-host copy of the row counts; CPU figure is the vectorised "
              "restatement, the reference's literal walk does one host call per mask element")
-    rows["C2_nested_tensor_pack_from_device_tensors"] = entry(ms_pack, 2 * 4 * nvalid2)
+    rows["C2_nested_tensor_pack_from_device_tensors"] = entry(ms_pack, 2 * 4 * nvalid2, c_pack)
 
     # ---- metadata scan --------------------------------------------------------
     sizes = torch.randint(1, 2049, (4096, 2), dtype=torch.int64).to(dev)
@@ -435,14 +438,19 @@ def bench_rows(args, torch, dev):
         ms_ln = _time_gpu(torch, lambda: _ops.layer_norm(x_rw, (E_rw,), w_rw, b_rw, 1e-5))
         ms_rln = _time_gpu(torch, lambda: _ops.layer_norm(x_rw, (E_rw,), w_rw, b_rw, 1e-5, residual=r_rw))
         ms_add = _time_gpu(torch, lambda: _ops.add(x_rw, r_rw))
-        c_ln = None
+        c_ln = c_rln = c_add = None
         if cpu and tag == "C3":
-            parts_rw = [p.reshape(L, E_rw) for p, L in zip(buf.cpu().split([L * E_rw for L in lens_rw]), lens_rw)]
-            ref_rw = oracle.ref_nested_tensor(parts_rw, dtype=torch.float16)
-            c_ln = _time_cpu(lambda: oracle.layer_norm(ref_rw, (E_rw,), w_rw.cpu(), b_rw.cpu(), 1e-5), 2)
+            def _split(t):
+                return [p.reshape(L, E_rw) for p, L in zip(t.cpu().split([L * E_rw for L in lens_rw]), lens_rw)]
+            ref_rw = oracle.ref_nested_tensor(_split(buf), dtype=torch.float16)
+            ref_res = oracle.ref_nested_tensor(_split(r_rw.buffer), dtype=torch.float16)
+            w_c, b_c = w_rw.cpu(), b_rw.cpu()
+            c_ln = _time_cpu(lambda: oracle.layer_norm(ref_rw, (E_rw,), w_c, b_c, 1e-5), 2)
+            c_add = _time_cpu(lambda: oracle.add(ref_rw, ref_res), 2)
+            c_rln = _time_cpu(lambda: oracle.layer_norm(oracle.add(ref_rw, ref_res), (E_rw,), w_c, b_c, 1e-5), 2)
         rows[tag + "_layer_norm_fp16"] = entry(ms_ln, 2 * nb, c_ln, rows=T_rw, width=E_rw)
-        rows[tag + "_residual_layer_norm_fp16"] = entry(ms_rln, 3 * nb, None, rows=T_rw, width=E_rw)
-        rows[tag + "_packed_add_fp16"] = entry(ms_add, 3 * nb, None, rows=T_rw, width=E_rw)
+        rows[tag + "_residual_layer_norm_fp16"] = entry(ms_rln, 3 * nb, c_rln, rows=T_rw, width=E_rw)
+        rows[tag + "_packed_add_fp16"] = entry(ms_add, 3 * nb, c_add, rows=T_rw, width=E_rw)
         del buf, x_rw, r_rw
 
     # ---- interop formats built from the offsets array ------------------------------
@@ -457,16 +465,19 @@ def bench_rows(args, torch, dev):
     ms_bag = _time_gpu(torch, lambda: torch.nn.functional.embedding_bag(a_ids, table, mode="sum"))
     x_io = torch.nn.functional.embedding(a_ids, table)
     ms_ps = _time_gpu(torch, lambda: x_io.to_packed_sequence())
-    c_emb = c_ps = None
+    c_emb = c_ps = c_bag = None
     if cpu:
         ref_ids = oracle.ref_nested_tensor(ids_io, dtype=torch.int64)
         tcpu = table.cpu()
         c_emb = _time_cpu(lambda: oracle.embedding(tcpu, ref_ids), 2)
+        tcpu32 = tcpu.float()
+        c_bag = _time_cpu(lambda: oracle.embedding_bag(ref_ids, tcpu32, "sum"), 2)
         ref_x = oracle.ref_nested_tensor([p.cpu() for p in x_io.unbind()], dtype=torch.float16)
         c_ps = _time_cpu(lambda: oracle.to_packed_sequence(ref_x), 2)
     rows["C3_embedding_fp16"] = entry(ms_emb, T_io * (8 + 2 * 2 * E_io), c_emb,
                                       note="includes the device-to-host read of the out-of-range counter")
-    rows["C3_embedding_bag_sum_fp16"] = entry(ms_bag, T_io * (8 + 2 * E_io) + 32 * 2 * E_io)
+    rows["C3_embedding_bag_sum_fp16"] = entry(ms_bag, T_io * (8 + 2 * E_io) + 32 * 2 * E_io, c_bag,
+                                              note="CPU figure on an fp32 table (torch's CPU embedding_bag has no fp16 path)")
     rows["C3_to_packed_sequence_fp16"] = entry(ms_ps, T_io * (8 + 2 * 2 * E_io), c_ps)
     big_T, big_E = 1 << 20, 1024
     big_idx = torch.randint(V_io, (big_T,), device=dev)
@@ -492,6 +503,18 @@ def bench_rows(args, torch, dev):
     assert torch.equal(_ops.transpose_nhwc_nchw(nhwc).buffer, buf_t)
     rows["C2x64ch_transpose_nchw_nhwc_fp16"] = entry(ms_t0, 2 * 2 * buf_t.numel())
     rows["C2x64ch_transpose_nhwc_nchw_fp16"] = entry(ms_t1, 2 * 2 * buf_t.numel())
+    if cpu:
+        # CPU side on the first two images (GB/s does not depend on the count)
+        n2 = int(sizes_t[:2].prod(1).sum())
+        parts_t = [p.reshape(tuple(int(v) for v in sz)) for p, sz in
+                   zip(buf_t[:n2].cpu().split([int(v) for v in sizes_t[:2].prod(1)]), sizes_t[:2])]
+        ref_t = oracle.ref_nested_tensor(parts_t, dtype=torch.float16)
+        ref_nhwc = oracle.transpose_nchw_nhwc(ref_t)
+        for key, fn in (("C2x64ch_transpose_nchw_nhwc_fp16", lambda: oracle.transpose_nchw_nhwc(ref_t)),
+                        ("C2x64ch_transpose_nhwc_nchw_fp16", lambda: oracle.transpose_nhwc_nchw(ref_nhwc))):
+            c_ms = _time_cpu(fn, 2)
+            rows[key]["cpu_oracle_GBps"] = 2 * 2 * n2 / (c_ms * 1e-3) / 1e9
+            rows[key]["cpu_oracle_sample"] = "first 2 of 16 images, %.1f ms" % c_ms
     # 1x1 convolution 64 -> 256 channels: row-major input (transpose, GEMM, transpose)
     # against the channels-last storage of the same images (the GEMM alone)
     w11 = (torch.randn(256, 64, 1, 1, device=dev) * 0.1).half()
@@ -504,6 +527,15 @@ def bench_rows(args, torch, dev):
                       ("C2x64ch_conv2d_1x1_to_256ch_channels_last_fp16", ms_c1)):
         rows[key] = entry(ms_c, conv_bytes, None, pixels=pix)
         rows[key]["tflops"] = 2.0 * pix * 64 * 256 / (ms_c * 1e-3) / 1e12
+    if cpu:
+        h0, w0 = int(sizes_t[0, 1]), int(sizes_t[0, 2])
+        x0 = buf_t[:64 * h0 * w0].reshape(64, h0, w0).float().cpu()
+        ref_c = oracle.ref_nested_tensor([x0], dtype=torch.float32)
+        w_c = w11.float().cpu()
+        c_ms = _time_cpu(lambda: oracle.conv2d(ref_c, w_c), 1)
+        for key in ("C2x64ch_conv2d_1x1_to_256ch_fp16", "C2x64ch_conv2d_1x1_to_256ch_channels_last_fp16"):
+            rows[key]["cpu_oracle_tflops"] = 2.0 * h0 * w0 * 64 * 256 / (c_ms * 1e-3) / 1e12
+            rows[key]["cpu_oracle_sample"] = "first of 16 images in fp32, %.1f ms" % c_ms
     del buf_t, img, nhwc, img_cl, w11
 
     # ---- C4: bt_min_mha bf16, high raggedness ---------------------------------
