@@ -250,10 +250,12 @@ int nt_ragged_arange(const int64_t* offsets, int64_t B, int64_t max_len, int64_t
  * of a nested tensor of 1-D index tensors and offsets is its offsets array: the
  * reference builds the same offsets in a host loop and calls torch.embedding_bag
  * (nestedtensor/nested/nested.py:43-118).  Indices out of range are skipped and
- * counted in *oob_count if it is not NULL. */
+ * counted in *oob_count if it is not NULL.  num_indices = offsets[B], the length
+ * of indices, as the host knows it: it only sizes the workgroups (bags of 64
+ * indices or more on average get 16 wavefronts each instead of 4). */
 int nt_embedding_bag(const void* weight, int64_t ldw, int64_t num_embeddings, const int64_t* indices,
-                     const int64_t* offsets, void* out, int64_t B, int64_t n, int mode, int dtype,
-                     int32_t* oob_count, void* stream);
+                     int64_t num_indices, const int64_t* offsets, void* out, int64_t B, int64_t n,
+                     int mode, int dtype, int32_t* oob_count, void* stream);
 
 /* Per-constituent 2-D transpose on the packed buffer: constituent b, a row-major
  * [rows[b], cols[b]] matrix at element offset offsets[b], is written as its

@@ -128,18 +128,22 @@ __global__ __launch_bounds__(64) void embedding_bag_kernel(
 }
 
 // Rows of whole, aligned 16-byte pieces: a lane owns 8 (16-bit) or 4 (32-bit)
-// consecutive columns, the four wavefronts of a workgroup take every fourth token
-// of the bag with kAhead rows in flight each, and the partial results are combined
-// through LDS (so sums are formed in a different order than a sequential loop).
-template <typename T>
-__global__ __launch_bounds__(256) void embedding_bag_vec_kernel(
+// consecutive columns, the kBagWaves wavefronts of a workgroup take blocks of
+// kAhead tokens of the bag in turn, all kAhead rows in flight at once, and the
+// partial results are combined through LDS in wavefront order (so sums are formed
+// in a different order than a sequential loop, but always in the same one).  A
+// bag is a chain of index -> row loads, so what it costs is the number of such
+// rounds: 16 wavefronts x 8 rows cover a few hundred tokens in two or three; short
+// bags get 4 wavefronts.
+template <typename T, int kBagWaves>
+__global__ __launch_bounds__(kBagWaves * 64) void embedding_bag_vec_kernel(
     const T* __restrict__ weight, int64_t ldw, int64_t num_embeddings,
     const int64_t* __restrict__ indices, const int64_t* __restrict__ offsets, T* __restrict__ out,
     int64_t n, int mode, int32_t* __restrict__ oob) {
   constexpr int kPer = 16 / sizeof(T);
   constexpr int kAhead = 8;
-  __shared__ float part[4][kWave][kPer];
-  __shared__ int any_row[4];
+  __shared__ float part[kBagWaves][kWave][kPer];
+  __shared__ int any_row[kBagWaves];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int64_t b = blockIdx.x;
@@ -150,7 +154,7 @@ __global__ __launch_bounds__(256) void embedding_bag_vec_kernel(
 #pragma unroll
   for (int j = 0; j < kPer; ++j) acc[j] = 0.0f;
   bool first = true;
-  for (int64_t t0 = begin + wave * kAhead; t0 < end; t0 += 4 * kAhead) {
+  for (int64_t t0 = begin + wave * kAhead; t0 < end; t0 += kBagWaves * kAhead) {
     u32x4 raw[kAhead];
     bool use[kAhead];
 #pragma unroll
@@ -190,7 +194,7 @@ __global__ __launch_bounds__(256) void embedding_bag_vec_kernel(
 #pragma unroll
   for (int e = 0; e < kPer; ++e) res[e] = 0.0f;
 #pragma unroll
-  for (int w = 0; w < 4; ++w) {
+  for (int w = 0; w < kBagWaves; ++w) {
     if (!any_row[w]) continue;   // uniform
 #pragma unroll
     for (int e = 0; e < kPer; ++e) {
@@ -287,9 +291,10 @@ extern "C" int nt_ragged_arange(const int64_t* offsets, int64_t B, int64_t max_l
 }
 
 extern "C" int nt_embedding_bag(const void* weight, int64_t ldw, int64_t num_embeddings,
-                                const int64_t* indices, const int64_t* offsets, void* out, int64_t B,
-                                int64_t n, int mode, int dtype, int32_t* oob_count, void* stream) {
-  if (B < 0 || n < 0 || num_embeddings < 0 || ldw < n) {
+                                const int64_t* indices, int64_t num_indices, const int64_t* offsets,
+                                void* out, int64_t B, int64_t n, int mode, int dtype,
+                                int32_t* oob_count, void* stream) {
+  if (B < 0 || n < 0 || num_embeddings < 0 || ldw < n || num_indices < 0) {
     return fail(NT_ERR_INVALID_ARGUMENT, "embedding_bag: bad shape");
   }
   if (mode < 0 || mode > 2) return fail(NT_ERR_INVALID_ARGUMENT, "embedding_bag: mode %d", mode);
@@ -304,11 +309,18 @@ extern "C" int nt_embedding_bag(const void* weight, int64_t ldw, int64_t num_emb
   const int64_t per = 16 / elem;
   const bool vec = n % per == 0 && ldw % per == 0 && (uintptr_t)weight % 16 == 0 && (uintptr_t)out % 16 == 0;
   dim3 grid((unsigned)B, (unsigned)(vec ? (n / per + 63) / 64 : (n + 63) / 64));
+  const bool long_bags = num_indices >= 64 * B;     // 64 tokens per bag or more on average
 #define NT_BAG_CASE(TYPE)                                                                         \
   if (vec) {                                                                                      \
-    hipLaunchKernelGGL((embedding_bag_vec_kernel<TYPE>), grid, dim3(256), 0, s,                   \
-                       static_cast<const TYPE*>(weight), ldw, num_embeddings, indices, offsets,   \
-                       static_cast<TYPE*>(out), n, mode, oob_count);                              \
+    if (long_bags) {                                                                              \
+      hipLaunchKernelGGL((embedding_bag_vec_kernel<TYPE, 16>), grid, dim3(16 * 64), 0, s,         \
+                         static_cast<const TYPE*>(weight), ldw, num_embeddings, indices, offsets, \
+                         static_cast<TYPE*>(out), n, mode, oob_count);                            \
+    } else {                                                                                      \
+      hipLaunchKernelGGL((embedding_bag_vec_kernel<TYPE, 4>), grid, dim3(4 * 64), 0, s,           \
+                         static_cast<const TYPE*>(weight), ldw, num_embeddings, indices, offsets, \
+                         static_cast<TYPE*>(out), n, mode, oob_count);                            \
+    }                                                                                             \
   } else {                                                                                        \
     hipLaunchKernelGGL((embedding_bag_kernel<TYPE>), grid, dim3(64), 0, s,                        \
                        static_cast<const TYPE*>(weight), ldw, num_embeddings, indices, offsets,   \
@@ -336,10 +348,8 @@ extern "C" int nt_embedding_bag(const void* weight, int64_t ldw, int64_t num_emb
 // through LDS, so that both the reads and the writes are contiguous per
 // wavefront; tile_offsets[b] = number of tiles of all constituents before b, and
 // a workgroup finds its constituent by binary search.  The caller picks the tile
-// shape: 64 x 64 in general, and a tile that is longer along the long side of a
-// narrow matrix (the [C, H*W] / [H*W, C] matrices of images have C of 64 or so),
-// so that the strided side moves 256 or 512 contiguous bytes per row of the tile
-// instead of 128.
+// shape; 64 x 64 keeps the most workgroups in flight and is the fastest on image
+// shapes, the taller and wider ones move longer contiguous pieces per tile row.
 namespace nt {
 
 constexpr int kTrMaxTileBytes = 32 * 1024;

@@ -677,7 +677,8 @@ def embedding_bag(input, weight, offsets=None, max_norm=None, norm_type=2, scale
     out = torch.empty((B, E), dtype=weight.dtype, device=weight.device)
     oob = torch.zeros(1, dtype=torch.int32, device=weight.device)
     with torch.cuda.device(weight.device):
-        _C.check(_C.lib.nt_embedding_bag(_C.ptr(weight), E, V, _C.ptr(idx64), _C.ptr(input.offsets_dev()),
+        _C.check(_C.lib.nt_embedding_bag(_C.ptr(weight), E, V, _C.ptr(idx64), idx64.numel(),
+                                         _C.ptr(input.offsets_dev()),
                                          _C.ptr(out), B, E, modes[mode], _C.dtype_code(weight.dtype),
                                          _C.ptr(oob), _C.current_stream(weight.device)))
     _raise_if_oob(oob, "embedding_bag")
