@@ -214,6 +214,16 @@ int nt_layer_norm(const void* x, const void* residual, const void* gamma, const 
 int nt_add_packed(const void* a, const void* b, double alpha, void* out, int64_t numel,
                   int64_t period, int dtype, void* stream);
 
+/* out[i] = scale * a[i] * b[i % period] in fp32, rounded once; b == NULL gives
+ * out[i] = scale * a[i] (period is then ignored).  period == numel: nested *
+ * nested of equal nested size; period == last-dim size: nested * 1-D vector;
+ * b == NULL: nested * scalar, the q * scaling step of min_mha.  Replaces the
+ * per-constituent at::mul of NestedTensor_mul_Tensor
+ * (nestedtensor/csrc/BinaryOps.cpp:241-300, call site nestedtensor/csrc/mha.cpp:46)
+ * by one launch over the packed buffer. */
+int nt_mul_packed(const void* a, const void* b, double scale, void* out, int64_t numel,
+                  int64_t period, int dtype, void* stream);
+
 /* ---- consumers of the offsets array (interop formats) ------------------- */
 
 /* dst row r = src row index[r]; rows of row_bytes bytes, src has src_rows rows.

@@ -1,10 +1,11 @@
 // Row-wise ops on the packed token buffer of a nested tensor (gfx950): layer
 // normalisation over the (regular) last dim, with an optional residual input, and
-// the two packed additions of the reference (nested + nested of equal nested
-// size, nested + 1-D vector over the last dim).  A nested tensor [B, L_i, n] is
+// the packed additions and multiplications of the reference (nested with nested
+// of equal nested size, nested with a 1-D vector over the last dim, nested times
+// a scalar).  A nested tensor [B, L_i, n] is
 // one contiguous [T, n] matrix here, so none of these needs the nested size:
 // they are the per-constituent at::layer_norm / at::add of the reference
-// (nestedtensor/csrc/functions.cpp:65-112, BinaryOps.cpp:18-44, 97-107) done in
+// (nestedtensor/csrc/functions.cpp:65-112, BinaryOps.cpp:18-44, 97-107, 241-300) done in
 // one launch over all constituents.  All are HBM-bound: every input element is
 // read once and every output element written once.
 //
@@ -209,33 +210,45 @@ static int launch_layer_norm(const void* x, const void* residual, const void* ga
   return check_launch("layer_norm_rows_generic_kernel");
 }
 
-// out[i] = a[i] + alpha * b[i % period]   (period == numel: plain packed add)
-template <typename T, bool VEC>
+// OP 0: out[i] = a[i] + alpha * b[i % period]   (period == numel: plain packed add)
+// OP 1: out[i] = alpha * a[i] * b[i % period], or alpha * a[i] when b is NULL
+enum { kBinAdd = 0, kBinMul = 1 };
+
+template <int OP>
+__device__ __forceinline__ float bin_op(float a, float b, float alpha, bool has_b) {
+  if (OP == kBinAdd) return a + alpha * b;
+  return has_b ? alpha * (a * b) : alpha * a;
+}
+
+template <typename T, bool VEC, int OP>
 __global__ __launch_bounds__(256) void add_kernel(const T* __restrict__ a, const T* __restrict__ b,
                                                   float alpha, T* __restrict__ out, int64_t numel,
                                                   int64_t period) {
   constexpr int kPer = VEC ? 16 / sizeof(T) : 1;
+  const bool has_b = b != nullptr;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x * kPer;
   for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * kPer; i < numel; i += stride) {
     if (VEC) {
       // period is a multiple of kPer here, so a piece never wraps
       const u32x4 ra = *reinterpret_cast<const u32x4*>(a + i);
-      const u32x4 rb = *reinterpret_cast<const u32x4*>(b + (period == numel ? i : i % period));
+      u32x4 rb = ra;
+      if (has_b) rb = *reinterpret_cast<const u32x4*>(b + (period == numel ? i : i % period));
       T va[kPer], vb[kPer], vo[kPer];
       __builtin_memcpy(va, &ra, 16);
       __builtin_memcpy(vb, &rb, 16);
 #pragma unroll
-      for (int j = 0; j < kPer; ++j) vo[j] = (T)((float)va[j] + alpha * (float)vb[j]);
+      for (int j = 0; j < kPer; ++j) vo[j] = (T)bin_op<OP>((float)va[j], (float)vb[j], alpha, has_b);
       u32x4 o;
       __builtin_memcpy(&o, vo, 16);
       store16_stream(reinterpret_cast<char*>(out + i), o);
     } else {
-      out[i] = (T)((float)a[i] + alpha * (float)b[period == numel ? i : i % period]);
+      const float fb = has_b ? (float)b[period == numel ? i : i % period] : 0.0f;
+      out[i] = (T)bin_op<OP>((float)a[i], fb, alpha, has_b);
     }
   }
 }
 
-template <typename T>
+template <typename T, int OP>
 static int launch_add(const void* a, const void* b, double alpha, void* out, int64_t numel,
                       int64_t period, hipStream_t stream) {
   constexpr int kPer = 16 / sizeof(T);
@@ -248,10 +261,10 @@ static int launch_add(const void* a, const void* b, double alpha, void* out, int
   const T* pb = static_cast<const T*>(b);
   T* po = static_cast<T*>(out);
   if (vec) {
-    hipLaunchKernelGGL((add_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, stream, pa, pb,
+    hipLaunchKernelGGL((add_kernel<T, true, OP>), dim3((unsigned)blocks), dim3(256), 0, stream, pa, pb,
                        (float)alpha, po, numel, period);
   } else {
-    hipLaunchKernelGGL((add_kernel<T, false>), dim3((unsigned)blocks), dim3(256), 0, stream, pa, pb,
+    hipLaunchKernelGGL((add_kernel<T, false, OP>), dim3((unsigned)blocks), dim3(256), 0, stream, pa, pb,
                        (float)alpha, po, numel, period);
   }
   return check_launch("add_kernel");
@@ -286,9 +299,28 @@ extern "C" int nt_add_packed(const void* a, const void* b, double alpha, void* o
   if (!a || !b || !out) return fail(NT_ERR_INVALID_ARGUMENT, "add_packed: NULL pointer");
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case NT_F32: return launch_add<float>(a, b, alpha, out, numel, period, s);
-    case NT_F16: return launch_add<_Float16>(a, b, alpha, out, numel, period, s);
-    case NT_BF16: return launch_add<__bf16>(a, b, alpha, out, numel, period, s);
+    case NT_F32: return launch_add<float, kBinAdd>(a, b, alpha, out, numel, period, s);
+    case NT_F16: return launch_add<_Float16, kBinAdd>(a, b, alpha, out, numel, period, s);
+    case NT_BF16: return launch_add<__bf16, kBinAdd>(a, b, alpha, out, numel, period, s);
     default: return fail(NT_ERR_UNSUPPORTED, "add_packed: dtype %d is not f32, f16 or bf16", dtype);
+  }
+}
+
+extern "C" int nt_mul_packed(const void* a, const void* b, double scale, void* out, int64_t numel,
+                             int64_t period, int dtype, void* stream) {
+  if (numel < 0 || period < 0) return fail(NT_ERR_INVALID_ARGUMENT, "mul_packed: negative extent");
+  if (numel == 0) return NT_OK;
+  if (!b) period = numel;
+  if (period == 0 || numel % period != 0) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "mul_packed: numel %lld is not a multiple of the period %lld",
+                (long long)numel, (long long)period);
+  }
+  if (!a || !out) return fail(NT_ERR_INVALID_ARGUMENT, "mul_packed: NULL pointer");
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case NT_F32: return launch_add<float, kBinMul>(a, b, scale, out, numel, period, s);
+    case NT_F16: return launch_add<_Float16, kBinMul>(a, b, scale, out, numel, period, s);
+    case NT_BF16: return launch_add<__bf16, kBinMul>(a, b, scale, out, numel, period, s);
+    default: return fail(NT_ERR_UNSUPPORTED, "mul_packed: dtype %d is not f32, f16 or bf16", dtype);
   }
 }

@@ -282,6 +282,22 @@ class NestedTensor:
     def add(self, other, *, alpha=1):
         return torch.add(self, other, alpha=alpha)
 
+    # --- packed element-wise mul (BinaryOps.cpp:241-300), packed matmul (matmul.cpp:13-41) ---
+    def __mul__(self, other):
+        return torch.mul(self, other)
+
+    def __rmul__(self, other):
+        return torch.mul(self, other)
+
+    def mul(self, other):
+        return torch.mul(self, other)
+
+    def __matmul__(self, other):
+        return torch.matmul(self, other)
+
+    def matmul(self, other):
+        return torch.matmul(self, other)
+
     # --- dispatch ---
     @classmethod
     def __torch_function__(cls, func, types, args=(), kwargs=None):
@@ -336,6 +352,14 @@ def _add(input, other, *, alpha=1, out=None):
             raise NotImplementedError("tensor + alpha * nested is not on the packed path.")
         input, other = other, input
     return ops.add(input, other, alpha)
+
+
+def _mul(input, other, *, out=None):
+    if out is not None:
+        raise NotImplementedError("mul on a NestedTensor does not take out=.")
+    if not isinstance(input, NestedTensorImpl):      # tensor * nested, scalar * nested
+        input, other = other, input
+    return ops.mul(input, other)
 
 
 def _to_tensor_list(impl):
@@ -401,12 +425,19 @@ _HANDLERS = {
     torch.Tensor.add: _add,
     torch.Tensor.__add__: _add,
     torch.Tensor.__radd__: _add,
+    torch.mul: _mul,
+    torch.Tensor.mul: _mul,
+    torch.Tensor.__mul__: _mul,
+    torch.Tensor.__rmul__: _mul,
+    torch.matmul: ops.matmul,
+    torch.Tensor.matmul: ops.matmul,
+    torch.Tensor.__matmul__: ops.matmul,
 }
 
 # handlers that look at the storage layout themselves (or only at the nested
 # size); every other handler is given row-major operands
 _LAYOUT_AWARE = {
     _to_tensor_list, _get_max_size, _is_nested_tensor_impl, _nested_dim, _sizes, _len, _get_dim, _get_numel,
-    ops.is_contiguous, ops.contiguous, ops.conv2d, ops.max_pool2d, _add,
+    ops.is_contiguous, ops.contiguous, ops.conv2d, ops.max_pool2d, _add, _mul,
     ops.transpose_nchw_nhwc, ops.transpose_nhwc_nchw,
 }

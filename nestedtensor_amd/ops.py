@@ -511,6 +511,56 @@ def add(impl, other, alpha=1):
     return impl.with_buffer(out)
 
 
+def mul(impl, other):
+    """NestedTensor_mul_Tensor on the packed buffer (BinaryOps.cpp:241-300): nested
+    * scalar (the q * scaling step of min_mha, mha.cpp:46), nested * nested of
+    equal nested size, nested * 1-D tensor over a regular last dim."""
+    _C.require_device(impl.buffer, "mul")
+    b, period, scale = None, 0, 1.0
+    if isinstance(other, NestedTensorImpl):
+        if other.sizes.shape != impl.sizes.shape or not torch.equal(other.sizes, impl.sizes):
+            raise NotImplementedError("mul of nested tensors of different nested size is not on the packed path.")
+        if not (impl.channels_last and other.channels_last):
+            impl, other = contiguous(impl), contiguous(other)
+        b, period = other.buffer, impl.buffer.numel()
+    elif isinstance(other, (int, float)) or (isinstance(other, torch.Tensor) and other.dim() == 0):
+        scale = float(other)            # the layout does not matter
+    elif isinstance(other, torch.Tensor) and other.dim() == 1:
+        impl = contiguous(impl)
+        opt = impl.opt_sizes()
+        if opt[impl.dim() - 1] is None or opt[impl.dim() - 1] != other.size(0):
+            raise NotImplementedError("mul by a 1-D tensor needs a regular last dim of the same size.")
+        b, period = other.contiguous(), other.size(0)
+    else:
+        raise NotImplementedError("mul: only nested * scalar, nested * nested (same nested size) and "
+                                  "nested * 1-D tensor are on the packed path.")
+    buf = impl.buffer
+    if b is not None and (b.dtype != buf.dtype or b.device != buf.device):
+        raise RuntimeError("mul: both operands must have the same dtype and device")
+    out = torch.empty_like(buf)
+    if buf.numel() > 0:
+        with torch.cuda.device(buf.device):
+            _C.check(_C.lib.nt_mul_packed(_C.ptr(buf), _C.ptr(b), scale, _C.ptr(out), buf.numel(), period,
+                                          _C.dtype_code(buf.dtype), _C.current_stream(buf.device)))
+    return impl.with_buffer(out)
+
+
+def matmul(impl, other):
+    """NestedTensor_matmul, packed fast path (matmul.cpp:13-41): a nested tensor
+    [B, L_i, K] times a dense [K, N] matrix is one GEMM over the packed [T, K]
+    buffer.  nt_linear wants the weight K-contiguous, so `other` is transposed
+    first (a copy of K * N elements)."""
+    if isinstance(other, NestedTensorImpl) or not isinstance(impl, NestedTensorImpl):
+        raise NotImplementedError("matmul: only nested [B, L_i, K] x dense [K, N] is on the packed path.")
+    opt = impl.opt_sizes()
+    if impl.dim() != 3 or other.dim() != 2 or opt[2] is None or opt[2] != other.size(0):
+        raise NotImplementedError("matmul: only nested [B, L_i, K] x dense [K, N] is on the packed path.")
+    out = linear(impl.buffer.reshape(-1, opt[2]), other.t().contiguous(), None)
+    sizes = impl.sizes.clone()
+    sizes[:, 1] = other.size(1)
+    return NestedTensorImpl(out.reshape(-1), sizes)
+
+
 # ---- dense ops called through pad -> op -> un-pad (pooling.cpp:41-57, conv2d.cpp:77-92) ----
 
 def _pair(v):

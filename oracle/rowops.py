@@ -57,3 +57,19 @@ def add(nt, other, alpha=1):
     else:
         outs = [torch.add(a, other, alpha=alpha) for a in nt.unbind()]
     return RefNestedTensor(outs, nt.dtype)
+
+
+def mul(nt, other):
+    """NestedTensor_mul_Tensor (BinaryOps.cpp:296-299): at::mul per constituent;
+    `other` a nested tensor of the same nested size, a scalar, or a tensor that
+    broadcasts against every constituent."""
+    if isinstance(other, RefNestedTensor):
+        outs = [torch.mul(a, b) for a, b in zip(nt.unbind(), other.unbind())]
+    else:
+        outs = [torch.mul(a, other) for a in nt.unbind()]
+    return RefNestedTensor(outs, nt.dtype)
+
+
+def matmul(nt, other):
+    """NestedTensor_matmul (matmul.cpp:44-49): at::matmul per constituent."""
+    return RefNestedTensor([torch.matmul(a, other) for a in nt.unbind()], nt.dtype)

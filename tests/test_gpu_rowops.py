@@ -93,6 +93,52 @@ def test_add_nested_and_vector(dtype):
         a + odd
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_mul_scalar_nested_and_vector(dtype):
+    # BinaryOps.cpp:241-300; one rounding of an fp32 product: bit-exact against at::mul
+    shapes = [(3, 40), (7, 40), (1, 40)]
+    ta, tb = _tensors(shapes, dtype, 1), _tensors(shapes, dtype, 2)
+    a, b = nt.nested_tensor(ta, device=DEV, dtype=dtype), nt.nested_tensor(tb, device=DEV, dtype=dtype)
+    ra, rb = oracle.ref_nested_tensor(ta, dtype=dtype), oracle.ref_nested_tensor(tb, dtype=dtype)
+    assert torch.equal((a * b)._impl.buffer.cpu(), oracle.mul(ra, rb).buffer)
+    assert torch.equal(torch.mul(a, b)._impl.buffer.cpu(), oracle.mul(ra, rb).buffer)
+    for sc in (0.125, 3, -1.7):                                   # 0.125 = the head_dim 64 scaling of min_mha
+        assert torch.equal((a * sc)._impl.buffer.cpu(), oracle.mul(ra, sc).buffer)
+        assert torch.equal((sc * a)._impl.buffer.cpu(), oracle.mul(ra, sc).buffer)
+    v = torch.randn(40, generator=torch.Generator().manual_seed(3)).to(dtype)
+    assert torch.equal((a * v.to(DEV))._impl.buffer.cpu(), oracle.mul(ra, v).buffer)
+    assert torch.equal((v.to(DEV) * a)._impl.buffer.cpu(), oracle.mul(ra, v).buffer)
+    odd_t = _tensors([(3, 7), (2, 7)], dtype, 4)                      # unaligned rows
+    odd = nt.nested_tensor(odd_t, device=DEV, dtype=dtype)
+    ro = oracle.ref_nested_tensor(odd_t, dtype=dtype)
+    v7 = torch.arange(7.0).to(dtype)
+    assert torch.equal((odd * v7.to(DEV))._impl.buffer.cpu(), oracle.mul(ro, v7).buffer)
+    assert torch.equal((odd * 0.3)._impl.buffer.cpu(), oracle.mul(ro, 0.3).buffer)
+    with pytest.raises(NotImplementedError):
+        a * odd
+    with pytest.raises(NotImplementedError):
+        a * torch.ones(3, 40, device=DEV, dtype=dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_matmul_packed_fast_path(dtype):
+    # matmul.cpp:13-41: nested [B, L_i, K] x dense [K, N] is one GEMM on the packed buffer
+    K, N = 64, 96
+    ts = _tensors([(5, K), (130, K), (1, K)], dtype, 7)
+    w = (torch.randn(K, N, generator=torch.Generator().manual_seed(8)) * 0.2).to(dtype)
+    a = nt.nested_tensor(ts, device=DEV, dtype=dtype)
+    got = torch.matmul(a, w.to(DEV))
+    assert (a @ w.to(DEV)).nested_size() == got.nested_size()
+    ref = oracle.matmul(oracle.ref_nested_tensor([t.float() for t in ts], dtype=torch.float32), w.float())
+    assert [tuple(x.shape) for x in got.unbind()] == [tuple(x.shape) for x in ref.unbind()]
+    err = (got._impl.buffer.float().cpu() - ref.buffer).abs().max().item()
+    assert err <= (1e-5 if dtype == torch.float32 else 2e-2) * max(1.0, ref.buffer.abs().max().item()), err
+    with pytest.raises(NotImplementedError):
+        torch.matmul(a, torch.randn(K + 1, N, device=DEV).to(dtype))
+    with pytest.raises(NotImplementedError):
+        torch.matmul(a, a)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_residual_layer_norm_equals_two_ops(dtype):
     # ops.layer_norm(x, residual=r) == layer_norm(x + r): the sum is rounded to the

@@ -76,3 +76,20 @@ def test_dense_ops_output_sizes_closed_form():
     for t, o in zip(nt.unbind(), got.unbind()):
         exp = ((t.shape[1] + 2 - 2 * 1 - 1) // 1 + 1, (t.shape[2] + 0 - 1 * 1 - 1) // 2 + 1)
         assert tuple(o.shape) == (5,) + exp
+
+
+def test_mul_and_matmul_known_answers():
+    a = oracle.ref_nested_tensor([torch.tensor([[1.0, 2.0], [3.0, 4.0]]), torch.tensor([[5.0, 6.0]])])
+    b = oracle.ref_nested_tensor([torch.tensor([[2.0, 2.0], [0.5, -1.0]]), torch.tensor([[0.0, 1.0]])])
+    assert oracle.mul(a, b).buffer.tolist() == [2.0, 4.0, 1.5, -4.0, 0.0, 6.0]
+    assert oracle.mul(a, 0.5).buffer.tolist() == [0.5, 1.0, 1.5, 2.0, 2.5, 3.0]
+    assert oracle.mul(a, torch.tensor([10.0, -1.0])).buffer.tolist() == [10.0, -2.0, 30.0, -4.0, 50.0, -6.0]
+    w = torch.tensor([[1.0, 0.0, 2.0], [0.0, 1.0, -1.0]])              # [K=2, N=3]
+    got = oracle.matmul(a, w)
+    assert got.opt_sizes() == [2, None, 3]
+    assert got.buffer.tolist() == [1.0, 2.0, 0.0, 3.0, 4.0, 2.0, 5.0, 6.0, 4.0]
+    # against an fp64 product of the packed buffer (matmul.cpp:13-41: the fast path is one GEMM)
+    x = _nt([(3, 8), (5, 8)], seed=5)
+    w8 = torch.randn(8, 6, generator=torch.Generator().manual_seed(6))
+    ref = (x.buffer.reshape(-1, 8).double() @ w8.double()).reshape(-1)
+    assert (oracle.matmul(x, w8).buffer.double() - ref).abs().max() < 1e-5
