@@ -453,6 +453,23 @@ def bench_rows(args, torch, dev):
         rows[tag + "_packed_add_fp16"] = entry(ms_add, 3 * nb, c_add, rows=T_rw, width=E_rw)
         del buf, x_rw, r_rw
 
+    # ---- softmax over the ragged last dim: the [H, L_i, L_i] score blocks of C3 -------
+    g = torch.Generator().manual_seed(1010 + 2)
+    lens_sm = [int(v) for v in torch.randint(32, 513, (32,), generator=g)]
+    sizes_sm = torch.tensor([[12, L, L] for L in lens_sm], dtype=torch.int64)
+    buf_sm = torch.randn(int(sizes_sm.prod(1).sum()), device=dev, dtype=torch.float16)
+    from nestedtensor_amd.impl import NestedTensorImpl as _ImplSm
+    x_sm = _ImplSm(buf_sm, sizes_sm)
+    ms_sm = _time_gpu(torch, lambda: _ops.softmax(x_sm, -1))
+    c_sm = None
+    if cpu:
+        parts_sm = [p.reshape(12, L, L) for p, L in zip(buf_sm.cpu().split([12 * L * L for L in lens_sm]), lens_sm)]
+        ref_sm = oracle.ref_nested_tensor(parts_sm, dtype=torch.float16)
+        c_sm = _time_cpu(lambda: oracle.softmax(ref_sm, -1), 2)
+    rows["C3_scores_softmax_fp16"] = entry(ms_sm, 2 * 2 * buf_sm.numel(), c_sm, rows=int((sizes_sm[:, 0] * sizes_sm[:, 1]).sum()),
+                                           note="what the fused attention kernel never writes: the per-sequence score blocks")
+    del buf_sm, x_sm
+
     # ---- interop formats built from the offsets array ------------------------------
     g = torch.Generator().manual_seed(1010 + 2)
     lens_io = [int(v) for v in torch.randint(32, 513, (32,), generator=g)]

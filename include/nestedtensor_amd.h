@@ -214,6 +214,20 @@ int nt_layer_norm(const void* x, const void* residual, const void* gamma, const 
 int nt_add_packed(const void* a, const void* b, double alpha, void* out, int64_t numel,
                   int64_t period, int dtype, void* stream);
 
+/* Softmax (log_softmax != 0: log-softmax) over the last dim of every constituent
+ * of a nested tensor, on the packed buffer: constituent b has row_offsets[b + 1]
+ * - row_offsets[b] rows of (offsets[b + 1] - offsets[b]) / rows elements each at
+ * element offset offsets[b]; the row length may differ between constituents (a
+ * ragged last dim, the [H, L_i, L_i] scores of per-sequence attention).  fp32
+ * arithmetic, one rounding.  One launch for the per-constituent at::softmax of
+ * NestedTensor_softmax / NestedTensor_log_softmax
+ * (nestedtensor/csrc/SoftMax.cpp:12-46, call site nestedtensor/csrc/mha.cpp:58);
+ * it is also the masked row softmax of the reference's GPU path
+ * (nestedtensor/csrc/cuda/attention.cu:229-304) without the padding.  offsets and
+ * row_offsets are int64[B + 1] on the device; total_rows = row_offsets[B]. */
+int nt_softmax_rows(const void* x, void* out, const int64_t* offsets, const int64_t* row_offsets,
+                    int64_t B, int64_t total_rows, int log_softmax, int dtype, void* stream);
+
 /* out[i] = scale * a[i] * b[i % period] in fp32, rounded once; b == NULL gives
  * out[i] = scale * a[i] (period is then ignored).  period == numel: nested *
  * nested of equal nested size; period == last-dim size: nested * 1-D vector;

@@ -57,6 +57,7 @@ SIGNATURES = {
     "nt_layer_norm": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _f64, _int,
                              _c_void_p]),
     "nt_add_packed": (_int, [_c_void_p, _c_void_p, _f64, _c_void_p, _i64, _i64, _int, _c_void_p]),
+    "nt_softmax_rows": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _int, _int, _c_void_p]),
     "nt_mul_packed": (_int, [_c_void_p, _c_void_p, _f64, _c_void_p, _i64, _i64, _int, _c_void_p]),
     "nt_gather_rows": (_int, [_c_void_p, _i64, _i64, _c_void_p, _c_void_p, _i64, _c_void_p, _c_void_p]),
     "nt_packed_sequence_index": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _c_void_p]),

@@ -44,20 +44,6 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(
   }
 }
 
-// b with offsets[b] <= i < offsets[b + 1] (offsets non-decreasing, offsets[B] > i)
-__device__ __forceinline__ int64_t find_segment(const int64_t* offsets, int64_t B, int64_t i) {
-  int64_t lo = 0, hi = B;   // answer in [lo, hi)
-  while (hi - lo > 1) {
-    const int64_t mid = (lo + hi) >> 1;
-    if (offsets[mid] <= i) {
-      lo = mid;
-    } else {
-      hi = mid;
-    }
-  }
-  return lo;
-}
-
 // Time-major order of a PackedSequence: token t of the sequence at sorted
 // position r goes to row step_starts[t] + r.  index_out[that row] = source row.
 __global__ __launch_bounds__(256) void packed_sequence_index_kernel(

@@ -210,6 +210,170 @@ static int launch_layer_norm(const void* x, const void* residual, const void* ga
   return check_launch("layer_norm_rows_generic_kernel");
 }
 
+// Softmax (or log-softmax) over the last dim of every constituent.  Constituent b
+// holds row_offsets[b + 1] - row_offsets[b] rows of equal length at element
+// offset offsets[b]; the length differs between constituents when the last dim
+// is ragged (the [H, L_i, L_i] score blocks of per-sequence attention).  One
+// wavefront per row: it finds its constituent by binary search and keeps a row
+// of up to 256 8-byte pieces (1024 16-bit or 512 32-bit elements) in registers;
+// longer rows take three passes (maximum, sum of exponentials, result), the last
+// two from cache.  fp32 arithmetic, one rounding, like at::softmax.
+// exp(x) for x <= 0 through the hardware's 2^x: the argument's rounding adds a
+// relative error of |x| * 1e-7 at most, and exp(x) is negligible long before that
+// matters
+__device__ __forceinline__ float fast_exp(float x) {
+  return __builtin_amdgcn_exp2f(x * 1.4426950408889634f);
+}
+
+// one row of n elements, by one wavefront
+template <typename T, bool LOG>
+__device__ __forceinline__ void softmax_row(const T* __restrict__ src, T* __restrict__ dst, int64_t n,
+                                            int lane) {
+  constexpr int V = 8 / (int)sizeof(T);      // elements per 8-byte piece
+  constexpr int kCache = 4;                  // pieces a lane keeps in registers
+  const int64_t pieces = (n + V - 1) / V;
+  if (pieces <= kWave * kCache) {
+    // the row fits the wavefront's registers: one read, one write, 8 bytes per
+    // lane and access at any alignment (rows of odd length start anywhere)
+    float v[kCache][V];
+    float m = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < kCache; ++k) {
+      const int64_t i0 = (int64_t)(lane + k * kWave) * V;
+      if ((int64_t)k * kWave * V >= n) {             // uniform: nobody has elements in this slot
+#pragma unroll
+        for (int j = 0; j < V; ++j) v[k][j] = -INFINITY;
+        continue;
+      }
+      if (i0 + V <= n) {
+        T t[V];
+        __builtin_memcpy(t, src + i0, 8);
+#pragma unroll
+        for (int j = 0; j < V; ++j) v[k][j] = (float)t[j];
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j) v[k][j] = i0 + j < n ? (float)src[i0 + j] : -INFINITY;
+      }
+#pragma unroll
+      for (int j = 0; j < V; ++j) m = fmaxf(m, v[k][j]);
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, kWave));
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < kCache; ++k) {
+      if ((int64_t)k * kWave * V >= n) break;
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        const float e = fast_exp(v[k][j] - m);   // exp(-inf) = 0 for the slots past the row
+        s += e;
+        if (!LOG) v[k][j] = e;
+      }
+    }
+    s = wave_sum<T>(s);
+    const float inv = 1.0f / s, ls = logf(s);
+#pragma unroll
+    for (int k = 0; k < kCache; ++k) {
+      if ((int64_t)k * kWave * V >= n) break;
+      const int64_t i0 = (int64_t)(lane + k * kWave) * V;
+      T t[V];
+#pragma unroll
+      for (int j = 0; j < V; ++j) t[j] = (T)(LOG ? v[k][j] - m - ls : v[k][j] * inv);
+      if (i0 + V <= n) {
+        __builtin_memcpy(dst + i0, t, 8);
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+          if (i0 + j < n) dst[i0 + j] = t[j];
+      }
+    }
+    return;
+  }
+  // longer rows: three passes in 8-byte pieces, the second and third from cache
+  const int64_t whole = n / V;                       // pieces without a tail
+  float m = -INFINITY;
+  for (int64_t p = lane; p < whole; p += kWave) {
+    T t[V];
+    __builtin_memcpy(t, src + p * V, 8);
+#pragma unroll
+    for (int j = 0; j < V; ++j) m = fmaxf(m, (float)t[j]);
+  }
+  for (int64_t i = whole * V + lane; i < n; i += kWave) m = fmaxf(m, (float)src[i]);
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, kWave));
+  float s = 0.0f;
+  for (int64_t p = lane; p < whole; p += kWave) {
+    T t[V];
+    __builtin_memcpy(t, src + p * V, 8);
+#pragma unroll
+    for (int j = 0; j < V; ++j) s += fast_exp((float)t[j] - m);
+  }
+  for (int64_t i = whole * V + lane; i < n; i += kWave) s += fast_exp((float)src[i] - m);
+  s = wave_sum<T>(s);
+  const float inv = 1.0f / s, ls = logf(s);
+  for (int64_t p = lane; p < whole; p += kWave) {
+    T t[V];
+    __builtin_memcpy(t, src + p * V, 8);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      const float f = (float)t[j];
+      t[j] = (T)(LOG ? f - m - ls : fast_exp(f - m) * inv);
+    }
+    __builtin_memcpy(dst + p * V, t, 8);
+  }
+  for (int64_t i = whole * V + lane; i < n; i += kWave) {
+    const float f = (float)src[i];
+    dst[i] = (T)(LOG ? f - m - ls : fast_exp(f - m) * inv);
+  }
+}
+
+// One wavefront per row.  The two offset arrays are copied into LDS first when
+// they fit (the search for the row's constituent is then a chain of LDS reads
+// instead of global ones: the kernel is latency-bound on short rows).
+constexpr int kSoftmaxMeta = 1024;
+
+template <typename T, bool LOG>
+__global__ __launch_bounds__(256) void softmax_rows_kernel(
+    const T* __restrict__ x, T* __restrict__ out, const int64_t* __restrict__ offsets,
+    const int64_t* __restrict__ row_offsets, int64_t B, int64_t total_rows) {
+  __shared__ int64_t s_rows[kSoftmaxMeta], s_offs[kSoftmaxMeta];
+  const int64_t* ro = row_offsets;
+  const int64_t* eo = offsets;
+  if (B + 1 <= kSoftmaxMeta) {                       // uniform over the grid
+    for (int i = threadIdx.x; i <= B; i += 256) {
+      s_rows[i] = row_offsets[i];
+      s_offs[i] = offsets[i];
+    }
+    __syncthreads();
+    ro = s_rows;
+    eo = s_offs;
+  }
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t r = (int64_t)blockIdx.x * (256 / kWave) + (threadIdx.x / kWave);
+  if (r >= total_rows) return;                       // after the only barrier
+  const int64_t b = find_segment(ro, B, r);
+  const int64_t first = ro[b], rows_b = ro[b + 1] - first;
+  if (rows_b <= 0) return;                           // total_rows beyond row_offsets[B]: nothing to do
+  const int64_t base = eo[b];
+  const int64_t n = (eo[b + 1] - base) / rows_b;
+  softmax_row<T, LOG>(x + base + (r - first) * n, out + base + (r - first) * n, n, lane);
+}
+
+template <typename T>
+static int launch_softmax(const void* x, void* out, const int64_t* offsets, const int64_t* row_offsets,
+                          int64_t B, int64_t total_rows, int log_softmax, hipStream_t stream) {
+  const int64_t blocks = (total_rows + 3) / 4;
+  if (blocks > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "softmax_rows: too many rows");
+  if (log_softmax) {
+    hipLaunchKernelGGL((softmax_rows_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                       static_cast<const T*>(x), static_cast<T*>(out), offsets, row_offsets, B, total_rows);
+  } else {
+    hipLaunchKernelGGL((softmax_rows_kernel<T, false>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                       static_cast<const T*>(x), static_cast<T*>(out), offsets, row_offsets, B, total_rows);
+  }
+  return check_launch("softmax_rows_kernel");
+}
+
 // OP 0: out[i] = a[i] + alpha * b[i % period]   (period == numel: plain packed add)
 // OP 1: out[i] = alpha * a[i] * b[i % period], or alpha * a[i] when b is NULL
 enum { kBinAdd = 0, kBinMul = 1 };
@@ -285,6 +449,21 @@ extern "C" int nt_layer_norm(const void* x, const void* residual, const void* ga
     case NT_F16: return launch_layer_norm<_Float16>(x, residual, gamma, beta, out, rows, n, eps, s);
     case NT_BF16: return launch_layer_norm<__bf16>(x, residual, gamma, beta, out, rows, n, eps, s);
     default: return fail(NT_ERR_UNSUPPORTED, "layer_norm: dtype %d is not f32, f16 or bf16", dtype);
+  }
+}
+
+extern "C" int nt_softmax_rows(const void* x, void* out, const int64_t* offsets,
+                               const int64_t* row_offsets, int64_t B, int64_t total_rows,
+                               int log_softmax, int dtype, void* stream) {
+  if (B < 0 || total_rows < 0) return fail(NT_ERR_INVALID_ARGUMENT, "softmax_rows: negative extent");
+  if (B == 0 || total_rows == 0) return NT_OK;
+  if (!x || !out || !offsets || !row_offsets) return fail(NT_ERR_INVALID_ARGUMENT, "softmax_rows: NULL pointer");
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case NT_F32: return launch_softmax<float>(x, out, offsets, row_offsets, B, total_rows, log_softmax, s);
+    case NT_F16: return launch_softmax<_Float16>(x, out, offsets, row_offsets, B, total_rows, log_softmax, s);
+    case NT_BF16: return launch_softmax<__bf16>(x, out, offsets, row_offsets, B, total_rows, log_softmax, s);
+    default: return fail(NT_ERR_UNSUPPORTED, "softmax_rows: dtype %d is not f32, f16 or bf16", dtype);
   }
 }
 

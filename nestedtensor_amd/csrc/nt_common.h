@@ -48,4 +48,18 @@ __device__ __forceinline__ void store16_stream(char* p, u32x4 v) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
 }
 
+// b with offsets[b] <= i < offsets[b + 1] (offsets non-decreasing, offsets[B] > i)
+__device__ __forceinline__ int64_t find_segment(const int64_t* offsets, int64_t B, int64_t i) {
+  int64_t lo = 0, hi = B;   // answer in [lo, hi)
+  while (hi - lo > 1) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (offsets[mid] <= i) {
+      lo = mid;
+    } else {
+      hi = mid;
+    }
+  }
+  return lo;
+}
+
 }  // namespace nt

@@ -25,7 +25,7 @@ from . import _C
 
 class NestedTensorImpl:
     __slots__ = ("buffer", "sizes", "_opt_sizes", "_sizes_dev", "_offsets_dev",
-                 "_row_offsets_dev", "_max_sizes", "_attn_schedule", "channels_last")
+                 "_row_offsets_dev", "_max_sizes", "_attn_schedule", "_last_dim_rows", "channels_last")
 
     def __init__(self, buffer, sizes, channels_last=False):
         """buffer: 1-D contiguous tensor; sizes: CPU int64 [B, D], or 0-d for an
@@ -47,6 +47,7 @@ class NestedTensorImpl:
         self._row_offsets_dev = None
         self._max_sizes = None
         self._attn_schedule = None
+        self._last_dim_rows = None
 
     # ---- host metadata ----------------------------------------------------
     @property
@@ -133,6 +134,17 @@ class NestedTensorImpl:
             self._row_offsets_dev = device_offsets(first, self.B, 1)
         return self._row_offsets_dev
 
+    def last_dim_rows(self):
+        """(row_offsets, total_rows): int64 [B + 1] on the device, the number of
+        rows along the last dim (product of all other constituent dims) of the
+        constituents before b, and their total."""
+        if self._last_dim_rows is None:
+            rows = self.sizes[:, :-1].prod(1)
+            row_offsets = torch.zeros(self.B + 1, dtype=torch.int64)
+            row_offsets[1:] = torch.cumsum(rows, 0)
+            self._last_dim_rows = (row_offsets.to(self.buffer.device), int(row_offsets[-1]))
+        return self._last_dim_rows
+
     def attention_schedule(self, q_tile=128):
         """Work list of the self-attention kernel, built from the host copy of the
         nested size and cached on the device: int32 [n_work, 4] rows
@@ -166,6 +178,7 @@ class NestedTensorImpl:
             out._offsets_dev = self._offsets_dev
             out._row_offsets_dev = self._row_offsets_dev
             out._attn_schedule = self._attn_schedule
+            out._last_dim_rows = self._last_dim_rows
         return out
 
 

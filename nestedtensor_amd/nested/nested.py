@@ -292,6 +292,12 @@ class NestedTensor:
     def mul(self, other):
         return torch.mul(self, other)
 
+    def softmax(self, dim, dtype=None):
+        return torch.softmax(self, dim, dtype=dtype)
+
+    def log_softmax(self, dim, dtype=None):
+        return torch.log_softmax(self, dim, dtype=dtype)
+
     def __matmul__(self, other):
         return torch.matmul(self, other)
 
@@ -362,6 +368,18 @@ def _mul(input, other, *, out=None):
     return ops.mul(input, other)
 
 
+def _softmax(input, dim=None, _stacklevel=3, dtype=None):
+    if dim is None:
+        raise RuntimeError("softmax on a NestedTensor needs an explicit dim.")
+    return ops.softmax(input, dim, dtype, log=False)
+
+
+def _log_softmax(input, dim=None, _stacklevel=3, dtype=None):
+    if dim is None:
+        raise RuntimeError("log_softmax on a NestedTensor needs an explicit dim.")
+    return ops.softmax(input, dim, dtype, log=True)
+
+
 def _to_tensor_list(impl):
     return list(NestedTensor(impl).unbind())
 
@@ -425,6 +443,12 @@ _HANDLERS = {
     torch.Tensor.add: _add,
     torch.Tensor.__add__: _add,
     torch.Tensor.__radd__: _add,
+    torch.nn.functional.softmax: _softmax,
+    torch.softmax: _softmax,
+    torch.Tensor.softmax: _softmax,
+    torch.nn.functional.log_softmax: _log_softmax,
+    torch.log_softmax: _log_softmax,
+    torch.Tensor.log_softmax: _log_softmax,
     torch.mul: _mul,
     torch.Tensor.mul: _mul,
     torch.Tensor.__mul__: _mul,

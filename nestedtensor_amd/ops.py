@@ -511,6 +511,38 @@ def add(impl, other, alpha=1):
     return impl.with_buffer(out)
 
 
+def softmax(impl, dim, dtype=None, log=False):
+    """NestedTensor_softmax / NestedTensor_log_softmax (SoftMax.cpp:12-46) over the
+    last dim, which may be ragged, in one launch over the packed buffer
+    (nt_softmax_rows).  Other dims of the constituents are not on the packed
+    path; dim 0 is the nested dim and is refused like in the reference."""
+    name = "log_softmax" if log else "softmax"
+    nd = impl.dim()
+    if not -nd <= dim < nd:
+        raise IndexError("Dimension out of range (expected to be in range of [%d, %d], but got %d)"
+                         % (-nd, nd - 1, dim))
+    dim = dim % nd
+    if dim < impl.nested_dim():
+        raise RuntimeError("Cannot apply %s across nested dimensions %d" % (name, dim))
+    if dim != nd - 1:
+        raise NotImplementedError("%s on a NestedTensor: only the last dim is on the packed path." % name)
+    buf = impl.buffer
+    _C.require_device(buf, name)
+    if dtype is not None and dtype != buf.dtype:
+        buf = buf.to(dtype)
+        impl = impl.with_buffer(buf)
+    out = torch.empty_like(buf)
+    B, D = impl.B, impl.D
+    if buf.numel() == 0:
+        return impl.with_buffer(out)
+    row_offsets, total_rows = impl.last_dim_rows()
+    with torch.cuda.device(buf.device):
+        _C.check(_C.lib.nt_softmax_rows(_C.ptr(buf), _C.ptr(out), _C.ptr(impl.offsets_dev()),
+                                        _C.ptr(row_offsets), B, total_rows, 1 if log else 0,
+                                        _C.dtype_code(buf.dtype), _C.current_stream(buf.device)))
+    return impl.with_buffer(out)
+
+
 def mul(impl, other):
     """NestedTensor_mul_Tensor on the packed buffer (BinaryOps.cpp:241-300): nested
     * scalar (the q * scaling step of min_mha, mha.cpp:46), nested * nested of

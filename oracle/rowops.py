@@ -73,3 +73,15 @@ def mul(nt, other):
 def matmul(nt, other):
     """NestedTensor_matmul (matmul.cpp:44-49): at::matmul per constituent."""
     return RefNestedTensor([torch.matmul(a, other) for a in nt.unbind()], nt.dtype)
+
+
+def softmax(nt, dim, dtype=None, log=False):
+    """NestedTensor_softmax / NestedTensor_log_softmax (SoftMax.cpp:12-46):
+    at::softmax(t, dim - nested_dim) per constituent; dim 0 is refused."""
+    nd = nt.dim()
+    dim = dim % nd
+    if dim < 1:
+        raise RuntimeError("Cannot apply %s across nested dimensions %d" % ("log_softmax" if log else "softmax", dim))
+    fn = torch.log_softmax if log else torch.softmax
+    outs = [fn(t, dim - 1, dtype=dtype) for t in nt.unbind()]
+    return RefNestedTensor(outs, outs[0].dtype if outs else nt.dtype)

@@ -121,6 +121,36 @@ def test_mul_scalar_nested_and_vector(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("log", [False, True])
+def test_softmax_last_dim(dtype, log):
+    # SoftMax.cpp:12-46; the shapes: per-sequence attention scores [H, L_i, L_i] (ragged last dim),
+    # a regular last dim, 1-D constituents, rows longer than a wavefront, a single element
+    import torch.nn.functional as F
+    cases = [[(4, 5, 5), (4, 130, 130), (4, 1, 1)], [(3, 40), (7, 40)], [(9,), (300,), (1,)],
+             [(2, 1100), (3, 513)], [(2, 3, 1023), (2, 3, 1025)], [(2, 511), (1, 4097), (1, 9001)]]   # around the register-cached row limits
+    for k, shapes in enumerate(cases):
+        ts = [t * 3 for t in _tensors(shapes, dtype, 20 + k)]
+        a = nt.nested_tensor(ts, device=DEV, dtype=dtype)
+        fn = F.log_softmax if log else F.softmax
+        got = fn(a, -1)
+        ref = oracle.softmax(oracle.ref_nested_tensor([t.float() for t in ts], dtype=torch.float32), -1, log=log)
+        assert got.nested_size() == a.nested_size() and got.dtype == dtype
+        # probabilities are at most 1: absolute; log-probabilities reach -20 or so: relative to |value|
+        err = ((got._impl.buffer.float().cpu() - ref.buffer).abs() / ref.buffer.abs().clamp(min=1.0)).max().item()
+        assert err <= (1e-5 if dtype == torch.float32 else 2e-2), err
+        assert torch.equal((a.log_softmax(a.dim() - 1) if log else a.softmax(a.dim() - 1))._impl.buffer,
+                           got._impl.buffer)
+    a = nt.nested_tensor(_tensors([(2, 3, 4), (2, 5, 4)], dtype, 30), device=DEV, dtype=dtype)
+    with pytest.raises(RuntimeError, match="across nested dimensions 0"):
+        torch.softmax(a, 0)
+    with pytest.raises(NotImplementedError):
+        torch.softmax(a, 1)
+    if dtype != torch.float32 and not log:
+        up = torch.softmax(a, -1, dtype=torch.float32)          # at::softmax's dtype argument
+        assert up.dtype == torch.float32
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 def test_matmul_packed_fast_path(dtype):
     # matmul.cpp:13-41: nested [B, L_i, K] x dense [K, N] is one GEMM on the packed buffer
     K, N = 64, 96

@@ -93,3 +93,29 @@ def test_mul_and_matmul_known_answers():
     w8 = torch.randn(8, 6, generator=torch.Generator().manual_seed(6))
     ref = (x.buffer.reshape(-1, 8).double() @ w8.double()).reshape(-1)
     assert (oracle.matmul(x, w8).buffer.double() - ref).abs().max() < 1e-5
+
+
+def test_softmax_closed_forms():
+    import math
+    ts = [torch.randn(2, 3, 5, generator=torch.Generator().manual_seed(1)),
+          torch.randn(2, 4, 2, generator=torch.Generator().manual_seed(2))]      # ragged last dim
+    a = oracle.ref_nested_tensor(ts)
+    got = oracle.softmax(a, -1)
+    lg = oracle.softmax(a, 3, log=True)
+    for t, o, l in zip(ts, got.unbind(), lg.unbind()):
+        assert o.shape == t.shape
+        for h in range(t.size(0)):
+            for r in range(t.size(1)):
+                row = [float(v) for v in t[h, r]]
+                den = sum(math.exp(v) for v in row)
+                for c, v in enumerate(row):
+                    assert abs(float(o[h, r, c]) - math.exp(v) / den) < 1e-6
+                    assert abs(float(l[h, r, c]) - math.log(math.exp(v) / den)) < 1e-5
+        assert torch.allclose(o.sum(-1), torch.ones(t.shape[:-1]), atol=1e-6)
+    shifted = oracle.ref_nested_tensor([t + 3.0 for t in ts])
+    assert (oracle.softmax(shifted, -1).buffer - got.buffer).abs().max() < 1e-6
+    with pytest.raises(RuntimeError, match="Cannot apply softmax across nested dimensions 0"):
+        oracle.softmax(a, 0)
+    # dims other than the last follow at::softmax per constituent too (SoftMax.cpp:24-27)
+    other = oracle.softmax(a, 1)
+    assert torch.allclose(other.unbind()[0].sum(0), torch.ones(3, 5), atol=1e-6)
