@@ -5,8 +5,10 @@ import pytest
 import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-if ROOT not in sys.path:
-    sys.path.insert(0, ROOT)
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+for path in (ROOT, GOLDEN):
+    if path not in sys.path:
+        sys.path.insert(0, path)
 
 
 def pytest_configure(config):

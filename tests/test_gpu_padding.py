@@ -1,7 +1,7 @@
 """Parity of the HIP pack / pad / un-pad / mask path with the CPU oracle
 (bit-exact), through the product's Python surface down to the C ABI.  The cases
 mirror the reference's GPU-vs-CPU tests (test/test_nested_tensor_class.py:754-817)
-and replay its literal masking cases (tests/cases.py) on the device."""
+and replay its literal masking cases (tests/golden/masking_cases.py) on the device."""
 
 import random
 
@@ -12,7 +12,7 @@ import nestedtensor_amd as nt
 import oracle
 from nestedtensor_amd import _C
 from nestedtensor_amd.impl import device_offsets
-from cases import (TO_TENSOR_MASK, FROM_TENSOR_MASK, ROUND_TRIP_DATA, ROUND_TRIP_MASK)
+from masking_cases import (TO_TENSOR_MASK, FROM_TENSOR_MASK, ROUND_TRIP_DATA, ROUND_TRIP_MASK)
 
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda", 0)

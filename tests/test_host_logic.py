@@ -12,7 +12,7 @@ import torch
 
 import nestedtensor_amd as nt
 from nestedtensor_amd import _C
-from cases import FROM_TENSOR_MASK_ERRORS, TO_TENSOR_MASK_ERRORS
+from masking_cases import FROM_TENSOR_MASK_ERRORS, TO_TENSOR_MASK_ERRORS
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 

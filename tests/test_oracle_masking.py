@@ -1,5 +1,5 @@
 """Pins the CPU oracle for packing / padding / masks: replay of the reference's
-literal test cases (tests/cases.py), independent library cross-checks and
+literal test cases (tests/golden/masking_cases.py), independent library cross-checks and
 closed forms.  No GPU, no product code."""
 
 import random
@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import oracle
-from cases import (TO_TENSOR_MASK, TO_TENSOR_MASK_ERRORS, FROM_TENSOR_MASK,
+from masking_cases import (TO_TENSOR_MASK, TO_TENSOR_MASK_ERRORS, FROM_TENSOR_MASK,
                    FROM_TENSOR_MASK_ERRORS, ROUND_TRIP_DATA, ROUND_TRIP_MASK)
 
 
