@@ -354,6 +354,51 @@ def test_config_c2_images_tensor_mask_round_trip():
     nt_matches(back, parts, torch.float32)
 
 
+def test_config_c5_chunk_full_size_properties():
+    """One chunk of the largest configuration at its real shape: 512 fp16
+    constituents [L_i, 4096], L_i ~ U[1, 2048], generated on the device (more
+    than 2^31 packed elements, so every index is exercised as int64).  Checked
+    through properties that do not need the oracle at this size: the round trip
+    is bit-exact, every constituent's bits sum to the same value before and after
+    padding, the padding holds the pad value and nothing else, and three
+    constituents (first, longest, last) are compared element by element."""
+    from nestedtensor_amd.impl import NestedTensorImpl
+    from nestedtensor_amd.nested.nested import NestedTensor
+    g = torch.Generator().manual_seed(1010 + 4)
+    E = 4096
+    lens = torch.randint(1, 2049, (512,), generator=g)
+    sizes = torch.stack([lens, torch.full_like(lens, E)], 1).contiguous()
+    total = int(lens.sum()) * E
+    assert total > 2 ** 31
+    bits = torch.randint(-32768, 32767, (total,), device=DEV, dtype=torch.int16)     # any bit pattern
+    a = NestedTensor(NestedTensorImpl(bits.view(torch.float16), sizes))
+    Lmax = int(lens.max())
+    padded = torch.ops.nestedtensor.to_padded_tensor(a, float("nan"))
+    assert tuple(padded.shape) == (512, Lmax, E)
+    pview = padded.view(torch.int16)
+    # the canonical fp16 NaN the pad value converts to
+    nan_bits = int(torch.tensor(float("nan"), dtype=torch.float16).view(torch.int16))
+    # round trip
+    back = nt.from_padded_tensor(padded, a)
+    assert torch.equal(back._impl.buffer.view(torch.int16), bits)
+    # per-constituent checksums and pad region
+    starts = (torch.cumsum(lens, 0) - lens) * E
+    row_valid = torch.arange(Lmax, device=DEV).unsqueeze(0) < lens.to(DEV).unsqueeze(1)      # [512, Lmax]
+    row_sums = pview.sum(2, dtype=torch.int64)                                            # [512, Lmax]
+    got_valid = (row_sums * row_valid).sum(1)
+    cs = torch.zeros(total // E + 1, dtype=torch.int64, device=DEV)
+    cs[1:] = torch.cumsum(bits.view(-1, E).sum(1, dtype=torch.int64), 0)
+    tok = torch.cumsum(lens, 0).to(DEV)
+    exp_valid = cs[tok] - cs[tok - lens.to(DEV)]
+    assert torch.equal(got_valid, exp_valid)
+    pad_rows = ~row_valid
+    assert bool((pview[pad_rows] == nan_bits).all())
+    for b in (0, int(lens.argmax()), 511):
+        L, s0 = int(lens[b]), int(starts[b])
+        assert torch.equal(pview[b, :L].reshape(-1), bits[s0:s0 + L * E])
+    del padded, pview, back, row_sums
+
+
 # ---- row statistics kernels (C ABI level) -------------------------------------------
 
 def _cpu_counts_prefix(keep):
