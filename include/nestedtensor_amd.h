@@ -78,6 +78,19 @@ int nt_add_padding(const void* packed, void* padded, const int64_t* offsets,
                    const int64_t* padded_sizes_host, int elem_bytes, uint64_t pad_bits,
                    void* stream);
 
+/* nt_add_padding plus the mask of the same shape in one launch: mask[b, i...] = 1
+ * where padded[b, i...] holds data and 0 where it holds padding, one byte per
+ * element of padded (a bool tensor).  Replaces add_padding_mask_kernelLauncher
+ * (nestedtensor/csrc/cuda/padding.cu:217-262, called from to_tensor_mask,
+ * nestedtensor/csrc/masking.cpp:251-296), which covers 3-d nested tensors with a
+ * [B, L] mask only; this one covers the case where the mask keeps every dim of
+ * the data (no trailing regular dim to collapse, e.g. ragged images), the only
+ * case where the mask is large enough to matter.  Arguments as nt_add_padding. */
+int nt_add_padding_mask(const void* packed, void* padded, uint8_t* mask, const int64_t* offsets,
+                        const int64_t* sizes, int64_t B, int64_t D, int64_t n_ragged,
+                        const int64_t* padded_sizes_host, int elem_bytes, uint64_t pad_bits,
+                        void* stream);
+
 /* packed[offsets[b] + lin(i)] = padded[b, i] for i inside sizes[b]: the
  * length-based inverse of nt_add_padding.  Replaces
  * remove_padding_kernelLauncher<T> (nestedtensor/csrc/cuda/padding.h:36-45,

@@ -35,6 +35,8 @@ SIGNATURES = {
     "nt_offsets_from_sizes": (_int, [_c_void_p, _i64, _i64, _c_void_p, _c_void_p, _size_t, _c_void_p]),
     "nt_add_padding": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64,
                               ctypes.POINTER(_i64), _int, _u64, _c_void_p]),
+    "nt_add_padding_mask": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64,
+                                   ctypes.POINTER(_i64), _int, _u64, _c_void_p]),
     "nt_remove_padding": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64,
                                  ctypes.POINTER(_i64), _int, _c_void_p]),
     "nt_build_mask": (_int, [_c_void_p, _c_void_p, _i64, _i64, _i64, ctypes.POINTER(_i64), _c_void_p]),

@@ -43,7 +43,7 @@
 
 namespace nt {
 
-enum Mode { kPad = 0, kUnpad = 1, kOnes = 2, kPack = 3 };
+enum Mode { kPad = 0, kUnpad = 1, kOnes = 2, kPack = 3, kPadMask = 4 };
 
 struct RowParams {
   const char* src;
@@ -57,6 +57,7 @@ struct RowParams {
   int64_t inner;   // elements of the trailing regular dims
   int64_t nrows;
   u32x4 pad;       // padding value replicated to 16 bytes
+  char* mask;      // kPadMask: one byte per element of dst, 1 where the element holds data
 };
 
 template <int EB> struct ElemT;
@@ -211,8 +212,13 @@ __global__ __launch_bounds__(256) void row_kernel(RowParams p) {
     move_row<EB, kOnes, kT>(p.dst + row * row_bytes, nullptr, valid, row_bytes, p.pad);
   } else {
     const int64_t packed_byte = (p.offsets[b] + src_off * p.inner) * EB;
-    if (MODE == kPad) {
+    if (MODE == kPad || MODE == kPadMask) {
       move_row<EB, kPad, kT>(p.dst + row * row_bytes, p.src + packed_byte, valid, row_bytes, p.pad);
+      if (MODE == kPadMask) {
+        // the same workgroups write the row's mask bytes: ones over the valid prefix
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        move_row<1, kOnes, kT>(p.mask + row * (row_bytes / EB), nullptr, valid / EB, row_bytes / EB, zero);
+      }
     } else {
       if (valid > 0) {
         move_row<EB, kUnpad, kT>(p.dst + packed_byte, p.src + row * row_bytes, valid, valid, p.pad);
@@ -253,7 +259,8 @@ static int launch_rows_t(int eb, const RowParams& p, int64_t max_row_bytes, hipS
   // walked by a bounded number of workgroups that each loop over tiles.
   int64_t y_cap = (int64_t)NT_ROW_TARGET_WGS / grid_rows;
   if (y_cap < 1) y_cap = 1;
-  const int64_t max_tiles = (MODE == kPad || MODE == kOnes) ? NT_ROW_MAX_TILES_PAD : NT_ROW_MAX_TILES_UNPAD;
+  const int64_t max_tiles =
+      (MODE == kPad || MODE == kOnes || MODE == kPadMask) ? NT_ROW_MAX_TILES_PAD : NT_ROW_MAX_TILES_UNPAD;
   if (y_cap > max_tiles) y_cap = max_tiles;
   int64_t gy = tiles < y_cap ? tiles : y_cap;
   if (gy < 1) gy = 1;
@@ -331,6 +338,25 @@ extern "C" int nt_add_padding(const void* packed, void* padded, const int64_t* o
   p.sizes = sizes;
   p.pad = replicate_pad(elem_bytes, pad_bits);
   return launch_rows<kPad>(elem_bytes, p, max_row_elems * elem_bytes, (hipStream_t)stream);
+}
+
+extern "C" int nt_add_padding_mask(const void* packed, void* padded, uint8_t* mask,
+                                   const int64_t* offsets, const int64_t* sizes, int64_t B, int64_t D,
+                                   int64_t n_ragged, const int64_t* padded_sizes_host, int elem_bytes,
+                                   uint64_t pad_bits, void* stream) {
+  RowParams p = {};
+  int64_t max_row_elems = 0;
+  int rc = fill_geometry(p, B, D, n_ragged, padded_sizes_host, D, &max_row_elems);
+  if (rc != NT_OK) return rc;
+  if (B == 0 || max_row_elems == 0) return NT_OK;
+  if (!padded || !mask || !offsets || !sizes) return fail(NT_ERR_INVALID_ARGUMENT, "NULL pointer");
+  p.src = static_cast<const char*>(packed);
+  p.dst = static_cast<char*>(padded);
+  p.mask = reinterpret_cast<char*>(mask);
+  p.offsets = offsets;
+  p.sizes = sizes;
+  p.pad = replicate_pad(elem_bytes, pad_bits);
+  return launch_rows<kPadMask>(elem_bytes, p, max_row_elems * elem_bytes, (hipStream_t)stream);
 }
 
 extern "C" int nt_remove_padding(const void* padded, void* packed, const int64_t* offsets,

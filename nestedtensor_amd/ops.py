@@ -92,8 +92,10 @@ def _check_no_empty(impl):
 # packed -> padded
 
 
-def add_padding(impl, padding):
-    """Launch nt_add_padding: [B, max_1..max_D] from the packed buffer."""
+def add_padding(impl, padding, with_mask=False):
+    """Launch nt_add_padding: [B, max_1..max_D] from the packed buffer.  With
+    with_mask, nt_add_padding_mask writes the bool mask of the same shape in the
+    same launch and (padded, mask) is returned."""
     _C.require_device(impl.buffer, "to_padded_tensor")
     B, D = impl.B, impl.D
     max_size = impl.max_sizes()
@@ -104,6 +106,13 @@ def add_padding(impl, padding):
     eb = _elem_bytes(impl.buffer.dtype)
     dev = impl.buffer.device
     with torch.cuda.device(dev):
+        if with_mask:
+            mask = torch.empty([B] + max_size, dtype=torch.bool, device=dev)
+            _C.check(_C.lib.nt_add_padding_mask(
+                _C.ptr(impl.buffer), _C.ptr(out), _C.ptr(mask), _C.ptr(impl.offsets_dev()),
+                _C.ptr(impl.sizes_dev()), B, D, nrag, _C.i64_array(max_size), eb,
+                _pad_bits(padding, impl.buffer.dtype), _C.current_stream(dev)))
+            return out, mask
         _C.check(_C.lib.nt_add_padding(
             _C.ptr(impl.buffer), _C.ptr(out), _C.ptr(impl.offsets_dev()), _C.ptr(impl.sizes_dev()),
             B, D, nrag, _C.i64_array(max_size), eb, _pad_bits(padding, impl.buffer.dtype),
@@ -202,6 +211,10 @@ def to_tensor_mask(impl, mask_dim=None):
         raise RuntimeError("Internal error: Expected sizes_size_1 to be greater than 0.")
     _check_no_empty(impl)
     kept = _collapsed_mask_dims(impl, mask_dim)
+    if kept == impl.dim() and _n_ragged(impl) <= 3:
+        # nothing collapsed: the mask has the shape of the data and is written by
+        # the same launch (the fused kernel of padding.cu:217-262, generalised)
+        return add_padding(impl, 0, with_mask=True)
     data = add_padding(impl, 0)
     return data, build_mask(impl, kept)
 
