@@ -572,6 +572,38 @@ def bench_rows(args, torch, dev):
     rows["C4_bt_min_mha_bf16"] = dict(ms=ms4, tokens=T4, tokens_per_s=T4 / (ms4 * 1e-3), flops=fl4,
                                       TFLOPs=fl4 / (ms4 * 1e-3) / 1e12,
                                       frac_of_mfma_peak=fl4 / (ms4 * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS)
+
+    # ---- cross-attention: 100 queries per sequence over ragged memories (decoder-style) ----
+    g = torch.Generator().manual_seed(1010 + 5)
+    Ex, Hx = 512, 8
+    kv_lens = [int(v) for v in torch.randint(256, 1025, (32,), generator=g)]
+    qs = [torch.randn(100, Ex, generator=g).half() for _ in kv_lens]
+    mems = [torch.randn(L, Ex, generator=g).half() for L in kv_lens]
+    Wx_in = (torch.randn(3 * Ex, Ex, generator=g) * 0.03).half()
+    Wx_out = (torch.randn(Ex, Ex, generator=g) * 0.03).half()
+    bx_in, bx_out = torch.zeros(3 * Ex).half(), torch.zeros(Ex).half()
+    aq, am = nt.nested_tensor(qs, device=dev, dtype=torch.float16), nt.nested_tensor(mems, device=dev, dtype=torch.float16)
+    xargs = (Wx_in.to(dev), bx_in.to(dev), 64 ** -0.5, Wx_out.to(dev), bx_out.to(dev))
+    msx = _time_gpu(torch, lambda: torch.ops.nestedtensor.min_mha(Hx, 64, 0.0, False, aq, am, am, *xargs),
+                    iters=50, warmup=5)
+    Tq, Tk = 100 * len(kv_lens), sum(kv_lens)
+    flx = 2 * Ex * Ex * (2 * Tq + 2 * Tk) + 4 * Ex * 100 * Tk
+    rows["cross_attention_fp16"] = dict(
+        ms=msx, workload="B=32, 100 queries per sequence, memory L~U[256,1024], d=512, 8x64",
+        query_tokens=Tq, memory_tokens=Tk, flops=flx, TFLOPs=flx / (msx * 1e-3) / 1e12,
+        frac_of_mfma_peak=flx / (msx * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS)
+    if cpu:
+        rq, rm = oracle.ref_nested_tensor(qs, dtype=torch.float16), oracle.ref_nested_tensor(mems, dtype=torch.float16)
+        ref_out = None
+
+        def _cpu_cross():
+            nonlocal ref_out
+            ref_out = oracle.min_mha(Hx, 64, 0.0, False, rq, rm, rm, Wx_in, bx_in, 64 ** -0.5, Wx_out, bx_out)
+        rows["cross_attention_fp16"]["cpu_oracle_ms"] = _time_cpu(_cpu_cross, 1)
+        got = torch.ops.nestedtensor.min_mha(Hx, 64, 0.0, False, aq, am, am, *xargs)
+        exp = torch.cat([p.reshape(-1) for p in ref_out]).float()
+        rows["cross_attention_fp16"]["max_abs_err_vs_oracle"] = float(
+            (got._impl.buffer.float().cpu() - exp).abs().max())
     return rows
 
 

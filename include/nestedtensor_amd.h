@@ -189,19 +189,29 @@ int nt_linear_qkv(const void* A, int64_t lda, const void* W, const void* bias, v
                   int64_t ldqk, void* Vt, int64_t ldvt, int64_t M, int64_t E, int64_t K,
                   int dtype, void* stream);
 
-/* Self-attention (query, key and value are one nested tensor) on the output of
- * nt_linear_qkv: Q at column h*64 and K at column k_col + h*64 of QK, V^T in Vt;
- * head_dim is 64, dtype f16 or bf16.  `schedule` is a device array of n_work
- * int32[4] work items {first token of the sequence, sequence length, first query
- * row of the tile (multiple of 128), 0}: one per 128-query tile of every
- * sequence, in the order they should start (longest sequences first); a
+/* Ct[n][m] = (A[M, K] * W[N, K]^T + bias[N])[m][n]: nt_linear with the result
+ * written transposed (row stride ldct >= M).  The value projection of
+ * cross-attention (nestedtensor/csrc/mha.cpp:48-54, the `v` matmul and bias add)
+ * in the layout nt_varlen_attention_vt reads; it wants ldct >= M + 72. */
+int nt_linear_transposed(const void* A, int64_t lda, const void* W, const void* bias, void* Ct,
+                         int64_t ldct, int64_t M, int64_t N, int64_t K, int dtype, void* stream);
+
+/* Attention on projections in the layout the GEMMs above write: Q rows at
+ * q[token * ldq + h*64], K rows at k[token * ldk + h*64], V transposed in
+ * Vt[(h*64 + d) * ldvt + token]; head_dim is 64, dtype f16 or bf16.  For
+ * self-attention on the output of nt_linear_qkv, q = QK, k = QK + E, ldq = ldk =
+ * ldqk.  `schedule` is a device array of n_work int32[8] work items {first query
+ * token, query length, first query row of the tile (multiple of 128), 0, first
+ * key token, key length (>= 1), 0, 0}: one per 128-query tile of every sequence
+ * (for cross-attention: of every query sequence, with the key sequence it
+ * attends to), in the order they should start (longest key sequences first); a
  * workgroup is launched per (item, head), so no padded tile is ever issued.  The
- * rows of Vt must be readable up to 72 elements past the last token
- * (ldvt >= total_tokens + 72); what is stored there is ignored.  Output and
+ * rows of Vt must be readable up to 72 elements past the last key token
+ * (ldvt >= total_kv_tokens + 72); what is stored there is ignored.  Output and
  * semantics as nt_varlen_attention. */
-int nt_varlen_attention_vt(const void* qk, int64_t ldqk, int64_t k_col, const void* vt,
+int nt_varlen_attention_vt(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* vt,
                            int64_t ldvt, void* out, int64_t ldo, const int32_t* schedule,
-                           int64_t n_work, int64_t num_heads, int64_t total_tokens, float scale,
+                           int64_t n_work, int64_t num_heads, int64_t total_kv_tokens, float scale,
                            int dtype, void* stream);
 
 /* ---- row-wise ops on the packed buffer (the steps either side of attention

@@ -303,9 +303,9 @@ __global__ __launch_bounds__(256) void varlen_attention_kernel(
 
 template <typename T>
 __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt_kernel(
-    const T* __restrict__ QK, int64_t ldqk, int64_t k_col, const T* __restrict__ Vt, int64_t ldvt,
-    T* __restrict__ O, int64_t ldo, const int4* __restrict__ schedule, unsigned num_heads,
-    float scale_log2e) {
+    const T* __restrict__ Q, int64_t ldq, const T* __restrict__ K, int64_t ldk,
+    const T* __restrict__ Vt, int64_t ldvt, T* __restrict__ O, int64_t ldo,
+    const int4* __restrict__ schedule, unsigned num_heads, float scale_log2e) {
   typedef AttnT<T> AT;
   typedef typename AT::Frag Frag;
 
@@ -317,10 +317,16 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
   // item index fastest, the long items of the last heads would start last and
   // run alone at the end).
   const int h = (int)(blockIdx.x % num_heads);
-  const int4 item = schedule[blockIdx.x / num_heads];
-  const int64_t begin = item.x;
-  const int L = item.y;
+  // item: {first query token, query length, first query row of this tile, 0,
+  //        first key token, key length, 0, 0}; self-attention lists the same
+  //        sequence twice, cross-attention the two sequences of the pair
+  const int4 item = schedule[2 * (blockIdx.x / num_heads)];
+  const int4 item_kv = schedule[2 * (blockIdx.x / num_heads) + 1];
+  const int64_t q_begin = item.x;
+  const int Lq = item.y;
   const int q0 = item.z;
+  const int64_t begin = item_kv.x;   // of the keys
+  const int L = item_kv.y;           // number of keys
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -329,12 +335,12 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
   const int g = lane >> 5;
 
   const int q_row = q0 + wave * 32 + l32;
-  const bool wave_active = (q0 + wave * 32) < L;
+  const bool wave_active = (q0 + wave * 32) < Lq;
   Frag qf[4];
   {
-    // rows past L read the last row; their results are never stored
-    const int qr = q_row < L ? q_row : L - 1;
-    const T* qp = QK + (begin + qr) * ldqk + h * kHd + g * 8;
+    // rows past Lq read the last row; their results are never stored
+    const int qr = q_row < Lq ? q_row : Lq - 1;
+    const T* qp = Q + (q_begin + qr) * ldq + h * kHd + g * 8;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       u32x4 v = load16_unaligned(reinterpret_cast<const char*>(qp + s * 16));
@@ -350,7 +356,7 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
   float m_run = -INFINITY;
 
   const int ntiles = (L + kKTile - 1) / kKTile;
-  const T* kbase = QK + begin * ldqk + k_col + h * kHd;
+  const T* kbase = K + begin * ldk + h * kHd;
   const T* vbase = Vt + (int64_t)h * kHd * ldvt + begin;
 
   // Each thread moves two 16-byte pieces of a K tile and two of a V^T tile.
@@ -360,8 +366,8 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
   const int r0 = tid >> 3;      // row of piece 0 (piece 1: r0 + 32)
   const int cc = tid & 7;
   u32x4 rk[2], rv[2];
-  const char* k_last = reinterpret_cast<const char*>(kbase + (int64_t)(L - 1) * ldqk + cc * 8);
-  const int64_t k_step = (int64_t)kKTile * ldqk * (int64_t)sizeof(T);
+  const char* k_last = reinterpret_cast<const char*>(kbase + (int64_t)(L - 1) * ldk + cc * 8);
+  const int64_t k_step = (int64_t)kKTile * ldk * (int64_t)sizeof(T);
   const char* v_ptr[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
@@ -374,7 +380,7 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
     for (int i = 0; i < 2; ++i) {
       // rows past L read row L - 1 (a valid key: it cannot raise the row maximum)
       const int kr = t * kKTile + r0 + i * 32;
-      const char* src = tile + (int64_t)(r0 + i * 32) * ldqk * (int64_t)sizeof(T);
+      const char* src = tile + (int64_t)(r0 + i * 32) * ldk * (int64_t)sizeof(T);
       rk[i] = load16_unaligned(kr < L ? src : k_last);
     }
   };
@@ -548,10 +554,10 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
     __syncthreads();
   }
 
-  if (!wave_active || q_row >= L) return;
+  if (!wave_active || q_row >= Lq) return;
   const float l_tot = l_acc[0];
   const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
-  T* op = O + (begin + q_row) * ldo + h * kHd;
+  T* op = O + (q_begin + q_row) * ldo + h * kHd;
 #pragma unroll
   for (int db = 0; db < 2; ++db) {
 #pragma unroll
@@ -720,22 +726,22 @@ extern "C" int nt_varlen_attention(const void* q, int64_t ldq, const void* k, in
   }
 }
 
-extern "C" int nt_varlen_attention_vt(const void* qk, int64_t ldqk, int64_t k_col, const void* vt,
-                                      int64_t ldvt, void* out, int64_t ldo,
+extern "C" int nt_varlen_attention_vt(const void* q, int64_t ldq, const void* k, int64_t ldk,
+                                      const void* vt, int64_t ldvt, void* out, int64_t ldo,
                                       const int32_t* schedule, int64_t n_work, int64_t num_heads,
-                                      int64_t total_tokens, float scale, int dtype, void* stream) {
-  if (n_work < 0 || num_heads < 1 || total_tokens < 0) {
+                                      int64_t total_kv_tokens, float scale, int dtype, void* stream) {
+  if (n_work < 0 || num_heads < 1 || total_kv_tokens < 0) {
     return fail(NT_ERR_INVALID_ARGUMENT, "attention_vt: bad shape");
   }
   if (n_work == 0) return NT_OK;
-  if (!qk || !vt || !out || !schedule) return fail(NT_ERR_INVALID_ARGUMENT, "attention_vt: NULL pointer");
-  if (n_work > 0x7fffffffLL || num_heads > 65535 || total_tokens > 0x7fffffffLL) {
+  if (!q || !k || !vt || !out || !schedule) return fail(NT_ERR_INVALID_ARGUMENT, "attention_vt: NULL pointer");
+  if (n_work > 0x3fffffffLL || num_heads > 65535 || total_kv_tokens > 0x7fffffffLL) {
     return fail(NT_ERR_UNSUPPORTED, "attention_vt: too many work items, heads or tokens");
   }
   const int64_t E = num_heads * kHd;
-  if (ldqk < k_col + E || ldo < E || ldvt < total_tokens + 72) {
+  if (ldq < E || ldk < E || ldo < E || ldvt < total_kv_tokens + 72) {
     return fail(NT_ERR_INVALID_ARGUMENT,
-                "attention_vt: row strides too small (ldvt must be >= total_tokens + 72)");
+                "attention_vt: row strides too small (ldvt must be >= total_kv_tokens + 72)");
   }
   if (n_work * num_heads > 0x7fffffffLL) {
     return fail(NT_ERR_UNSUPPORTED, "attention_vt: too many workgroups");
@@ -746,13 +752,14 @@ extern "C" int nt_varlen_attention_vt(const void* qk, int64_t ldqk, int64_t k_co
   const int4* sched = reinterpret_cast<const int4*>(schedule);
   if (dtype == NT_F16) {
     hipLaunchKernelGGL((varlen_attention_vt_kernel<_Float16>), grid, dim3(256), 0, s,
-                       static_cast<const _Float16*>(qk), ldqk, k_col,
+                       static_cast<const _Float16*>(q), ldq, static_cast<const _Float16*>(k), ldk,
                        static_cast<const _Float16*>(vt), ldvt, static_cast<_Float16*>(out), ldo,
                        sched, (unsigned)num_heads, scale_log2e);
   } else if (dtype == NT_BF16) {
     hipLaunchKernelGGL((varlen_attention_vt_kernel<__bf16>), grid, dim3(256), 0, s,
-                       static_cast<const __bf16*>(qk), ldqk, k_col, static_cast<const __bf16*>(vt),
-                       ldvt, static_cast<__bf16*>(out), ldo, sched, (unsigned)num_heads, scale_log2e);
+                       static_cast<const __bf16*>(q), ldq, static_cast<const __bf16*>(k), ldk,
+                       static_cast<const __bf16*>(vt), ldvt, static_cast<__bf16*>(out), ldo, sched,
+                       (unsigned)num_heads, scale_log2e);
   } else {
     return fail(NT_ERR_UNSUPPORTED, "attention_vt: dtype must be f16 or bf16");
   }

@@ -638,3 +638,33 @@ extern "C" int nt_linear_qkv(const void* A, int64_t lda, const void* W, const vo
   }
 #undef NT_QKV_CASE
 }
+
+extern "C" int nt_linear_transposed(const void* A, int64_t lda, const void* W, const void* bias,
+                                    void* Ct, int64_t ldct, int64_t M, int64_t N, int64_t K, int dtype,
+                                    void* stream) {
+  int rc = check_linear(A, lda, W, Ct, ldct, M, N, K);
+  if (rc != NT_OK) return rc;
+  if (ldct < M) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "linear_transposed: ldct %lld < M %lld", (long long)ldct,
+                (long long)M);
+  }
+  if (M == 0 || N == 0) return NT_OK;
+  hipStream_t s = (hipStream_t)stream;
+  // every tile is a transposed-output tile of the fused QKV kernel: split at column 0
+#define NT_LT_CASE(TYPE)                                                     \
+  {                                                                          \
+    GemmArgs<TYPE> a = make_args<TYPE>(A, lda, W, bias, Ct, ldct, M, N, K);  \
+    a.C = nullptr;                                                           \
+    a.Vt = static_cast<TYPE*>(Ct);                                           \
+    a.ldvt = ldct;                                                           \
+    a.n_split = 0;                                                           \
+    return launch_linear<TYPE>(a, true, s);                                  \
+  }
+  switch (dtype) {
+    case NT_F32: NT_LT_CASE(float)
+    case NT_F16: NT_LT_CASE(_Float16)
+    case NT_BF16: NT_LT_CASE(__bf16)
+    default: return fail(NT_ERR_INVALID_ARGUMENT, "linear_transposed: unknown dtype %d", dtype);
+  }
+#undef NT_LT_CASE
+}

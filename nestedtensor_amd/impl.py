@@ -145,25 +145,33 @@ class NestedTensorImpl:
             self._last_dim_rows = (row_offsets.to(self.buffer.device), int(row_offsets[-1]))
         return self._last_dim_rows
 
-    def attention_schedule(self, q_tile=128):
-        """Work list of the self-attention kernel, built from the host copy of the
-        nested size and cached on the device: int32 [n_work, 4] rows
-        {first token, length, first query row of the tile, 0}, one per q_tile
-        query rows of every sequence, longest sequences first (they take the
-        most key tiles, so they should start first).  Tiles that do not exist
-        are never listed, hence never launched."""
-        if self._attn_schedule is None:
-            lens = self.sizes[:, 0]
-            starts = torch.cumsum(lens, 0) - lens
-            order = torch.argsort(lens, descending=True, stable=True)
-            lens_o, starts_o = lens[order], starts[order]
-            ntile = (lens_o + q_tile - 1) // q_tile
-            seq = torch.repeat_interleave(torch.arange(lens_o.numel()), ntile)
-            first = torch.cumsum(ntile, 0) - ntile
-            q0 = (torch.arange(int(ntile.sum())) - first[seq]) * q_tile
-            items = torch.stack([starts_o[seq], lens_o[seq], q0, torch.zeros_like(q0)], 1)
-            self._attn_schedule = items.to(torch.int32).contiguous().to(self.buffer.device)
-        return self._attn_schedule
+    def attention_schedule(self, kv=None, q_tile=128):
+        """Work list of the attention kernel, built from the host copies of the
+        nested sizes and cached on the device: int32 [n_work, 8] rows {first query
+        token, query length, first query row of the tile, 0, first key token, key
+        length, 0, 0}, one per q_tile query rows of every sequence, longest key
+        sequences first (they take the most key tiles, so they should start
+        first).  Tiles that do not exist are never listed, hence never launched.
+        kv: the nested tensor of the keys (None: self-attention)."""
+        if kv is None or kv.sizes is self.sizes:
+            kv = self
+        cached = self._attn_schedule
+        if cached is not None and cached[0] is kv.sizes:
+            return cached[1]
+        q_lens, k_lens = self.sizes[:, 0], kv.sizes[:, 0]
+        q_starts = torch.cumsum(q_lens, 0) - q_lens
+        k_starts = torch.cumsum(k_lens, 0) - k_lens
+        order = torch.argsort(k_lens, descending=True, stable=True)
+        ntile = (q_lens[order] + q_tile - 1) // q_tile
+        seq = order[torch.repeat_interleave(torch.arange(order.numel()), ntile)]
+        first = torch.cumsum(ntile, 0) - ntile
+        rank = torch.repeat_interleave(torch.arange(order.numel()), ntile)
+        q0 = (torch.arange(int(ntile.sum())) - first[rank]) * q_tile
+        zero = torch.zeros_like(q0)
+        items = torch.stack([q_starts[seq], q_lens[seq], q0, zero, k_starts[seq], k_lens[seq], zero, zero], 1)
+        sched = items.to(torch.int32).contiguous().to(self.buffer.device)
+        self._attn_schedule = (kv.sizes, sched)      # holds kv.sizes, so the identity test stays valid
+        return sched
 
     def with_buffer(self, buffer, channels_last=None):
         """Same nested size over another buffer (in the same layout unless

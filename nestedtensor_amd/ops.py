@@ -376,7 +376,8 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
     T_tokens = xq.size(0)
     max_q = int(query.sizes[:, 0].max()) if query.B > 0 else 0
     attn = torch.empty((T_tokens, E), dtype=dtype, device=dev)
-    fused = same and head_dim == 64 and dtype in (torch.float16, torch.bfloat16) and (2 * E) % 128 == 0
+    mfma_path = head_dim == 64 and dtype in (torch.float16, torch.bfloat16)
+    fused = same and mfma_path and (2 * E) % 128 == 0
     if in_proj_bias is not None:
         in_proj_bias = in_proj_bias.contiguous()
         if in_proj_bias.dtype != dtype:
@@ -396,8 +397,30 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
                 _C.ptr(vt), ldvt, T_tokens, E, E, _C.dtype_code(dtype), stream))
             sched = query.attention_schedule()
             _C.check(_C.lib.nt_varlen_attention_vt(
-                _C.ptr(qk), 2 * E, E, _C.ptr(vt), ldvt, _C.ptr(attn), E,
+                _C.ptr(qk), 2 * E, _offset_ptr(qk, E), 2 * E, _C.ptr(vt), ldvt, _C.ptr(attn), E,
                 _C.ptr(sched), sched.size(0), num_heads, T_tokens,
+                float(scaling), _C.dtype_code(dtype), stream))
+    elif mfma_path and not same and bool((key.sizes[:, 0] > 0).all()):
+        # cross-attention, head_dim 64: three projections (the value one written
+        # transposed), then the same attention kernel with one key sequence per
+        # query sequence
+        b = in_proj_bias
+        T_kv = key.buffer.numel() // E
+        q_t = linear(xq, W[0:E], None if b is None else b[0:E])
+        k_t = linear(key.buffer.reshape(-1, E), W[E:2 * E], None if b is None else b[E:2 * E])
+        ldvt = (T_kv + 72 + 7) // 8 * 8
+        vt = torch.empty((E, ldvt), dtype=dtype, device=dev)
+        xv = value.buffer.reshape(-1, E)
+        bv = None if b is None else b[2 * E:].contiguous()
+        with torch.cuda.device(dev):
+            stream = _C.current_stream(dev)
+            _C.check(_C.lib.nt_linear_transposed(
+                _C.ptr(xv), xv.stride(0), _C.ptr(W[2 * E:]), _C.ptr(bv), _C.ptr(vt), ldvt, T_kv, E, E,
+                _C.dtype_code(dtype), stream))
+            sched = query.attention_schedule(kv=key)
+            _C.check(_C.lib.nt_varlen_attention_vt(
+                _C.ptr(q_t), E, _C.ptr(k_t), E, _C.ptr(vt), ldvt, _C.ptr(attn), E,
+                _C.ptr(sched), sched.size(0), num_heads, T_kv,
                 float(scaling), _C.dtype_code(dtype), stream))
     else:
         if same:

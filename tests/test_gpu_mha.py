@@ -133,13 +133,21 @@ def test_bt_min_mha_ignores_out_bias_and_min_mha_adds_it():
     assert not torch.equal(r_bt._impl.buffer, r_min._impl.buffer)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
-def test_cross_attention_different_kv_lengths(dtype):
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("q_lens,kv_lens", [((3, 130, 64), (77, 2, 200)),
+                                            ((100, 100, 100, 1), (1, 64, 65, 513)),     # DETR-like: fixed queries
+                                            ((257, 5), (128, 129))])
+def test_cross_attention_different_kv_lengths(dtype, q_lens, kv_lens):
+    # fp16 / bf16 with head_dim 64 take the MFMA kernel with one key sequence per query
+    # sequence; fp32 the general kernel
     H, hd = 4, 64
     E = H * hd
     g = torch.Generator().manual_seed(5)
-    q = [torch.randn(L, E, generator=g).to(dtype) for L in (3, 130, 64)]
-    kv = [torch.randn(L, E, generator=g).to(dtype) for L in (77, 2, 200)]
+    # bf16 keeps 8 bits: inputs at half the scale hold the outputs below 2, where one unit of
+    # output rounding (the fused path rounds once, the reference after every op) is under 2e-2
+    amp = 0.5 if dtype == torch.bfloat16 else 1.0
+    q = [(torch.randn(L, E, generator=g) * amp).to(dtype) for L in q_lens]
+    kv = [(torch.randn(L, E, generator=g) * amp).to(dtype) for L in kv_lens]
     _, W_in, b_in, W_out, b_out = make_case(E, [1], 6, dtype, w_std=E ** -0.5, bias_std=0.1)
     qa, ka = nt.nested_tensor(q, device=DEV, dtype=dtype), nt.nested_tensor(kv, device=DEV, dtype=dtype)
     got = torch.ops.nestedtensor.min_mha(H, hd, 0.0, False, qa, ka, ka, W_in.to(DEV), b_in.to(DEV),
@@ -147,6 +155,34 @@ def test_cross_attention_different_kv_lengths(dtype):
     rq, rk = oracle.ref_nested_tensor(q, dtype=dtype), oracle.ref_nested_tensor(kv, dtype=dtype)
     exp = oracle.min_mha(H, hd, 0.0, False, rq, rk, rk, W_in, b_in, hd ** -0.5, W_out, b_out)
     check(got, exp, dtype)
+    # key and value of the same nested size but different contents (key = memory + position)
+    v2 = [(torch.randn(L, E, generator=g) * amp).to(dtype) for L in kv_lens]
+    va = nt.nested_tensor(v2, device=DEV, dtype=dtype)
+    got = torch.ops.nestedtensor.min_mha(H, hd, 0.0, False, qa, ka, va, W_in.to(DEV), b_in.to(DEV),
+                                         hd ** -0.5, W_out.to(DEV), b_out.to(DEV))
+    rv = oracle.ref_nested_tensor(v2, dtype=dtype)
+    exp = oracle.min_mha(H, hd, 0.0, False, rq, rk, rv, W_in, b_in, hd ** -0.5, W_out, b_out)
+    check(got, exp, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M,N,K", [(300, 256, 128), (1000, 192, 64), (257, 70, 96), (5, 64, 40)])
+def test_linear_transposed(M, N, K, dtype):
+    from nestedtensor_amd import _C
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) * 0.2).to(dtype)
+    b = torch.randn(N, generator=g).to(dtype)
+    ld = (M + 72 + 7) // 8 * 8
+    ct = torch.full((N, ld), 7.0, dtype=dtype, device=DEV)
+    xd, wd, bd = x.to(DEV), w.to(DEV), b.to(DEV)
+    _C.check(_C.lib.nt_linear_transposed(_C.ptr(xd), K, _C.ptr(wd), _C.ptr(bd), _C.ptr(ct), ld, M, N, K,
+                                         _C.dtype_code(dtype), _C.current_stream(DEV)))
+    ref = (x.double() @ w.double().t() + b.double()).t()
+    got = ct[:, :M].double().cpu()
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert (got - ref).abs().max().item() <= tol * max(1.0, ref.abs().max().item())
+    assert bool((ct[:, M:] == 7.0).all())          # nothing is written past column M
 
 
 def test_mha_input_errors():
