@@ -212,8 +212,20 @@ class NestedTensor:
     def unbind(self, dim=0):
         """Views into the packed buffer, one per constituent
         (nested_tensor_impl.cpp:207-232 with build_structure, Packed.h:21-64)."""
+        nd = self.dim()
+        if not -nd <= dim < nd:
+            raise IndexError("Dimension out of range (expected to be in range of [%d, %d], but got %d)"
+                             % (-nd, nd - 1, dim))
+        dim = dim % nd
         if dim != 0:
-            raise RuntimeError("unbind() only supports dim == 0 in this build.")
+            # splitting the tree one level down (nested_tensor_impl.cpp:216-231): result j
+            # holds slice j along `dim` of every constituent that is long enough
+            from . import creation
+            pieces = [t.unbind(dim - 1) for t in self.unbind(0)]
+            n = max((len(p) for p in pieces), default=0)
+            return tuple(
+                creation.nested_tensor([p[j] for p in pieces if len(p) > j], dtype=self.dtype, device=self.device)
+                for j in range(n))
         out, off = [], 0
         for s in self._impl.shapes():
             n = 1
@@ -380,6 +392,10 @@ def _log_softmax(input, dim=None, _stacklevel=3, dtype=None):
     return ops.softmax(input, dim, dtype, log=True)
 
 
+def _unbind(input, dim=0):
+    return NestedTensor(input).unbind(dim)
+
+
 def _to_tensor_list(impl):
     return list(NestedTensor(impl).unbind())
 
@@ -443,6 +459,8 @@ _HANDLERS = {
     torch.Tensor.add: _add,
     torch.Tensor.__add__: _add,
     torch.Tensor.__radd__: _add,
+    torch.unbind: _unbind,
+    torch.Tensor.unbind: _unbind,
     torch.nn.functional.softmax: _softmax,
     torch.softmax: _softmax,
     torch.Tensor.softmax: _softmax,
@@ -461,7 +479,7 @@ _HANDLERS = {
 # handlers that look at the storage layout themselves (or only at the nested
 # size); every other handler is given row-major operands
 _LAYOUT_AWARE = {
-    _to_tensor_list, _get_max_size, _is_nested_tensor_impl, _nested_dim, _sizes, _len, _get_dim, _get_numel,
+    _unbind, _to_tensor_list, _get_max_size, _is_nested_tensor_impl, _nested_dim, _sizes, _len, _get_dim, _get_numel,
     ops.is_contiguous, ops.contiguous, ops.conv2d, ops.max_pool2d, _add, _mul,
     ops.transpose_nchw_nhwc, ops.transpose_nhwc_nchw,
 }

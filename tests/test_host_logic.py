@@ -246,3 +246,29 @@ def test_channels_last_metadata_and_views():
         b.contiguous(memory_format=torch.channels_last)
     with pytest.raises(RuntimeError, match="requires 4 dim input"):
         nt.nested_tensor([torch.randn(2, 3)]).contiguous(memory_format=torch.channels_last)
+
+
+def test_unbind_across_constituent_dims():
+    # test/test_nested_tensor_class.py:394-429
+    for unbind_fn in (lambda x, dim: x.unbind(dim), lambda x, dim: torch.unbind(x, dim)):
+        a = torch.rand(3, 2)
+        x = nt.nested_tensor([a])
+        for d in (1, 2):
+            got = unbind_fn(x, d)
+            exp = [nt.nested_tensor([p]) for p in a.unbind(d - 1)]
+            assert len(got) == len(exp)
+            for g_, e_ in zip(got, exp):
+                assert g_.nested_size() == e_.nested_size()
+                assert all(torch.equal(u, v) for u, v in zip(g_.unbind(), e_.unbind()))
+        b = torch.rand(2, 3)
+        x = nt.nested_tensor([a, b])
+        assert all(torch.equal(u, v) for u, v in zip(unbind_fn(x, 0), (a, b)))
+        got = unbind_fn(x, 1)
+        exp = [nt.nested_tensor([a[0], b[0]]), nt.nested_tensor([a[1], b[1]]), nt.nested_tensor([a[2]])]
+        assert len(got) == 3
+        for g_, e_ in zip(got, exp):
+            assert g_.nested_size() == e_.nested_size()
+            assert all(torch.equal(u, v) for u, v in zip(g_.unbind(), e_.unbind()))
+        assert len(unbind_fn(x, -1)) == 3          # slices along the last dim: 2 and 3 columns
+        with pytest.raises(IndexError):
+            unbind_fn(x, 3)
