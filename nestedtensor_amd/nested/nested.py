@@ -243,6 +243,20 @@ class NestedTensor:
     def to_tensor_list(self):
         return list(self.unbind())
 
+    def to_tensor(self, dim=0):
+        """The stack of the constituents when every dim is regular
+        (NestedTensor_to_tensor, totensor.cpp:45-63); a copy, not a view."""
+        nd = self.dim()
+        if dim is not None and dim % nd != 0:
+            raise RuntimeError("Non-zero dimension %d is currently not supported." % dim)
+        opt = self._impl.opt_sizes()
+        if any(v is None for v in opt):
+            raise IndexError("to_tensor()/to_tensor(0) only works if there is no None in size().")
+        if len(self) == 0:
+            return torch.empty(0, dtype=self.dtype, device=self.device)
+        impl = ops.contiguous(self._impl) if self._impl.channels_last else self._impl
+        return impl.buffer.reshape(opt).clone()
+
     def __iter__(self):
         return iter(self.unbind())
 

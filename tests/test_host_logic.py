@@ -272,3 +272,17 @@ def test_unbind_across_constituent_dims():
         assert len(unbind_fn(x, -1)) == 3          # slices along the last dim: 2 and 3 columns
         with pytest.raises(IndexError):
             unbind_fn(x, 3)
+
+
+def test_to_tensor_needs_regular_sizes():
+    # totensor.cpp:30-42, 45-63
+    ts = [torch.rand(3, 2), torch.rand(3, 2)]
+    a = nt.nested_tensor(ts)
+    got = a.to_tensor()
+    assert torch.equal(got, torch.stack(ts)) and got.data_ptr() != a._impl.buffer.data_ptr()
+    assert torch.equal(a.to_tensor(0), torch.stack(ts))
+    with pytest.raises(IndexError, match="only works if there is no None in size"):
+        nt.nested_tensor([torch.rand(3, 2), torch.rand(2, 2)]).to_tensor()
+    with pytest.raises(RuntimeError, match="Non-zero dimension 1 is currently not supported."):
+        a.to_tensor(1)
+    assert nt.nested_tensor([]).to_tensor().numel() == 0
