@@ -261,12 +261,35 @@ class NestedTensor:
         return iter(self.unbind())
 
     def __getitem__(self, key):
+        """get_item (py_init.cpp:26-108) at nested_dim 1: an int picks a constituent
+        (a view), a slice a NestedTensor of constituents (a copy); further tuple
+        entries index every selected constituent."""
+        from . import creation
+        if isinstance(key, tuple):
+            if len(key) == 0:
+                return self
+            first, rest = key[0], key[1:]
+            if first is None:
+                raise RuntimeError("Only nested_dim of 1 is currently supported.")
+            if not isinstance(first, (int, slice)):
+                raise RuntimeError("First entry of tuple doesn't have accepted type. " + str(first))
+            sel = self[first]
+            if not rest:
+                return sel
+            if torch.is_tensor(sel):
+                return sel[rest]
+            return creation.nested_tensor([t[rest] for t in sel.unbind()], dtype=self.dtype, device=self.device)
         if isinstance(key, int):
+            n = len(self)
+            if not -max(n, 1) <= key < max(n, 1):
+                raise IndexError("Dimension out of range (expected to be in range of [%d, %d], but got %d)"
+                                 % (-max(n, 1), max(n, 1) - 1, key))
             return self.unbind()[key]
         if isinstance(key, slice):
-            from . import creation
             return creation.nested_tensor(list(self.unbind()[key]), dtype=self.dtype, device=self.device)
-        raise IndexError("NestedTensor indexing supports an int or a slice of the nested dimension.")
+        if key is None:
+            raise RuntimeError("Only nested_dim of 1 is currently supported.")
+        raise IndexError("NestedTensor indexing supports ints, slices and tuples of them.")
 
     def __bool__(self):
         raise NotImplementedError("NestedTensor doesn't support function __bool__")

@@ -286,3 +286,23 @@ def test_to_tensor_needs_regular_sizes():
     with pytest.raises(RuntimeError, match="Non-zero dimension 1 is currently not supported."):
         a.to_tensor(1)
     assert nt.nested_tensor([]).to_tensor().numel() == 0
+
+
+def test_getitem_int_slice_tuple():
+    # py_init.cpp:26-108 at nested_dim 1 (cases of test/test_nested_tensor_class.py:679-707 that need no deeper nesting)
+    a, b, c = torch.randn(3, 4), torch.randn(4, 3), torch.randn(1, 3)
+    x = nt.nested_tensor([a, b, c])
+    assert torch.equal(x[0], a) and torch.equal(x[-1], c)
+    assert x[0].data_ptr() == x._impl.buffer.data_ptr()                 # a view
+    assert x[:].nested_size() == x.nested_size()
+    assert [tuple(t.shape) for t in x[-1:].unbind()] == [(1, 3)]
+    assert torch.equal(x[0, 1:], a[1:]) and torch.equal(x[1, :, 0], b[:, 0])
+    got = x[:, 0]
+    assert all(torch.equal(u, v) for u, v in zip(got.unbind(), (a[0], b[0], c[0])))
+    got = x[:2, :, -1:]
+    assert all(torch.equal(u, v) for u, v in zip(got.unbind(), (a[:, -1:], b[:, -1:])))
+    assert x[()] is x
+    with pytest.raises(IndexError, match=r"expected to be in range of \[-3, 2\], but got 3"):
+        x[3]
+    with pytest.raises(RuntimeError, match="Only nested_dim of 1"):
+        x[None]
