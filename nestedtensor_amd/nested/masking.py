@@ -295,6 +295,10 @@ def _nt_from_tensor_mask_op(tensor, mask, nested_dim):
 ops._lib.impl("nt_from_tensor_mask", _nt_from_tensor_mask_op, "CompositeExplicitAutograd")
 
 
+# masking.cpp:653-655: an op on plain tensors, one implementation for every device
+ops._lib.impl("merge_tensor_mask", ops.merge_tensor_mask, "CompositeExplicitAutograd")
+
+
 def _nt_from_padded_tensor_op(tensor, padding, nested_dim):
     impl = _from_value_native(tensor, padding, nested_dim)
     return impl.buffer, impl.sizes

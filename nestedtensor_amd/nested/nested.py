@@ -471,6 +471,7 @@ _HANDLERS = {
     _ns.to_tensor_mask: ops.to_tensor_mask,
     _ns.to_mask: ops.to_mask,
     _ns.get_max_size: _get_max_size,
+    _ns.pad_nt: ops.pad_nt,
     _ns.min_mha: ops.min_mha,
     _ns.bt_min_mha: ops.bt_min_mha,
     _ns.is_nested_tensor_impl: _is_nested_tensor_impl,

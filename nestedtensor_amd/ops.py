@@ -29,6 +29,8 @@ _SCHEMAS = [
     "to_mask(Tensor nt, int? mask_dim) -> Tensor",
     "nt_from_tensor_mask(Tensor tensor, Tensor mask, int nested_dim) -> (Tensor, Tensor)",
     "get_max_size(Tensor nt) -> int[]",
+    "pad_nt(Tensor nt, int[] shape) -> (Tensor, Tensor)",
+    "merge_tensor_mask(Tensor tensor, Tensor mask, int? mask_dim=None) -> (Tensor, Tensor)",
     # nestedtensor/csrc/mha.cpp:72, nestedtensor/csrc/cuda/mha.cpp:110-111
     "min_mha(int num_heads, int head_dim, float dropout_p, bool training, Tensor query, "
     "Tensor key, Tensor value, Tensor in_proje_weight, Tensor? in_proj_bias, float scaling, "
@@ -92,14 +94,24 @@ def _check_no_empty(impl):
 # packed -> padded
 
 
-def add_padding(impl, padding, with_mask=False):
-    """Launch nt_add_padding: [B, max_1..max_D] from the packed buffer.  With
+def add_padding(impl, padding, with_mask=False, shape=None):
+    """Launch nt_add_padding: [B, max_1..max_D] from the packed buffer (or
+    [B] + shape for a caller-given shape that holds every constituent).  With
     with_mask, nt_add_padding_mask writes the bool mask of the same shape in the
     same launch and (padded, mask) is returned."""
     _C.require_device(impl.buffer, "to_padded_tensor")
     B, D = impl.B, impl.D
     max_size = impl.max_sizes()
     nrag = _n_ragged(impl)
+    if shape is not None:
+        shape = [int(v) for v in shape]
+        if len(shape) != D or any(s < m for s, m in zip(shape, max_size)):
+            raise RuntimeError("pad_nt: shape %s does not hold constituents of up to %s" % (shape, max_size))
+        # a dim that is regular but shorter than the requested extent is walked as ragged
+        for k in range(D):
+            if shape[k] != max_size[k]:
+                nrag = max(nrag, k + 1)
+        max_size = shape
     if nrag > 3:
         raise RuntimeError("to_padded_tensor supports at most 3 irregular dimensions.")
     out = torch.empty([B] + max_size, dtype=impl.buffer.dtype, device=impl.buffer.device)
@@ -118,6 +130,37 @@ def add_padding(impl, padding, with_mask=False):
             B, D, nrag, _C.i64_array(max_size), eb, _pad_bits(padding, impl.buffer.dtype),
             _C.current_stream(dev)))
     return out
+
+
+def pad_nt(impl, shape):
+    """pad_nt (masking.cpp:138-179): every constituent padded with 0 to `shape`,
+    stacked, and the mask of the same shape (bool here, uint8 in the reference)."""
+    if impl.B == 0:
+        return torch.tensor([0]), torch.tensor([False])          # masking.cpp:164-167
+    _check_no_empty(impl)
+    if impl.D == 0:
+        return impl.buffer.clone(), torch.ones(impl.B, dtype=torch.bool, device=impl.buffer.device)
+    return add_padding(impl, 0, with_mask=True, shape=shape)
+
+
+def merge_tensor_mask(tensor, mask, mask_dim=None):
+    """merge_tensor_mask (masking.cpp:12-43) on a dense (tensor, mask) pair: the
+    last mask dim is dropped while every one of its rows is all ones or all
+    zeros; stops at mask_dim, and refuses a mask_dim it cannot reach."""
+    while True:
+        if mask_dim is not None and mask.dim() == mask_dim:
+            return tensor, mask
+        if mask.dim() == 0:
+            return tensor, mask
+        last = mask.size(-1)
+        collapsed = mask.sum(-1)
+        uniform = int(((collapsed == last) | (collapsed == 0)).sum())
+        if uniform == collapsed.numel():
+            mask = collapsed.to(torch.bool)
+            continue
+        if mask_dim is not None and mask_dim != mask.dim():
+            raise RuntimeError("Mask dimension is too small to represent data tensor.")
+        return tensor.contiguous(), mask.contiguous()
 
 
 def to_padded_tensor(impl, padding):

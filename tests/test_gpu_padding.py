@@ -315,6 +315,26 @@ def test_from_padded_tensor_length_based(dims, dtype):
     bits_equal(back2._impl.buffer, ref.buffer)
 
 
+def test_pad_nt_to_a_given_shape():
+    # pad_nt (masking.cpp:138-179): a caller-given goal shape, data padded with 0, full-shape mask
+    parts = [torch.randn(3, 5), torch.randn(1, 5), torch.randn(4, 2)]
+    a = nt.nested_tensor(parts, device=DEV)
+    ref = oracle.ref_nested_tensor(parts)
+    for shape in ([4, 5], [6, 9]):
+        data, mask = torch.ops.nestedtensor.pad_nt(a, shape)
+        exp_d, exp_m = oracle.pad_nt(ref, shape)
+        bits_equal(data, exp_d)
+        assert mask.dtype == torch.bool and torch.equal(mask.cpu(), exp_m.to(torch.bool))
+    # a regular dim shorter than the goal shape
+    reg = [torch.randn(2, 3), torch.randn(2, 3)]
+    data, mask = torch.ops.nestedtensor.pad_nt(nt.nested_tensor(reg, device=DEV), [2, 8])
+    exp_d, exp_m = oracle.pad_nt(oracle.ref_nested_tensor(reg), [2, 8])
+    bits_equal(data, exp_d)
+    assert torch.equal(mask.cpu(), exp_m.to(torch.bool))
+    with pytest.raises(RuntimeError, match="does not hold"):
+        torch.ops.nestedtensor.pad_nt(a, [3, 5])
+
+
 # ---- benchmark configurations -----------------------------------------------------
 
 def test_config_c1_round_trip_bit_exact():

@@ -306,3 +306,26 @@ def test_getitem_int_slice_tuple():
         x[3]
     with pytest.raises(RuntimeError, match="Only nested_dim of 1"):
         x[None]
+
+
+def test_merge_tensor_mask_op_matches_oracle():
+    # masking.cpp:12-43 as an op on plain tensors
+    import oracle
+    g = torch.Generator().manual_seed(3)
+    t = torch.randn(4, 3, 5, generator=g)
+    full_rows = torch.tensor([[1, 1, 0], [1, 0, 0], [1, 1, 1], [0, 0, 0]], dtype=torch.uint8)
+    cases = [full_rows.unsqueeze(-1).expand(4, 3, 5).contiguous(),            # collapses to [4, 3]
+             torch.ones(4, 3, 5, dtype=torch.uint8),                         # collapses to a scalar
+             (torch.rand(4, 3, 5, generator=g) > 0.5).to(torch.uint8)]       # does not collapse
+    for m in cases:
+        for mask_dim in (None, 1, 2, 3):
+            try:
+                exp = oracle.merge_tensor_mask(t, m, mask_dim)
+            except RuntimeError as e:
+                with pytest.raises(RuntimeError, match=str(e)):
+                    torch.ops.nestedtensor.merge_tensor_mask(t, m, mask_dim)
+                continue
+            got = torch.ops.nestedtensor.merge_tensor_mask(t, m, mask_dim)
+            assert got[1].shape == exp[1].shape
+            assert torch.equal(got[1].to(torch.bool), exp[1].to(torch.bool))
+            assert torch.equal(got[0], exp[0])
