@@ -243,6 +243,9 @@ class NestedTensor:
     def to_tensor_list(self):
         return list(self.unbind())
 
+    def to_nested_tensor(self, dim=0):
+        return torch.ops.nestedtensor.to_nested_tensor(self, dim)
+
     def to_tensor(self, dim=0):
         """The stack of the constituents when every dim is regular
         (NestedTensor_to_tensor, totensor.cpp:45-63); a copy, not a view."""
@@ -433,6 +436,19 @@ def _unbind(input, dim=0):
     return NestedTensor(input).unbind(dim)
 
 
+def _to_nested_tensor(impl, dim=None):
+    """NestedTensor_to_nested_tensor (nested_tensor_impl.cpp:244-263): already
+    nested up to dim 0; a deeper nesting would need nested_dim 2."""
+    nd = impl.dim() + 1
+    d = 0 if dim is None else dim
+    if not -nd <= d < nd:
+        raise IndexError("Dimension out of range (expected to be in range of [%d, %d], but got %d)"
+                         % (-nd, nd - 1, d))
+    if d % nd < impl.nested_dim():
+        return impl
+    raise RuntimeError("Only nested_dim of 1 is currently supported.")
+
+
 def _to_tensor_list(impl):
     return list(NestedTensor(impl).unbind())
 
@@ -476,6 +492,7 @@ _HANDLERS = {
     _ns.bt_min_mha: ops.bt_min_mha,
     _ns.is_nested_tensor_impl: _is_nested_tensor_impl,
     _ns.nested_dim: _nested_dim,
+    _ns.to_nested_tensor: _to_nested_tensor,
     _ns.sizes: _sizes,
     _ns.len: _len,
     _ns.get_dim: _get_dim,
@@ -517,7 +534,7 @@ _HANDLERS = {
 # handlers that look at the storage layout themselves (or only at the nested
 # size); every other handler is given row-major operands
 _LAYOUT_AWARE = {
-    _unbind, _to_tensor_list, _get_max_size, _is_nested_tensor_impl, _nested_dim, _sizes, _len, _get_dim, _get_numel,
+    _unbind, _to_nested_tensor, _to_tensor_list, _get_max_size, _is_nested_tensor_impl, _nested_dim, _sizes, _len, _get_dim, _get_numel,
     ops.is_contiguous, ops.contiguous, ops.conv2d, ops.max_pool2d, _add, _mul,
     ops.transpose_nchw_nhwc, ops.transpose_nhwc_nchw,
 }

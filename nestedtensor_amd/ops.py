@@ -41,6 +41,7 @@ _SCHEMAS = [
     # nestedtensor/csrc/py_init.cpp:132-216
     "is_nested_tensor_impl(Tensor tensor) -> bool",
     "nested_dim(Tensor tensor) -> int",
+    "to_nested_tensor(Tensor tensor, int? dim) -> Tensor",
     "sizes(Tensor tensor) -> int?[]",
     "len(Tensor self) -> int",
     "get_dim(Tensor self) -> int",
