@@ -294,10 +294,33 @@ def bench_mha_c3(args, torch, dev):
         graph_ms = "graph capture failed: %r" % (exc,)
     T = sum(lens)
     flops = 8 * T * E * E + 4 * E * sum(L * L for L in lens)
+    # the whole encoder layer on the packed layout: attention, residual + layer norm,
+    # feed-forward 768 -> 3072 (gelu in the GEMM epilogue) -> 768, residual + layer norm
+    from nestedtensor_amd import ops as _ops
+    W1 = (torch.randn(4 * E, E, generator=g) * 0.02).half().to(dev)
+    W2 = (torch.randn(E, 4 * E, generator=g) * 0.02).half().to(dev)
+    b1, b2 = torch.zeros(4 * E, device=dev).half(), torch.zeros(E, device=dev).half()
+    ln_w, ln_b = torch.ones(E, device=dev).half(), torch.zeros(E, device=dev).half()
+
+    def encoder_layer():
+        y = layer()
+        h = _ops.layer_norm(y._impl, (E,), ln_w, ln_b, 1e-5, residual=a._impl)
+        f = _ops.linear_nt(h, W1, b1, "gelu")
+        o = _ops.linear_nt(f, W2, b2)
+        return _ops.layer_norm(o, (E,), ln_w, ln_b, 1e-5, residual=h)
+
+    ms_enc = _time_gpu(torch, encoder_layer, iters=50, warmup=5)
+    flops_enc = flops + 16 * T * E * E
     res = dict(workload="C3: nested BERT-base self-attention, fp16, B=32, L~U[32,512], d=768, 12x64",
                tokens=T, ms_per_layer=ms, ms_per_layer_hip_graph=graph_ms, tokens_per_s=T / (ms * 1e-3), flops=flops,
                roofline=dict(bound="mfma", achieved=flops / (ms * 1e-3) / 1e12, peak=MFMA_F16_PEAK_TFLOPS,
                              unit="TFLOP/s", frac=flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS))
+    res["encoder_layer"] = dict(
+        workload="the same batch through a whole BERT-base encoder layer (attention, add + layer norm, "
+                 "768-3072-768 feed-forward with gelu, add + layer norm), 7 launches",
+        ms_per_layer=ms_enc, tokens_per_s=T / (ms_enc * 1e-3), flops=flops_enc,
+        TFLOPs=flops_enc / (ms_enc * 1e-3) / 1e12,
+        frac_of_mfma_peak=flops_enc / (ms_enc * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS)
     if not args.no_cpu:
         torch.set_num_threads(os.cpu_count() or 1)
         ref = oracle.ref_nested_tensor(xs, dtype=torch.float16)

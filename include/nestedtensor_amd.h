@@ -159,6 +159,16 @@ int nt_exclusive_scan_i32(const int32_t* in, int64_t n, int64_t* out, void* work
 int nt_linear(const void* A, int64_t lda, const void* W, const void* bias, void* C,
               int64_t ldc, int64_t M, int64_t N, int64_t K, int dtype, void* stream);
 
+/* nt_linear with an activation applied to A W^T + bias in fp32 before the one
+ * rounding: act 0 none, 1 relu, 2 gelu (erf form, torch's default).  The first
+ * feed-forward projection of an encoder layer in one launch; the reference has
+ * the pieces unfused: the packed matmul (nestedtensor/csrc/matmul.cpp:13-41), the
+ * packed bias add (nestedtensor/csrc/BinaryOps.cpp:97-107) and at::gelu / at::relu
+ * on the buffer (nestedtensor/csrc/activation.cpp:11-19, 34-46), plus an unwired
+ * add_bias_act kernel (nestedtensor/csrc/cuda/cuda_kernels.cu:73-107). */
+int nt_linear_act(const void* A, int64_t lda, const void* W, const void* bias, void* C,
+                  int64_t ldc, int64_t M, int64_t N, int64_t K, int act, int dtype, void* stream);
+
 /* Self/cross attention on packed projections, one softmax per (sequence, head)
  * over that sequence's own keys only:
  *   out[q_off[b] + i, h*hd + d] = sum_j softmax_j(scale * q_i . k_j) v_j[d]
@@ -250,6 +260,11 @@ int nt_add_packed(const void* a, const void* b, double alpha, void* out, int64_t
  * row_offsets are int64[B + 1] on the device; total_rows = row_offsets[B]. */
 int nt_softmax_rows(const void* x, void* out, const int64_t* offsets, const int64_t* row_offsets,
                     int64_t B, int64_t total_rows, int log_softmax, int dtype, void* stream);
+
+/* out[i] = relu(x[i]) (act 1) or gelu(x[i]) (act 2, erf form), fp32 arithmetic, one
+ * rounding: at::relu / at::gelu on the packed buffer, as NestedTensor_relu /
+ * NestedTensor_gelu do (nestedtensor/csrc/activation.cpp:11-19, 34-46). */
+int nt_activation_packed(const void* x, void* out, int64_t numel, int act, int dtype, void* stream);
 
 /* out[i] = scale * a[i] * b[i % period] in fp32, rounded once; b == NULL gives
  * out[i] = scale * a[i] (period is then ignored).  period == numel: nested *

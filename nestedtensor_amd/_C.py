@@ -49,6 +49,8 @@ SIGNATURES = {
     "nt_exclusive_scan_i32": (_int, [_c_void_p, _i64, _c_void_p, _c_void_p, _size_t, _c_void_p]),
     "nt_linear": (_int, [_c_void_p, _i64, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _i64,
                          _int, _c_void_p]),
+    "nt_linear_act": (_int, [_c_void_p, _i64, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _i64,
+                             _int, _int, _c_void_p]),
     "nt_linear_qkv": (_int, [_c_void_p, _i64, _c_void_p, _c_void_p, _c_void_p, _i64, _c_void_p, _i64, _i64,
                              _i64, _i64, _int, _c_void_p]),
     "nt_linear_transposed": (_int, [_c_void_p, _i64, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _i64,
@@ -62,6 +64,7 @@ SIGNATURES = {
                              _c_void_p]),
     "nt_add_packed": (_int, [_c_void_p, _c_void_p, _f64, _c_void_p, _i64, _i64, _int, _c_void_p]),
     "nt_softmax_rows": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _int, _int, _c_void_p]),
+    "nt_activation_packed": (_int, [_c_void_p, _c_void_p, _i64, _int, _int, _c_void_p]),
     "nt_mul_packed": (_int, [_c_void_p, _c_void_p, _f64, _c_void_p, _i64, _i64, _int, _c_void_p]),
     "nt_gather_rows": (_int, [_c_void_p, _i64, _i64, _c_void_p, _c_void_p, _i64, _c_void_p, _c_void_p]),
     "nt_packed_sequence_index": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _c_void_p, _c_void_p]),

@@ -19,6 +19,7 @@ from .nested.masking import from_padded_tensor
 from .nested.nested import NestedTensor
 from .nested.nested import transpose_nchw_nhwc
 from .nested.nested import transpose_nhwc_nchw
+from .nested.nested import linear_act
 
 from . import nested
 from . import nn

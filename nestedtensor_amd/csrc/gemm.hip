@@ -103,7 +103,16 @@ struct GemmArgs {
   T* Vt;            // QKV epilogue: transposed destination of columns >= n_split
   int64_t ldvt;
   int64_t n_split;
+  int act;          // row-major tiles: 0 none, 1 relu, 2 gelu (erf) applied to A W^T + bias
 };
+
+// The activation of a feed-forward layer, applied in fp32 before the one rounding
+// of the epilogue (wavefront-uniform switch; `act` is a kernel argument).
+__device__ __forceinline__ float apply_act(float v, int act) {
+  if (act == 1) return fmaxf(v, 0.0f);
+  if (act == 2) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f));
+  return v;
+}
 
 // 16-byte piece of a row at element k.
 // ALIGNED_K (K is a multiple of the K tile): branch-free and mask-free.
@@ -136,7 +145,10 @@ __device__ __forceinline__ u32x4 load_chunk(const T* base, int64_t ld, int64_t r
   return v;
 }
 
-enum { kEpiPlain = 0, kEpiQkv = 1 };
+// kEpiAct: the plain epilogue with the activation of GemmArgs::act; a kernel of
+// its own, because even a never-taken activation branch in the plain epilogue
+// costs the projection GEMMs 10 % (measured)
+enum { kEpiPlain = 0, kEpiQkv = 1, kEpiAct = 2 };
 
 // One BM x BN tile.  VT_OUT marks a V tile of the fused QKV projection, whose
 // result goes transposed into Vt.
@@ -150,7 +162,7 @@ enum { kEpiPlain = 0, kEpiQkv = 1 };
 // moves each 32-row strip through a private LDS region of the wavefront, 8 or
 // 16 bytes per lane in, and back out as 16-byte pieces of whole rows, so the
 // global stores are row-contiguous instead of 2 bytes per lane.
-template <typename T, class Cfg, bool VT_OUT, bool ALIGNED_K>
+template <typename T, class Cfg, bool VT_OUT, bool ALIGNED_K, bool ACT = false>
 __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int64_t n0, char* lds) {
   typedef Mma<T> MM;
   typedef typename MM::Frag Frag;
@@ -361,10 +373,17 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
           const int c0 = j * 32 + 8 * r + 4 * g;
           const float4 bv = *reinterpret_cast<const float4*>(lds_bias + wn * WN * 32 + c0);
           Quad q;
-          q[0] = (T)(acc[i][j][4 * r + 0] + bv.x);
-          q[1] = (T)(acc[i][j][4 * r + 1] + bv.y);
-          q[2] = (T)(acc[i][j][4 * r + 2] + bv.z);
-          q[3] = (T)(acc[i][j][4 * r + 3] + bv.w);
+          if (!ACT) {
+            q[0] = (T)(acc[i][j][4 * r + 0] + bv.x);
+            q[1] = (T)(acc[i][j][4 * r + 1] + bv.y);
+            q[2] = (T)(acc[i][j][4 * r + 2] + bv.z);
+            q[3] = (T)(acc[i][j][4 * r + 3] + bv.w);
+          } else {
+            q[0] = (T)apply_act(acc[i][j][4 * r + 0] + bv.x, a.act);
+            q[1] = (T)apply_act(acc[i][j][4 * r + 1] + bv.y, a.act);
+            q[2] = (T)apply_act(acc[i][j][4 * r + 2] + bv.z, a.act);
+            q[3] = (T)apply_act(acc[i][j][4 * r + 3] + bv.w, a.act);
+          }
           *reinterpret_cast<Quad*>(strip + l32 * kStripRow + c0 * (int)sizeof(T)) = q;
         }
       }
@@ -459,7 +478,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kWavesPerSimd) void linear_kern
   if (EPI == kEpiQkv && n0 >= a.n_split) {
     gemm_tile<T, Cfg, true, ALIGNED_K>(a, m0, n0, lds);    // V tile: transposed into Vt
   } else {
-    gemm_tile<T, Cfg, false, ALIGNED_K>(a, m0, n0, lds);
+    gemm_tile<T, Cfg, false, ALIGNED_K, EPI == kEpiAct>(a, m0, n0, lds);
   }
 }
 
@@ -559,7 +578,9 @@ static int launch_epi(const GemmArgs<T>& a, hipStream_t stream) {
 
 template <typename T>
 static int launch_linear(GemmArgs<T> a, bool qkv, hipStream_t stream) {
-  return qkv ? launch_epi<T, kEpiQkv>(a, stream) : launch_epi<T, kEpiPlain>(a, stream);
+  if (qkv) return launch_epi<T, kEpiQkv>(a, stream);
+  if (a.act != 0) return launch_epi<T, kEpiAct>(a, stream);
+  return launch_epi<T, kEpiPlain>(a, stream);
 }
 
 static int check_linear(const void* A, int64_t lda, const void* W, const void* C, int64_t ldc,
@@ -588,6 +609,7 @@ static GemmArgs<T> make_args(const void* A, int64_t lda, const void* W, const vo
   a.Vt = nullptr;
   a.ldvt = 0;
   a.n_split = N;
+  a.act = 0;
   return a;
 }
 
@@ -595,19 +617,33 @@ static GemmArgs<T> make_args(const void* A, int64_t lda, const void* W, const vo
 
 using namespace nt;
 
-extern "C" int nt_linear(const void* A, int64_t lda, const void* W, const void* bias, void* C,
-                         int64_t ldc, int64_t M, int64_t N, int64_t K, int dtype, void* stream) {
+extern "C" int nt_linear_act(const void* A, int64_t lda, const void* W, const void* bias, void* C,
+                             int64_t ldc, int64_t M, int64_t N, int64_t K, int act, int dtype,
+                             void* stream) {
   int rc = check_linear(A, lda, W, C, ldc, M, N, K);
   if (rc != NT_OK) return rc;
   if (ldc < N) return fail(NT_ERR_INVALID_ARGUMENT, "linear: ldc %lld < N %lld", (long long)ldc, (long long)N);
+  if (act < 0 || act > 2) return fail(NT_ERR_INVALID_ARGUMENT, "linear: activation %d is not 0, 1 or 2", act);
   if (M == 0 || N == 0) return NT_OK;
   hipStream_t s = (hipStream_t)stream;
+#define NT_LIN_CASE(TYPE)                                                   \
+  {                                                                         \
+    GemmArgs<TYPE> a = make_args<TYPE>(A, lda, W, bias, C, ldc, M, N, K);   \
+    a.act = act;                                                            \
+    return launch_linear<TYPE>(a, false, s);                                \
+  }
   switch (dtype) {
-    case NT_F32: return launch_linear<float>(make_args<float>(A, lda, W, bias, C, ldc, M, N, K), false, s);
-    case NT_F16: return launch_linear<_Float16>(make_args<_Float16>(A, lda, W, bias, C, ldc, M, N, K), false, s);
-    case NT_BF16: return launch_linear<__bf16>(make_args<__bf16>(A, lda, W, bias, C, ldc, M, N, K), false, s);
+    case NT_F32: NT_LIN_CASE(float)
+    case NT_F16: NT_LIN_CASE(_Float16)
+    case NT_BF16: NT_LIN_CASE(__bf16)
     default: return fail(NT_ERR_INVALID_ARGUMENT, "linear: unknown dtype %d", dtype);
   }
+#undef NT_LIN_CASE
+}
+
+extern "C" int nt_linear(const void* A, int64_t lda, const void* W, const void* bias, void* C,
+                         int64_t ldc, int64_t M, int64_t N, int64_t K, int dtype, void* stream) {
+  return nt_linear_act(A, lda, W, bias, C, ldc, M, N, K, 0, dtype, stream);
 }
 
 extern "C" int nt_linear_qkv(const void* A, int64_t lda, const void* W, const void* bias, void* QK,

@@ -374,6 +374,50 @@ static int launch_softmax(const void* x, void* out, const int64_t* offsets, cons
   return check_launch("softmax_rows_kernel");
 }
 
+// relu / gelu (erf) of every element of the packed buffer: the reference applies
+// at::relu / at::gelu to the buffer (nestedtensor/csrc/activation.cpp:11-19, 34-46)
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void activation_kernel(const T* __restrict__ x, T* __restrict__ out,
+                                                         int64_t numel, int act) {
+  constexpr int kPer = VEC ? 16 / sizeof(T) : 1;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x * kPer;
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * kPer; i < numel; i += stride) {
+    if (VEC) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(x + i);
+      T v[kPer];
+      __builtin_memcpy(v, &raw, 16);
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const float f = (float)v[j];
+        v[j] = (T)(act == 1 ? fmaxf(f, 0.0f) : 0.5f * f * (1.0f + erff(f * 0.70710678118654752f)));
+      }
+      u32x4 o;
+      __builtin_memcpy(&o, v, 16);
+      store16_stream(reinterpret_cast<char*>(out + i), o);
+    } else {
+      const float f = (float)x[i];
+      out[i] = (T)(act == 1 ? fmaxf(f, 0.0f) : 0.5f * f * (1.0f + erff(f * 0.70710678118654752f)));
+    }
+  }
+}
+
+template <typename T>
+static int launch_activation(const void* x, void* out, int64_t numel, int act, hipStream_t stream) {
+  constexpr int kPer = 16 / sizeof(T);
+  const bool vec = ((uintptr_t)x | (uintptr_t)out) % 16 == 0 && numel % kPer == 0;
+  const int64_t per_thread = vec ? kPer : 1;
+  int64_t blocks = (numel + 256 * per_thread - 1) / (256 * per_thread);
+  if (blocks > (1 << 20)) blocks = 1 << 20;
+  if (vec) {
+    hipLaunchKernelGGL((activation_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                       static_cast<const T*>(x), static_cast<T*>(out), numel, act);
+  } else {
+    hipLaunchKernelGGL((activation_kernel<T, false>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                       static_cast<const T*>(x), static_cast<T*>(out), numel, act);
+  }
+  return check_launch("activation_kernel");
+}
+
 // OP 0: out[i] = a[i] + alpha * b[i % period]   (period == numel: plain packed add)
 // OP 1: out[i] = alpha * a[i] * b[i % period], or alpha * a[i] when b is NULL
 enum { kBinAdd = 0, kBinMul = 1 };
@@ -482,6 +526,21 @@ extern "C" int nt_add_packed(const void* a, const void* b, double alpha, void* o
     case NT_F16: return launch_add<_Float16, kBinAdd>(a, b, alpha, out, numel, period, s);
     case NT_BF16: return launch_add<__bf16, kBinAdd>(a, b, alpha, out, numel, period, s);
     default: return fail(NT_ERR_UNSUPPORTED, "add_packed: dtype %d is not f32, f16 or bf16", dtype);
+  }
+}
+
+extern "C" int nt_activation_packed(const void* x, void* out, int64_t numel, int act, int dtype,
+                                    void* stream) {
+  if (numel < 0) return fail(NT_ERR_INVALID_ARGUMENT, "activation_packed: negative extent");
+  if (act != 1 && act != 2) return fail(NT_ERR_INVALID_ARGUMENT, "activation_packed: act %d is not 1 (relu) or 2 (gelu)", act);
+  if (numel == 0) return NT_OK;
+  if (!x || !out) return fail(NT_ERR_INVALID_ARGUMENT, "activation_packed: NULL pointer");
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case NT_F32: return launch_activation<float>(x, out, numel, act, s);
+    case NT_F16: return launch_activation<_Float16>(x, out, numel, act, s);
+    case NT_BF16: return launch_activation<__bf16>(x, out, numel, act, s);
+    default: return fail(NT_ERR_UNSUPPORTED, "activation_packed: dtype %d is not f32, f16 or bf16", dtype);
   }
 }
 

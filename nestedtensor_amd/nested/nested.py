@@ -379,13 +379,14 @@ class NestedTensor:
 def _nn_functional_linear(input, weight, bias=None):
     """nested.py:17-28 with the packed fast path of matmul.cpp:13-41: one GEMM
     on the packed [T, E] view."""
-    opt = input.opt_sizes()
-    if input.dim() != 3 or opt[2] is None:
-        raise NotImplementedError("linear on a NestedTensor needs dim 3 and a regular last dim.")
-    out = ops.linear(input.buffer.reshape(-1, opt[2]), weight, bias)
-    sizes = input.sizes.clone()
-    sizes[:, 1] = weight.size(0)
-    return NestedTensorImpl(out.reshape(-1), sizes)
+    return ops.linear_nt(input, weight, bias)
+
+
+def linear_act(input, weight, bias=None, activation="gelu"):
+    """act(F.linear(input, weight, bias)) on a NestedTensor in one launch: the
+    activation ('relu' or 'gelu', erf form) runs in the GEMM epilogue.  No
+    counterpart in the reference, which applies the three ops one after the other."""
+    return NestedTensor(ops.linear_nt(ops.contiguous(input._impl), weight, bias, activation))
 
 
 def transpose_nchw_nhwc(tensor):
@@ -447,6 +448,18 @@ def _to_nested_tensor(impl, dim=None):
     if d % nd < impl.nested_dim():
         return impl
     raise RuntimeError("Only nested_dim of 1 is currently supported.")
+
+
+def _relu(input, inplace=False):
+    if inplace:
+        raise NotImplementedError("relu on a NestedTensor is not done in place.")
+    return ops.activation(input, "relu")
+
+
+def _gelu(input, approximate="none"):
+    if approximate != "none":
+        raise NotImplementedError("gelu on a NestedTensor: only the erf form is implemented.")
+    return ops.activation(input, "gelu")
 
 
 def _to_tensor_list(impl):
@@ -514,6 +527,10 @@ _HANDLERS = {
     torch.Tensor.add: _add,
     torch.Tensor.__add__: _add,
     torch.Tensor.__radd__: _add,
+    torch.nn.functional.relu: _relu,
+    torch.relu: _relu,
+    torch.Tensor.relu: _relu,
+    torch.nn.functional.gelu: _gelu,
     torch.unbind: _unbind,
     torch.Tensor.unbind: _unbind,
     torch.nn.functional.softmax: _softmax,
@@ -535,6 +552,6 @@ _HANDLERS = {
 # size); every other handler is given row-major operands
 _LAYOUT_AWARE = {
     _unbind, _to_nested_tensor, _to_tensor_list, _get_max_size, _is_nested_tensor_impl, _nested_dim, _sizes, _len, _get_dim, _get_numel,
-    ops.is_contiguous, ops.contiguous, ops.conv2d, ops.max_pool2d, _add, _mul,
+    ops.is_contiguous, ops.contiguous, ops.conv2d, ops.max_pool2d, _add, _mul, _relu, _gelu,
     ops.transpose_nchw_nhwc, ops.transpose_nhwc_nchw,
 }

@@ -350,12 +350,18 @@ def pack_device(tensors, offsets_dev, total, dtype, device):
 # nested multi-head attention
 
 
-def linear(x, weight, bias):
-    """y = x @ weight.T + bias on a 2-D row-major view (nt_linear).  This is the
-    packed fast path of NestedTensor_matmul (matmul.cpp:13-41) with the packed
-    bias add (BinaryOps.cpp:97-107) fused into the GEMM epilogue."""
+_ACTS = {None: 0, "none": 0, "relu": 1, "gelu": 2}
+
+
+def linear(x, weight, bias, activation=None):
+    """y = act(x @ weight.T + bias) on a 2-D row-major view (nt_linear_act).  This
+    is the packed fast path of NestedTensor_matmul (matmul.cpp:13-41) with the
+    packed bias add (BinaryOps.cpp:97-107) and, optionally, relu / gelu
+    (activation.cpp:11-19, 34-46) fused into the GEMM epilogue."""
     _C.require_device(x, "linear")
     assert x.dim() == 2 and weight.dim() == 2 and x.stride(1) == 1
+    if activation not in _ACTS:
+        raise RuntimeError("linear: activation must be None, 'relu' or 'gelu', got %r" % (activation,))
     M, K = x.shape
     N = weight.size(0)
     if weight.size(1) != K:
@@ -368,10 +374,36 @@ def linear(x, weight, bias):
         bias = bias.contiguous()
     out = torch.empty((M, N), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
-        _C.check(_C.lib.nt_linear(
+        _C.check(_C.lib.nt_linear_act(
             _C.ptr(x), x.stride(0), _C.ptr(weight), _C.ptr(bias), _C.ptr(out), N, M, N, K,
-            _C.dtype_code(x.dtype), _C.current_stream(x.device)))
+            _ACTS[activation], _C.dtype_code(x.dtype), _C.current_stream(x.device)))
     return out
+
+
+def linear_nt(impl, weight, bias=None, activation=None):
+    """F.linear on a NestedTensor [B, L_i, K] (nested.py:17-28): one GEMM on the
+    packed [T, K] view, with an optional fused activation."""
+    opt = impl.opt_sizes()
+    if impl.dim() != 3 or opt[2] is None:
+        raise NotImplementedError("linear on a NestedTensor needs dim 3 and a regular last dim.")
+    out = linear(impl.buffer.reshape(-1, opt[2]), weight, bias, activation)
+    sizes = impl.sizes.clone()
+    sizes[:, 1] = weight.size(0)
+    return NestedTensorImpl(out.reshape(-1), sizes)
+
+
+def activation(impl, kind):
+    """relu / gelu of a NestedTensor: one launch over the packed buffer
+    (NestedTensor_relu / NestedTensor_gelu, activation.cpp:11-19, 34-46); the
+    storage layout does not matter."""
+    buf = impl.buffer
+    _C.require_device(buf, kind)
+    out = torch.empty_like(buf)
+    if buf.numel() > 0:
+        with torch.cuda.device(buf.device):
+            _C.check(_C.lib.nt_activation_packed(_C.ptr(buf), _C.ptr(out), buf.numel(), _ACTS[kind],
+                                                 _C.dtype_code(buf.dtype), _C.current_stream(buf.device)))
+    return impl.with_buffer(out)
 
 
 def _check_mha_inputs(query, key, value):

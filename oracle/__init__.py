@@ -54,6 +54,8 @@ Pinning (what each part was checked against, see tests/test_oracle_*.py):
 * softmax: rows sum to 1, invariance to a per-row shift, the closed form
   ``exp(x) / sum(exp(x))`` in fp64 written out with Python loops, and
   ``log_softmax == log(softmax)`` (tests/test_oracle_rowops.py).
+* activation: relu against ``max(x, 0)``, gelu against the closed form
+  ``x/2 (1 + erf(x / sqrt 2))`` with math.erf in fp64 (tests/test_oracle_rowops.py).
 * mul / matmul: per-constituent ``torch.mul`` / ``torch.matmul`` are the
   reference's own definition (BinaryOps.cpp:296-299, matmul.cpp:44-49); pinned
   against hand-computed values and an fp64 product in tests/test_oracle_rowops.py.
@@ -82,7 +84,7 @@ from .masking import (  # noqa: F401
     nested_tensor_from_padded_tensor,
 )
 from .mha import min_mha, bt_min_mha  # noqa: F401
-from .rowops import layer_norm, add, mul, matmul, softmax  # noqa: F401
+from .rowops import layer_norm, add, mul, matmul, softmax, activation  # noqa: F401
 from .dense import max_pool2d, conv2d  # noqa: F401
 from .interop import (  # noqa: F401
     embedding, embedding_bag, to_sparse_csr, to_packed_sequence, transpose_nchw_nhwc, transpose_nhwc_nchw,

@@ -85,3 +85,10 @@ def softmax(nt, dim, dtype=None, log=False):
     fn = torch.log_softmax if log else torch.softmax
     outs = [fn(t, dim - 1, dtype=dtype) for t in nt.unbind()]
     return RefNestedTensor(outs, outs[0].dtype if outs else nt.dtype)
+
+
+def activation(nt, kind):
+    """NestedTensor_relu / NestedTensor_gelu (activation.cpp:11-19, 34-46): at::relu
+    / at::gelu (erf form) per constituent."""
+    fn = {"relu": torch.relu, "gelu": torch.nn.functional.gelu}[kind]
+    return RefNestedTensor([fn(t) for t in nt.unbind()], nt.dtype)

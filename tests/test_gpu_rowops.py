@@ -151,6 +151,46 @@ def test_softmax_last_dim(dtype, log):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_relu_gelu_packed(dtype):
+    import torch.nn.functional as F
+    for shapes in ([(3, 40), (7, 40), (1, 40)], [(3, 7), (2, 7)], [(2, 3, 5, 4), (2, 1, 2, 4)]):
+        ts = [t * 2 for t in _tensors(shapes, dtype, 40)]
+        a = nt.nested_tensor(ts, device=DEV, dtype=dtype)
+        ref = oracle.ref_nested_tensor(ts, dtype=dtype)
+        assert torch.equal(F.relu(a)._impl.buffer.cpu(), oracle.activation(ref, "relu").buffer)
+        assert torch.equal(torch.relu(a)._impl.buffer.cpu(), oracle.activation(ref, "relu").buffer)
+        got = F.gelu(a)
+        exp = oracle.activation(oracle.ref_nested_tensor([t.float() for t in ts], dtype=torch.float32), "gelu")
+        assert got.nested_size() == a.nested_size()
+        err = (got._impl.buffer.float().cpu() - exp.buffer).abs().max().item()
+        assert err <= (1e-5 if dtype == torch.float32 else 2e-2), err
+        assert torch.equal(torch.nn.GELU()(a)._impl.buffer, got._impl.buffer)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("act", ["relu", "gelu"])
+def test_linear_act_equals_linear_then_activation(dtype, act):
+    import torch.nn.functional as F
+    K, N = 64, 200
+    ts = _tensors([(5, K), (300, K), (1, K)], dtype, 41)
+    w = (torch.randn(N, K, generator=torch.Generator().manual_seed(42)) * 0.3).to(dtype)
+    b = torch.randn(N, generator=torch.Generator().manual_seed(43)).to(dtype)
+    a = nt.nested_tensor(ts, device=DEV, dtype=dtype)
+    fused = nt.linear_act(a, w.to(DEV), b.to(DEV), activation=act)
+    xs = oracle.ref_nested_tensor([t.float() for t in ts], dtype=torch.float32)
+    lin = oracle.ref_nested_tensor([F.linear(t, w.float(), b.float()) for t in xs.unbind()], dtype=torch.float32)
+    exp = oracle.activation(lin, act)
+    assert [tuple(x.shape) for x in fused.unbind()] == [tuple(x.shape) for x in exp.unbind()]
+    err = (fused._impl.buffer.float().cpu() - exp.buffer).abs().max().item()
+    assert err <= (1e-5 if dtype == torch.float32 else 2e-2) * max(1.0, exp.buffer.abs().max().item()), err
+    # the fused launch rounds once; applying the activation to the rounded linear output
+    # may differ by that rounding only
+    two = (F.relu if act == "relu" else F.gelu)(F.linear(a, w.to(DEV), b.to(DEV)))
+    d = (fused._impl.buffer.float() - two._impl.buffer.float()).abs().max().item()
+    assert d <= (1e-5 if dtype == torch.float32 else 2e-2) * max(1.0, exp.buffer.abs().max().item())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 def test_matmul_packed_fast_path(dtype):
     # matmul.cpp:13-41: nested [B, L_i, K] x dense [K, N] is one GEMM on the packed buffer
     K, N = 64, 96

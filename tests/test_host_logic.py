@@ -184,8 +184,10 @@ def test_compute_ops_refuse_host_tensors():
     mha = torch.nn.MultiheadAttention(3, 1).eval()
     with pytest.raises(RuntimeError, match="HIP device only"):
         mha(a, a, a)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError, match="HIP device only"):
         torch.relu(a)
+    with pytest.raises(NotImplementedError):
+        torch.sigmoid(a)
 
 
 def test_mask_collapse_closed_form_matches_oracle():

@@ -119,3 +119,13 @@ def test_softmax_closed_forms():
     # dims other than the last follow at::softmax per constituent too (SoftMax.cpp:24-27)
     other = oracle.softmax(a, 1)
     assert torch.allclose(other.unbind()[0].sum(0), torch.ones(3, 5), atol=1e-6)
+
+
+def test_activation_closed_forms():
+    import math
+    x = _nt([(3, 8), (5, 8)], seed=9)
+    r = oracle.activation(x, "relu")
+    assert torch.equal(r.buffer, torch.clamp(x.buffer, min=0))
+    ge = oracle.activation(x, "gelu")
+    exp = torch.tensor([0.5 * v * (1.0 + math.erf(v / math.sqrt(2.0))) for v in x.buffer.double().tolist()])
+    assert (ge.buffer.double() - exp).abs().max() < 1e-6
