@@ -110,7 +110,7 @@ struct GemmArgs {
 // of the epilogue (wavefront-uniform switch; `act` is a kernel argument).
 __device__ __forceinline__ float apply_act(float v, int act) {
   if (act == 1) return fmaxf(v, 0.0f);
-  if (act == 2) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f));
+  if (act == 2) return gelu_erf(v);
   return v;
 }
 

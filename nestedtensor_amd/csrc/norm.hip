@@ -389,14 +389,14 @@ __global__ __launch_bounds__(256) void activation_kernel(const T* __restrict__ x
 #pragma unroll
       for (int j = 0; j < kPer; ++j) {
         const float f = (float)v[j];
-        v[j] = (T)(act == 1 ? fmaxf(f, 0.0f) : 0.5f * f * (1.0f + erff(f * 0.70710678118654752f)));
+        v[j] = (T)(act == 1 ? fmaxf(f, 0.0f) : gelu_erf(f));
       }
       u32x4 o;
       __builtin_memcpy(&o, v, 16);
       store16_stream(reinterpret_cast<char*>(out + i), o);
     } else {
       const float f = (float)x[i];
-      out[i] = (T)(act == 1 ? fmaxf(f, 0.0f) : 0.5f * f * (1.0f + erff(f * 0.70710678118654752f)));
+      out[i] = (T)(act == 1 ? fmaxf(f, 0.0f) : gelu_erf(f));
     }
   }
 }
