@@ -54,6 +54,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-mha", action="store_true", help="skip the C3 attention leg")
     ap.add_argument("--no-rows", action="store_true", help="skip the per-row measurements (C1, C2, C4)")
+    ap.add_argument("--no-encoder", action="store_true",
+                    help="skip the whole-encoder-layer figure of the attention leg (so that a kernel "
+                         "trace of that leg holds the three kernels of the attention layer only)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="one plain copy of known size, then one pad and one un-pad launch of the "
                          "first C5 chunk; meant to run under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
@@ -309,18 +312,19 @@ def bench_mha_c3(args, torch, dev):
         o = _ops.linear_nt(f, W2, b2)
         return _ops.layer_norm(o, (E,), ln_w, ln_b, 1e-5, residual=h)
 
-    ms_enc = _time_gpu(torch, encoder_layer, iters=50, warmup=5)
+    ms_enc = None if args.no_encoder else _time_gpu(torch, encoder_layer, iters=50, warmup=5)
     flops_enc = flops + 16 * T * E * E
     res = dict(workload="C3: nested BERT-base self-attention, fp16, B=32, L~U[32,512], d=768, 12x64",
                tokens=T, ms_per_layer=ms, ms_per_layer_hip_graph=graph_ms, tokens_per_s=T / (ms * 1e-3), flops=flops,
                roofline=dict(bound="mfma", achieved=flops / (ms * 1e-3) / 1e12, peak=MFMA_F16_PEAK_TFLOPS,
                              unit="TFLOP/s", frac=flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS))
-    res["encoder_layer"] = dict(
-        workload="the same batch through a whole BERT-base encoder layer (attention, add + layer norm, "
-                 "768-3072-768 feed-forward with gelu, add + layer norm), 7 launches",
-        ms_per_layer=ms_enc, tokens_per_s=T / (ms_enc * 1e-3), flops=flops_enc,
-        TFLOPs=flops_enc / (ms_enc * 1e-3) / 1e12,
-        frac_of_mfma_peak=flops_enc / (ms_enc * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS)
+    if ms_enc is not None:
+        res["encoder_layer"] = dict(
+            workload="the same batch through a whole BERT-base encoder layer (attention, add + layer norm, "
+                     "768-3072-768 feed-forward with gelu, add + layer norm), 7 launches",
+            ms_per_layer=ms_enc, tokens_per_s=T / (ms_enc * 1e-3), flops=flops_enc,
+            TFLOPs=flops_enc / (ms_enc * 1e-3) / 1e12,
+            frac_of_mfma_peak=flops_enc / (ms_enc * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS)
     if not args.no_cpu:
         torch.set_num_threads(os.cpu_count() or 1)
         ref = oracle.ref_nested_tensor(xs, dtype=torch.float16)
