@@ -315,6 +315,40 @@ def test_from_padded_tensor_length_based(dims, dtype):
     bits_equal(back2._impl.buffer, ref.buffer)
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_shapes_sweep_against_oracle(seed):
+    """Many small random nested tensors (1 to 3 constituent dims, extents 1..37 so
+    that every alignment of rows and of the valid / pad boundary turns up, some
+    dims regular at random, five element sizes): pad, mask and both inverses
+    against the oracle, bit for bit."""
+    g = torch.Generator().manual_seed(9000 + seed)
+    dtypes = [torch.float32, torch.float16, torch.uint8, torch.int64, torch.bfloat16, torch.float64]
+    for case in range(40):
+        D = int(torch.randint(1, 4, (1,), generator=g))
+        B = int(torch.randint(1, 9, (1,), generator=g))
+        dtype = dtypes[int(torch.randint(0, len(dtypes), (1,), generator=g))]
+        regular = [bool(torch.randint(0, 3, (1,), generator=g) == 0) for _ in range(D)]
+        fixed = [int(torch.randint(1, 38, (1,), generator=g)) for _ in range(D)]
+        parts = []
+        for _ in range(B):
+            shape = [fixed[k] if regular[k] else int(torch.randint(1, 38, (1,), generator=g)) for k in range(D)]
+            parts.append((torch.randn(*shape, generator=g) * 50).to(dtype))
+        a = nt.nested_tensor(parts, device=DEV, dtype=dtype)
+        ref = oracle.ref_nested_tensor(parts, dtype=dtype)
+        pad_value = 3 if dtype in (torch.uint8, torch.int64) else -1.5
+        padded = a.to_padded_tensor(pad_value)
+        bits_equal(padded, oracle.to_padded_tensor(ref, pad_value))
+        data, mask = a.to_tensor_mask()
+        exp_d, exp_m = oracle.to_tensor_mask(ref)
+        bits_equal(data, exp_d)
+        assert mask.shape == exp_m.shape and torch.equal(mask.cpu(), exp_m.to(torch.bool)), (case, parts[0].shape)
+        back = nt.from_padded_tensor(padded, a)
+        bits_equal(back._impl.buffer, ref.buffer)
+        full_mask = torch.ops.nestedtensor.to_mask(a, a.dim())
+        again = nt.nested_tensor_from_tensor_mask(data, full_mask)
+        nt_matches(again, parts, dtype)
+
+
 def test_pad_nt_to_a_given_shape():
     # pad_nt (masking.cpp:138-179): a caller-given goal shape, data padded with 0, full-shape mask
     parts = [torch.randn(3, 5), torch.randn(1, 5), torch.randn(4, 2)]
