@@ -207,8 +207,8 @@ int nt_linear_transposed(const void* A, int64_t lda, const void* W, const void* 
                          int64_t ldct, int64_t M, int64_t N, int64_t K, int dtype, void* stream);
 
 /* Attention on projections in the layout the GEMMs above write: Q rows at
- * q[token * ldq + h*64], K rows at k[token * ldk + h*64], V transposed in
- * Vt[(h*64 + d) * ldvt + token]; head_dim is 64, dtype f16 or bf16.  For
+ * q[token * ldq + h*hd], K rows at k[token * ldk + h*hd], V transposed in
+ * Vt[(h*hd + d) * ldvt + token]; head_dim hd is 32, 64 or 128, dtype f16 or bf16.  For
  * self-attention on the output of nt_linear_qkv, q = QK, k = QK + E, ldq = ldk =
  * ldqk.  `schedule` is a device array of n_work int32[8] work items {first query
  * token, query length, first query row of the tile (multiple of 128), 0, first
@@ -221,8 +221,8 @@ int nt_linear_transposed(const void* A, int64_t lda, const void* W, const void* 
  * semantics as nt_varlen_attention. */
 int nt_varlen_attention_vt(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* vt,
                            int64_t ldvt, void* out, int64_t ldo, const int32_t* schedule,
-                           int64_t n_work, int64_t num_heads, int64_t total_kv_tokens, float scale,
-                           int dtype, void* stream);
+                           int64_t n_work, int64_t num_heads, int64_t head_dim,
+                           int64_t total_kv_tokens, float scale, int dtype, void* stream);
 
 /* ---- row-wise ops on the packed buffer (the steps either side of attention
  *      in an encoder layer) ------------------------------------------------ */

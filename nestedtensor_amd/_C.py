@@ -56,7 +56,7 @@ SIGNATURES = {
     "nt_linear_transposed": (_int, [_c_void_p, _i64, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _i64,
                                     _int, _c_void_p]),
     "nt_varlen_attention_vt": (_int, [_c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64,
-                                      _c_void_p, _i64, _i64, _i64, _f32, _int, _c_void_p]),
+                                      _c_void_p, _i64, _i64, _i64, _i64, _f32, _int, _c_void_p]),
     "nt_varlen_attention": (_int, [_c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64,
                                    _c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _f32, _int,
                                    _c_void_p]),

@@ -301,16 +301,27 @@ __global__ __launch_bounds__(256) void varlen_attention_kernel(
 #define NT_ATTN_WAVES_PER_EU 3
 #endif
 
-template <typename T>
-__global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt_kernel(
+// HD: head_dim, 32, 64 or 128.  Per key tile a workgroup stages 64 K rows of HD
+// elements and HD V^T rows of 64 keys; a wavefront holds HD / 16 Q fragments and
+// HD / 32 output accumulator blocks.  The benchmark shapes have HD = 64; 128 needs
+// about 200 registers per lane, so two wavefronts per SIMD there.
+template <typename T, int HD>
+__global__ __launch_bounds__(256, (HD > 64 ? 2 : NT_ATTN_WAVES_PER_EU)) void varlen_attention_vt_kernel(
     const T* __restrict__ Q, int64_t ldq, const T* __restrict__ K, int64_t ldk,
     const T* __restrict__ Vt, int64_t ldvt, T* __restrict__ O, int64_t ldo,
     const int4* __restrict__ schedule, unsigned num_heads, float scale_log2e) {
   typedef AttnT<T> AT;
   typedef typename AT::Frag Frag;
 
-  __shared__ __align__(16) char lds_k[2][kKBytes];
-  __shared__ __align__(16) char lds_v[2][kVBytes + kVRow];   // row 64: ones (see below)
+  constexpr int kKR = HD * 2 + 16;          // LDS bytes per K row (16 pad: conflict-free fragment reads)
+  constexpr int kQF = HD / 16;              // Q fragments = MFMA k-steps of the score product
+  constexpr int kDB = HD / 32;              // 32-row blocks of O^T
+  constexpr int kKPieces = HD / 8;          // 16-byte pieces per K row
+  constexpr int kKRowsPerPass = 256 / kKPieces;
+  constexpr int kKP = kKTile / kKRowsPerPass;   // K pieces per thread and tile
+  constexpr int kVP = HD / 32;              // V^T pieces per thread and tile (8 per row, 32 rows a pass)
+  __shared__ __align__(16) char lds_k[2][kKTile * kKR];
+  __shared__ __align__(16) char lds_v[2][(HD + 1) * kVRow];   // row HD: ones (see below)
 
   // Head fastest: the schedule lists the longest sequences first, and this way
   // their items of ALL heads are dispatched before any short item (with the
@@ -336,51 +347,54 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
 
   const int q_row = q0 + wave * 32 + l32;
   const bool wave_active = (q0 + wave * 32) < Lq;
-  Frag qf[4];
+  Frag qf[kQF];
   {
     // rows past Lq read the last row; their results are never stored
     const int qr = q_row < Lq ? q_row : Lq - 1;
-    const T* qp = Q + (q_begin + qr) * ldq + h * kHd + g * 8;
+    const T* qp = Q + (q_begin + qr) * ldq + h * HD + g * 8;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
+    for (int s = 0; s < kQF; ++s) {
       u32x4 v = load16_unaligned(reinterpret_cast<const char*>(qp + s * 16));
       __builtin_memcpy(&qf[s], &v, 16);
     }
   }
 
-  acc16 o_acc[2];
+  acc16 o_acc[kDB];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < kDB; ++i)
 #pragma unroll
     for (int e = 0; e < 16; ++e) o_acc[i][e] = 0.0f;
   float m_run = -INFINITY;
 
   const int ntiles = (L + kKTile - 1) / kKTile;
-  const T* kbase = K + begin * ldk + h * kHd;
-  const T* vbase = Vt + (int64_t)h * kHd * ldvt + begin;
+  const T* kbase = K + begin * ldk + h * HD;
+  const T* vbase = Vt + (int64_t)h * HD * ldvt + begin;
 
-  // Each thread moves two 16-byte pieces of a K tile and two of a V^T tile.
+  // Each thread moves HD / 32 16-byte pieces of a K tile and as many of a V^T tile.
   // The loads are unconditional and unmasked (clamped addresses), so that the
   // wavefront only waits for them where the data is stored to LDS.  All per-thread
   // addressing is set up once; a step only advances pointers.
-  const int r0 = tid >> 3;      // row of piece 0 (piece 1: r0 + 32)
+  const int r0 = tid >> 3;      // V^T: row of piece 0 (piece i: r0 + 32 i), keys 8 cc .. 8 cc + 7
   const int cc = tid & 7;
-  u32x4 rk[2], rv[2];
-  const char* k_last = reinterpret_cast<const char*>(kbase + (int64_t)(L - 1) * ldk + cc * 8);
+  const int kr0 = tid / kKPieces;   // K: row of piece 0 (piece i: kr0 + i * kKRowsPerPass)
+  const int kc = tid % kKPieces;    //    elements 8 kc .. 8 kc + 7 of the row
+  u32x4 rk[kKP], rv[kVP];
+  const char* k_last = reinterpret_cast<const char*>(kbase + (int64_t)(L - 1) * ldk + kc * 8);
   const int64_t k_step = (int64_t)kKTile * ldk * (int64_t)sizeof(T);
-  const char* v_ptr[2];
+  const char* v_ptr[kVP];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < kVP; ++i) {
     v_ptr[i] = reinterpret_cast<const char*>(vbase + (int64_t)(r0 + i * 32) * ldvt + cc * 8);
   }
   auto gload_k = [&](int t_in) {
     const int t = t_in < ntiles ? t_in : ntiles - 1;   // past the end: re-read, never used
-    const char* tile = reinterpret_cast<const char*>(kbase + cc * 8) + t * k_step;
+    const char* tile = reinterpret_cast<const char*>(kbase + kc * 8) + t * k_step;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < kKP; ++i) {
       // rows past L read row L - 1 (a valid key: it cannot raise the row maximum)
-      const int kr = t * kKTile + r0 + i * 32;
-      const char* src = tile + (int64_t)(r0 + i * 32) * ldk * (int64_t)sizeof(T);
+      const int row = kr0 + i * kKRowsPerPass;
+      const int kr = t * kKTile + row;
+      const char* src = tile + (int64_t)row * ldk * (int64_t)sizeof(T);
       rk[i] = load16_unaligned(kr < L ? src : k_last);
     }
   };
@@ -389,13 +403,15 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
     // V^T piece: keys key0 .. key0+7 of row d, read where it lies (the rows of Vt
     // are readable 72 elements past the last token)
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < kVP; ++i) {
       rv[i] = load16_unaligned(v_ptr[i] + t * (kKTile * (int)sizeof(T)));
     }
   };
   auto lstore_k = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) store16(&lds_k[buf][(r0 + i * 32) * kKRow + cc * 16], rk[i]);
+    for (int i = 0; i < kKP; ++i) {
+      store16(&lds_k[buf][(kr0 + i * kKRowsPerPass) * kKR + kc * 16], rk[i]);
+    }
   };
   // piece cc = keys 8cc .. 8cc+7 = (ks = cc/2, a = cc%2); its low half (g = 0)
   // goes to position 16ks + 4a, its high half (g = 1) to 16ks + 8 + 4a.
@@ -420,7 +436,7 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
     const uint64_t ones = ((uint64_t)AT::kOnePair << 32) | AT::kOnePair;
 #pragma unroll
     for (int b2 = 0; b2 < 2; ++b2) {
-      char* row = &lds_v[b2][kHd * kVRow + v_lo];
+      char* row = &lds_v[b2][HD * kVRow + v_lo];
       *reinterpret_cast<uint64_t*>(row) = ones;
       *reinterpret_cast<uint64_t*>(row + 16) = ones;
     }
@@ -428,7 +444,7 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
   auto lstore_v = [&](int buf, int t) {
     if (t < ntiles - 1) {   // uniform: a full tile, nothing to mask
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < kVP; ++i) {
         char* row = &lds_v[buf][(r0 + i * 32) * kVRow + v_lo];
         *reinterpret_cast<uint64_t*>(row) = ((uint64_t)rv[i].y << 32) | rv[i].x;
         *reinterpret_cast<uint64_t*>(row + 16) = ((uint64_t)rv[i].w << 32) | rv[i].z;
@@ -436,7 +452,7 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
       return;
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < kVP; ++i) {
       char* row = &lds_v[buf][(r0 + i * 32) * kVRow + v_lo];
       const uint64_t lo = ((uint64_t)(rv[i].y & vm[1]) << 32) | (rv[i].x & vm[0]);
       const uint64_t hi = ((uint64_t)(rv[i].w & vm[3]) << 32) | (rv[i].z & vm[2]);
@@ -444,7 +460,7 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
       *reinterpret_cast<uint64_t*>(row + 16) = hi;
     }
     if (r0 == 0) {
-      char* row = &lds_v[buf][kHd * kVRow + v_lo];
+      char* row = &lds_v[buf][HD * kVRow + v_lo];
       const uint64_t lo = ((uint64_t)(AT::kOnePair & vm[1]) << 32) | (AT::kOnePair & vm[0]);
       const uint64_t hi = ((uint64_t)(AT::kOnePair & vm[3]) << 32) | (AT::kOnePair & vm[2]);
       *reinterpret_cast<uint64_t*>(row) = lo;
@@ -459,9 +475,9 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
     for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) sa[kb][e] = 0.0f;
-      const char* krow = &lds_k[buf][(kb * 32 + l32) * kKRow + g * 16];
+      const char* krow = &lds_k[buf][(kb * 32 + l32) * kKR + g * 16];
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
+      for (int s = 0; s < kQF; ++s) {
         Frag kf = *reinterpret_cast<const Frag*>(krow + s * 32);
         sa[kb] = AT::mma(kf, qf[s], sa[kb]);
       }
@@ -493,7 +509,7 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
     // every lane and the multiplications are skipped (wavefront-uniform)
     if (__any(alpha != 1.0f)) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < kDB; ++i)
 #pragma unroll
         for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
       l_acc[0] *= alpha;   // every element of l_acc holds the same sum; [0] is the one read
@@ -518,13 +534,13 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
-      for (int db = 0; db < 2; ++db) {
+      for (int db = 0; db < kDB; ++db) {
         const char* vrow = &lds_v[vbuf][(db * 32 + l32) * kVRow + g * 16];
         Frag vf = *reinterpret_cast<const Frag*>(vrow + ks * 32);
         o_acc[db] = AT::mma(vf, pf[ks], o_acc[db]);
       }
       // all 32 rows of this A-operand are the ones row: every lane gets l[q]
-      Frag of = *reinterpret_cast<const Frag*>(&lds_v[vbuf][kHd * kVRow + g * 16 + ks * 32]);
+      Frag of = *reinterpret_cast<const Frag*>(&lds_v[vbuf][HD * kVRow + g * 16 + ks * 32]);
       l_acc = AT::mma(of, pf[ks], l_acc);
     }
   };
@@ -557,9 +573,9 @@ __global__ __launch_bounds__(256, NT_ATTN_WAVES_PER_EU) void varlen_attention_vt
   if (!wave_active || q_row >= Lq) return;
   const float l_tot = l_acc[0];
   const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
-  T* op = O + (q_begin + q_row) * ldo + h * kHd;
+  T* op = O + (q_begin + q_row) * ldo + h * HD;
 #pragma unroll
-  for (int db = 0; db < 2; ++db) {
+  for (int db = 0; db < kDB; ++db) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       // d = 32 db + 8 r + 4 g + (0..3)
@@ -726,19 +742,35 @@ extern "C" int nt_varlen_attention(const void* q, int64_t ldq, const void* k, in
   }
 }
 
+template <typename T, int HD>
+static void launch_vt(dim3 grid, hipStream_t s, const void* q, int64_t ldq, const void* k, int64_t ldk,
+                      const void* vt, int64_t ldvt, void* out, int64_t ldo, const int4* sched,
+                      unsigned num_heads, float scale_log2e) {
+  hipLaunchKernelGGL((varlen_attention_vt_kernel<T, HD>), grid, dim3(256), 0, s, static_cast<const T*>(q),
+                     ldq, static_cast<const T*>(k), ldk, static_cast<const T*>(vt), ldvt,
+                     static_cast<T*>(out), ldo, sched, num_heads, scale_log2e);
+}
+
 extern "C" int nt_varlen_attention_vt(const void* q, int64_t ldq, const void* k, int64_t ldk,
                                       const void* vt, int64_t ldvt, void* out, int64_t ldo,
                                       const int32_t* schedule, int64_t n_work, int64_t num_heads,
-                                      int64_t total_kv_tokens, float scale, int dtype, void* stream) {
+                                      int64_t head_dim, int64_t total_kv_tokens, float scale, int dtype,
+                                      void* stream) {
   if (n_work < 0 || num_heads < 1 || total_kv_tokens < 0) {
     return fail(NT_ERR_INVALID_ARGUMENT, "attention_vt: bad shape");
+  }
+  if (head_dim != 32 && head_dim != 64 && head_dim != 128) {
+    return fail(NT_ERR_UNSUPPORTED, "attention_vt: head_dim %lld is not 32, 64 or 128", (long long)head_dim);
+  }
+  if (dtype != NT_F16 && dtype != NT_BF16) {
+    return fail(NT_ERR_UNSUPPORTED, "attention_vt: dtype must be f16 or bf16");
   }
   if (n_work == 0) return NT_OK;
   if (!q || !k || !vt || !out || !schedule) return fail(NT_ERR_INVALID_ARGUMENT, "attention_vt: NULL pointer");
   if (n_work > 0x3fffffffLL || num_heads > 65535 || total_kv_tokens > 0x7fffffffLL) {
     return fail(NT_ERR_UNSUPPORTED, "attention_vt: too many work items, heads or tokens");
   }
-  const int64_t E = num_heads * kHd;
+  const int64_t E = num_heads * head_dim;
   if (ldq < E || ldk < E || ldo < E || ldvt < total_kv_tokens + 72) {
     return fail(NT_ERR_INVALID_ARGUMENT,
                 "attention_vt: row strides too small (ldvt must be >= total_kv_tokens + 72)");
@@ -750,18 +782,17 @@ extern "C" int nt_varlen_attention_vt(const void* q, int64_t ldq, const void* k,
   const float scale_log2e = scale * 1.4426950408889634f;
   hipStream_t s = (hipStream_t)stream;
   const int4* sched = reinterpret_cast<const int4*>(schedule);
+  const unsigned nh = (unsigned)num_heads;
+#define NT_VT_ARGS grid, s, q, ldq, k, ldk, vt, ldvt, out, ldo, sched, nh, scale_log2e
   if (dtype == NT_F16) {
-    hipLaunchKernelGGL((varlen_attention_vt_kernel<_Float16>), grid, dim3(256), 0, s,
-                       static_cast<const _Float16*>(q), ldq, static_cast<const _Float16*>(k), ldk,
-                       static_cast<const _Float16*>(vt), ldvt, static_cast<_Float16*>(out), ldo,
-                       sched, (unsigned)num_heads, scale_log2e);
-  } else if (dtype == NT_BF16) {
-    hipLaunchKernelGGL((varlen_attention_vt_kernel<__bf16>), grid, dim3(256), 0, s,
-                       static_cast<const __bf16*>(q), ldq, static_cast<const __bf16*>(k), ldk,
-                       static_cast<const __bf16*>(vt), ldvt, static_cast<__bf16*>(out), ldo, sched,
-                       (unsigned)num_heads, scale_log2e);
+    if (head_dim == 32) launch_vt<_Float16, 32>(NT_VT_ARGS);
+    else if (head_dim == 64) launch_vt<_Float16, 64>(NT_VT_ARGS);
+    else launch_vt<_Float16, 128>(NT_VT_ARGS);
   } else {
-    return fail(NT_ERR_UNSUPPORTED, "attention_vt: dtype must be f16 or bf16");
+    if (head_dim == 32) launch_vt<__bf16, 32>(NT_VT_ARGS);
+    else if (head_dim == 64) launch_vt<__bf16, 64>(NT_VT_ARGS);
+    else launch_vt<__bf16, 128>(NT_VT_ARGS);
   }
+#undef NT_VT_ARGS
   return check_launch("varlen_attention_vt_kernel");
 }

@@ -452,7 +452,7 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
     T_tokens = xq.size(0)
     max_q = int(query.sizes[:, 0].max()) if query.B > 0 else 0
     attn = torch.empty((T_tokens, E), dtype=dtype, device=dev)
-    mfma_path = head_dim == 64 and dtype in (torch.float16, torch.bfloat16)
+    mfma_path = head_dim in (32, 64, 128) and dtype in (torch.float16, torch.bfloat16)
     fused = same and mfma_path and (2 * E) % 128 == 0
     if in_proj_bias is not None:
         in_proj_bias = in_proj_bias.contiguous()
@@ -461,7 +461,7 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
     if W.dtype != dtype:
         raise RuntimeError("linear: input, weight and bias must have the same dtype")
     if fused:
-        # self-attention, head_dim 64: Q|K row-major + V transposed straight out of
+        # self-attention, head_dim 32 / 64 / 128: Q|K row-major + V transposed straight out of
         # the projection GEMM, attention reads both without any re-layout pass
         ldvt = (T_tokens + 72 + 7) // 8 * 8   # rows readable 72 elements past the last token
         qk = torch.empty((T_tokens, 2 * E), dtype=dtype, device=dev)
@@ -474,10 +474,10 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
             sched = query.attention_schedule()
             _C.check(_C.lib.nt_varlen_attention_vt(
                 _C.ptr(qk), 2 * E, _offset_ptr(qk, E), 2 * E, _C.ptr(vt), ldvt, _C.ptr(attn), E,
-                _C.ptr(sched), sched.size(0), num_heads, T_tokens,
+                _C.ptr(sched), sched.size(0), num_heads, head_dim, T_tokens,
                 float(scaling), _C.dtype_code(dtype), stream))
     elif mfma_path and not same and bool((key.sizes[:, 0] > 0).all()):
-        # cross-attention, head_dim 64: three projections (the value one written
+        # cross-attention, head_dim 32 / 64 / 128: three projections (the value one written
         # transposed), then the same attention kernel with one key sequence per
         # query sequence
         b = in_proj_bias
@@ -496,7 +496,7 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
             sched = query.attention_schedule(kv=key)
             _C.check(_C.lib.nt_varlen_attention_vt(
                 _C.ptr(q_t), E, _C.ptr(k_t), E, _C.ptr(vt), ldvt, _C.ptr(attn), E,
-                _C.ptr(sched), sched.size(0), num_heads, T_kv,
+                _C.ptr(sched), sched.size(0), num_heads, head_dim, T_kv,
                 float(scaling), _C.dtype_code(dtype), stream))
     else:
         if same:

@@ -78,6 +78,30 @@ def test_min_mha_reference_shapes(dtype, H, B, Lmax, hd):
     assert got.nested_size() == nt.nested_tensor(xs).nested_size()
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("H,hd,lens", [(8, 32, (1, 64, 65, 300, 129)), (4, 128, (130, 7, 257, 64)),
+                                       (2, 32, (513,)), (3, 128, (1, 2, 3))])
+def test_mfma_attention_head_dims_32_and_128(dtype, H, hd, lens):
+    """head_dim 32 and 128 take the same MFMA kernel as 64 (self- and cross-attention)."""
+    E = H * hd
+    amp = 0.5 if dtype == torch.bfloat16 else 1.0
+    xs, W_in, b_in, W_out, b_out = make_case(E, list(lens), 23, dtype, w_std=E ** -0.5, bias_std=0.1, x_std=amp)
+    got = run_min_mha(H, hd, xs, W_in, b_in, W_out, b_out, dtype)
+    ref = oracle.ref_nested_tensor(xs, dtype=dtype)
+    exp = oracle.min_mha(H, hd, 0.0, False, ref, ref, ref, W_in, b_in, hd ** -0.5, W_out, b_out)
+    check(got, exp, dtype)
+    # cross-attention: the same queries over memories of other lengths
+    g = torch.Generator().manual_seed(29)
+    kv_lens = [max(1, (L * 3) // 2 + 5) for L in lens]
+    kv = [(torch.randn(L, E, generator=g) * amp).to(dtype) for L in kv_lens]
+    qa, ka = nt.nested_tensor(xs, device=DEV, dtype=dtype), nt.nested_tensor(kv, device=DEV, dtype=dtype)
+    got = torch.ops.nestedtensor.min_mha(H, hd, 0.0, False, qa, ka, ka, W_in.to(DEV), b_in.to(DEV),
+                                         hd ** -0.5, W_out.to(DEV), b_out.to(DEV))
+    rk = oracle.ref_nested_tensor(kv, dtype=dtype)
+    exp = oracle.min_mha(H, hd, 0.0, False, ref, rk, rk, W_in, b_in, hd ** -0.5, W_out, b_out)
+    check(got, exp, dtype)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_bt_min_mha_op_and_module_hook(dtype):
     # test_nested_tensor_functional.py:1087-1140: bt_min_mha == mha(nt, nt, nt)
