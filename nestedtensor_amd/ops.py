@@ -476,8 +476,9 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
                 _C.ptr(qk), 2 * E, _offset_ptr(qk, E), 2 * E, _C.ptr(vt), ldvt, _C.ptr(attn), E,
                 _C.ptr(sched), sched.size(0), num_heads, head_dim, T_tokens,
                 float(scaling), _C.dtype_code(dtype), stream))
-    elif mfma_path and not same and bool((key.sizes[:, 0] > 0).all()):
-        # cross-attention, head_dim 32 / 64 / 128: three projections (the value one written
+    elif mfma_path and bool((key.sizes[:, 0] > 0).all()):
+        # cross-attention (or an embedding size the fused projection does not tile),
+        # head_dim 32 / 64 / 128: three projections (the value one written
         # transposed), then the same attention kernel with one key sequence per
         # query sequence
         b = in_proj_bias

@@ -80,7 +80,8 @@ def test_min_mha_reference_shapes(dtype, H, B, Lmax, hd):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("H,hd,lens", [(8, 32, (1, 64, 65, 300, 129)), (4, 128, (130, 7, 257, 64)),
-                                       (2, 32, (513,)), (3, 128, (1, 2, 3))])
+                                       (2, 32, (513,)), (3, 128, (1, 2, 3)),
+                                       (3, 32, (70, 200))])     # E = 96: not a multiple of the fused tile
 def test_mfma_attention_head_dims_32_and_128(dtype, H, hd, lens):
     """head_dim 32 and 128 take the same MFMA kernel as 64 (self- and cross-attention)."""
     E = H * hd
