@@ -600,6 +600,26 @@ def bench_rows(args, torch, dev):
                                       TFLOPs=fl4 / (ms4 * 1e-3) / 1e12,
                                       frac_of_mfma_peak=fl4 / (ms4 * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS)
 
+    # ---- a larger layer for scale: 16 sequences of 256..2048 tokens, d = 2048, 16 heads of 128 ----
+    g = torch.Generator().manual_seed(1010 + 6)
+    El, Hl = 2048, 16
+    lens_l = [int(v) for v in torch.randint(256, 2049, (16,), generator=g)]
+    bufl = torch.randn(sum(lens_l) * El, device=dev, dtype=torch.float16)
+    from nestedtensor_amd.impl import NestedTensorImpl as _ImplL
+    al = nt.NestedTensor(_ImplL(bufl, torch.tensor([[L, El] for L in lens_l], dtype=torch.int64)))
+    Wl_in = (torch.randn(3 * El, El, device=dev) * 0.02).half()
+    Wl_out = (torch.randn(El, El, device=dev) * 0.02).half()
+    bl_in, bl_out = torch.zeros(3 * El, device=dev).half(), torch.zeros(El, device=dev).half()
+    msl = _time_gpu(torch, lambda: torch.ops.nestedtensor.min_mha(
+        Hl, 128, 0.0, False, al, al, al, Wl_in, bl_in, 128 ** -0.5, Wl_out, bl_out), iters=20, warmup=3)
+    Tl = sum(lens_l)
+    fll = 8 * Tl * El * El + 4 * El * sum(L * L for L in lens_l)
+    rows["large_min_mha_fp16"] = dict(
+        ms=msl, workload="B=16, L~U[256,2048], d=2048, 16x128", tokens=Tl, tokens_per_s=Tl / (msl * 1e-3),
+        flops=fll, TFLOPs=fll / (msl * 1e-3) / 1e12,
+        frac_of_mfma_peak=fll / (msl * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS)
+    del bufl, al, Wl_in, Wl_out
+
     # ---- cross-attention: 100 queries per sequence over ragged memories (decoder-style) ----
     g = torch.Generator().manual_seed(1010 + 5)
     Ex, Hx = 512, 8
