@@ -7,7 +7,7 @@ from .. import ops
 from ..impl import NestedTensorImpl, device_offsets
 from . import nested
 
-_ADVICE = (
+_HINT = (
     "To form a valid NestedTensor all Tensor / NestedTensor constiuents of the given list must be "
     "of the same dimension, layout, device, scalar type and either all or none require gradients.")
 
@@ -19,11 +19,11 @@ def _verify_variables(tensors):
         if t.dim() != first.dim():
             raise RuntimeError(
                 "Given Tensor / NestedTensor constiuent of dimension %d doesn't match another "
-                "constiuent of dimension %d. %s" % (t.dim(), first.dim(), _ADVICE))
+                "constiuent of dimension %d. %s" % (t.dim(), first.dim(), _HINT))
         if t.layout != first.layout:
             raise RuntimeError(
                 "Given Tensor / NestedTensor constiuent of layout %s doesn't match another "
-                "constiuent of layout %s. %s" % (t.layout, first.layout, _ADVICE))
+                "constiuent of layout %s. %s" % (t.layout, first.layout, _HINT))
         if t.device != first.device:
             raise RuntimeError(
                 "Given Tensor / NestedTensor constiuent of device %s doesn't match another "
@@ -35,7 +35,7 @@ def _verify_variables(tensors):
         if t.requires_grad != first.requires_grad:
             raise RuntimeError(
                 "Given Tensor / NestedTensor constiuent requires gradient in contrast to another "
-                "constiuent. " + _ADVICE)
+                "constiuent. " + _HINT)
 
 
 def nested_tensor_impl(data, dtype, device, requires_grad, pin_memory, channels_last):
