@@ -103,6 +103,30 @@ def test_mfma_attention_head_dims_32_and_128(dtype, H, hd, lens):
     check(got, exp, dtype)
 
 
+@pytest.mark.parametrize("hd", [32, 64, 128])
+def test_mfma_attention_boundary_lengths(hd):
+    """Every length around the 32-row wavefront blocks, the 64-key tiles and the
+    128-row query tiles, in one batch, as queries and (rotated) as keys."""
+    dtype = torch.float16
+    H = 2
+    E = H * hd
+    lens = [1, 2, 31, 32, 33, 63, 64, 65, 95, 96, 97, 127, 128, 129, 191, 192, 193, 255, 256, 257]
+    xs, W_in, b_in, W_out, b_out = make_case(E, lens, 31, dtype, w_std=E ** -0.5, bias_std=0.1)
+    got = run_min_mha(H, hd, xs, W_in, b_in, W_out, b_out, dtype)
+    ref = oracle.ref_nested_tensor(xs, dtype=dtype)
+    exp = oracle.min_mha(H, hd, 0.0, False, ref, ref, ref, W_in, b_in, hd ** -0.5, W_out, b_out)
+    check(got, exp, dtype)
+    g = torch.Generator().manual_seed(37)
+    kv_lens = lens[7:] + lens[:7]
+    kv = [torch.randn(L, E, generator=g).to(dtype) for L in kv_lens]
+    qa, ka = nt.nested_tensor(xs, device=DEV, dtype=dtype), nt.nested_tensor(kv, device=DEV, dtype=dtype)
+    got = torch.ops.nestedtensor.min_mha(H, hd, 0.0, False, qa, ka, ka, W_in.to(DEV), b_in.to(DEV),
+                                         hd ** -0.5, W_out.to(DEV), b_out.to(DEV))
+    rk = oracle.ref_nested_tensor(kv, dtype=dtype)
+    exp = oracle.min_mha(H, hd, 0.0, False, ref, rk, rk, W_in, b_in, hd ** -0.5, W_out, b_out)
+    check(got, exp, dtype)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_bt_min_mha_op_and_module_hook(dtype):
     # test_nested_tensor_functional.py:1087-1140: bt_min_mha == mha(nt, nt, nt)
