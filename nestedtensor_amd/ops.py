@@ -929,15 +929,16 @@ def to_packed_sequence(impl):
     T = int(lengths.sum())
     index = torch.empty(T, dtype=torch.int64, device=dev)
     data = torch.empty([T] + trailing, dtype=buf.dtype, device=dev)
-    rank_dev, starts_dev = unsorted_indices.to(dev), step_starts.to(dev)
+    # one upload for the three small index arrays
+    meta = torch.cat([unsorted_indices, sorted_indices, step_starts]).to(dev)
+    rank_dev, sorted_dev, starts_dev = meta[:B], meta[B:2 * B], meta[2 * B:]
     with torch.cuda.device(dev):
         stream = _C.current_stream(dev)
         _C.check(_C.lib.nt_packed_sequence_index(_C.ptr(impl.row_offsets_dev()), _C.ptr(rank_dev),
                                                  _C.ptr(starts_dev), B, T, _C.ptr(index), stream))
         _C.check(_C.lib.nt_gather_rows(_C.ptr(buf), T, row_elems * buf.element_size(), _C.ptr(index),
                                        _C.ptr(data), T, None, stream))
-    return torch.nn.utils.rnn.PackedSequence(data, batch_sizes, sorted_indices.to(dev),
-                                             unsorted_indices.to(dev))
+    return torch.nn.utils.rnn.PackedSequence(data, batch_sizes, sorted_dev, rank_dev)
 
 
 # ---- channels-last ragged images: per-constituent transposes ------------------------
