@@ -217,6 +217,10 @@ def _from_value_native(tensor, padding, nested_dim):
                       lambda: _as_byte_mask(tensor != padding))
 
 
+# from this many mask rows on, the lowest mask level is summarised on the device
+_DEVICE_REDUCE_ROWS = 4096
+
+
 def _from_rows(tensor, mask_dims, count_rows, byte_mask):
     """General case of nt_from_tensor_mask (masking.cpp:203-222) for a mask over
     the first `mask_dims` dims of `tensor`.  Rows = everything but the last mask
@@ -233,23 +237,45 @@ def _from_rows(tensor, mask_dims, count_rows, byte_mask):
     for v in rest:
         chunk *= v
     counts_dev, prefix_dev = count_rows(R, M)
-    # one device-to-host copy: the row counts plus "every row keeps a prefix"
-    if R > 0:
-        host = torch.cat([counts_dev, prefix_dev.min().to(torch.int32).reshape(1)]).cpu()
-        counts, all_prefix = host[:-1], bool(host[-1])
-    else:
-        counts, all_prefix = counts_dev.cpu(), True
-    counts = counts.to(torch.int64).reshape((B,) + inner_mask_shape[:-1])
-
     # Nested size from the counts: at every mask level the extent is the number
     # of children that keep anything (masking.cpp:203-222); the selection must
-    # be rectangular or at::stack would have thrown.
-    flat = counts.reshape(B, -1)
-    total = flat.sum(1)
-    extents = [flat.max(1).values]
-    alive = counts > 0
-    leading = all_prefix            # kept children come first at every level
-    while alive.dim() > 1:
+    # be rectangular or at::stack would have thrown.  `leading`: kept children
+    # come first at every level.
+    count_shape = (B,) + inner_mask_shape[:-1]
+    if R >= _DEVICE_REDUCE_ROWS:
+        # many rows: the lowest level is reduced on the device and only the
+        # per-constituent summaries cross to the host, in one copy
+        cd = counts_dev.reshape(count_shape).to(torch.int64)
+        flat = cd.reshape(B, -1)
+        pieces = [flat.sum(1), flat.max(1).values, prefix_dev.min().to(torch.int64).reshape(1)]
+        has_level = cd.dim() > 1
+        if has_level:
+            alive_d = cd > 0
+            lead_d = (alive_d[..., 1:] <= alive_d[..., :-1]).all() if alive_d.size(-1) > 1 \
+                else torch.ones((), dtype=torch.bool, device=cd.device)
+            pieces += [lead_d.to(torch.int64).reshape(1), alive_d.sum(-1).reshape(-1)]
+        host = torch.cat(pieces).cpu()
+        total, extents = host[:B], [host[B:2 * B]]
+        leading = bool(host[2 * B])
+        alive = None
+        if has_level:
+            leading = leading and bool(host[2 * B + 1])
+            c = host[2 * B + 2:].reshape(count_shape[:-1])
+            extents.append(c.reshape(B, -1).max(1).values)
+            alive = c > 0
+    else:
+        # one device-to-host copy: the row counts plus "every row keeps a prefix"
+        if R > 0:
+            host = torch.cat([counts_dev, prefix_dev.min().to(torch.int32).reshape(1)]).cpu()
+            counts, leading = host[:-1], bool(host[-1])
+        else:
+            counts, leading = counts_dev.cpu(), True
+        counts = counts.to(torch.int64).reshape(count_shape)
+        flat = counts.reshape(B, -1)
+        total = flat.sum(1)
+        extents = [flat.max(1).values]
+        alive = counts > 0
+    while alive is not None and alive.dim() > 1:
         if leading and alive.size(-1) > 1:
             leading = bool((alive[..., 1:] <= alive[..., :-1]).all())
         c = alive.sum(-1)

@@ -248,8 +248,13 @@ def test_reference_round_trip_literal_on_device():
     bits_equal(data3, exp)
 
 
+@pytest.mark.parametrize("device_reduce", [False, True])
 @pytest.mark.parametrize("mask_dims", [2, 3, 4])
-def test_from_tensor_mask_random_boxes_vs_literal_walk(mask_dims):
+def test_from_tensor_mask_random_boxes_vs_literal_walk(mask_dims, device_reduce, monkeypatch):
+    # device_reduce: take the path of masks with many rows, where the lowest mask level is
+    # summarised on the device before the counts cross to the host
+    from nestedtensor_amd.nested import masking as _masking
+    monkeypatch.setattr(_masking, "_DEVICE_REDUCE_ROWS", 1 if device_reduce else 1 << 60)
     g = torch.Generator().manual_seed(100 + mask_dims)
     for trial in range(8):
         B = 4
@@ -269,6 +274,23 @@ def test_from_tensor_mask_random_boxes_vs_literal_walk(mask_dims):
             continue
         res = nt.nested_tensor_from_tensor_mask(t.to(DEV), mask.to(DEV))
         nt_matches(res, exp, torch.float32)
+
+
+@pytest.mark.parametrize("device_reduce", [False, True])
+def test_from_tensor_mask_literals_both_reduction_paths(device_reduce, monkeypatch):
+    from nestedtensor_amd.nested import masking as _masking
+    monkeypatch.setattr(_masking, "_DEVICE_REDUCE_ROWS", 1 if device_reduce else 1 << 60)
+    for name, tensor, mask, parts, dtype in FROM_TENSOR_MASK:
+        res = nt.nested_tensor_from_tensor_mask(tensor.to(DEV), mask.to(DEV))
+        nt_matches(res, parts, dtype)
+    # a subset selection that is not a prefix, and a ragged one
+    t = torch.arange(24.).reshape(2, 3, 4)
+    m = torch.tensor([[[0, 1, 1, 0], [0, 1, 1, 0], [0, 0, 0, 0]], [[1, 1, 0, 0], [0, 0, 0, 0], [1, 1, 0, 0]]]).bool()
+    exp = oracle.nt_from_tensor_mask(t, m, 1)
+    nt_matches(nt.nested_tensor_from_tensor_mask(t.to(DEV), m.to(DEV)), exp, torch.float32)
+    bad = torch.tensor([[[1, 1, 1, 0], [1, 0, 0, 0], [0, 0, 0, 0]], [[1, 1, 0, 0], [0, 0, 0, 0], [0, 0, 0, 0]]]).bool()
+    with pytest.raises(RuntimeError):
+        nt.nested_tensor_from_tensor_mask(t.to(DEV), bad.to(DEV))
 
 
 def test_from_tensor_mask_subset_selection_and_ragged_error():
