@@ -12,6 +12,11 @@ _HINT = (
     "of the same dimension, layout, device, scalar type and either all or none require gradients.")
 
 
+# host constituents of at least this many bytes on average are copied to the
+# device one by one instead of being packed on the host first
+_DIRECT_COPY_BYTES = 256 * 1024
+
+
 def _verify_variables(tensors):
     # creation.cpp:28-171
     first = tensors[0]
@@ -80,6 +85,19 @@ def nested_tensor_impl(data, dtype, device, requires_grad, pin_memory, channels_
         if buffer.dtype != dtype or buffer.device != device:
             impl = impl.with_buffer(buffer.to(device, dtype))
         return impl
+    total = int(sizes.prod(1).sum())
+    if (device.type == "cuda" and src_device.type == "cpu"
+            and total * tensors[0].element_size() >= len(tensors) * _DIRECT_COPY_BYTES):
+        # large host constituents: each goes straight into its slot of the device
+        # buffer; packing them on the host first would cost one more pass over
+        # the data than the transfer itself
+        buffer = torch.empty(total, dtype=dtype, device=device)
+        off = 0
+        for t in tensors:
+            n = t.numel()
+            buffer[off:off + n].copy_(t.detach().reshape(-1))
+            off += n
+        return NestedTensorImpl(buffer, sizes)
     # host constituents: pack on the host, then one H2D copy of the packed
     # buffer (what creation.cpp:210-216 does).
     buffer = torch.cat([t.detach().contiguous().reshape(-1) for t in tensors])

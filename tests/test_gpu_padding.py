@@ -371,6 +371,20 @@ def test_random_shapes_sweep_against_oracle(seed):
         nt_matches(again, parts, dtype)
 
 
+def test_constructor_direct_copy_of_large_host_constituents():
+    # constituents of 256 KiB or more go to the device one by one (no host packing); with a dtype
+    # change and a non-contiguous constituent
+    g = torch.Generator().manual_seed(55)
+    parts = [torch.randn(300, 300, generator=g, dtype=torch.float64), torch.randn(700, 300, generator=g,
+                                                                                  dtype=torch.float64).t()]
+    parts[1] = parts[1].t()[:, :300].t()       # a strided view, shape [300, 700]
+    for dtype in (torch.float64, torch.float16):
+        a = nt.nested_tensor(parts, device=DEV, dtype=dtype)
+        ref = oracle.ref_nested_tensor(parts, dtype=dtype)
+        bits_equal(a._impl.buffer, ref.buffer)
+        assert a.nested_size().unbind() == [torch.Size(p.shape) for p in parts]
+
+
 def test_pad_nt_to_a_given_shape():
     # pad_nt (masking.cpp:138-179): a caller-given goal shape, data padded with 0, full-shape mask
     parts = [torch.randn(3, 5), torch.randn(1, 5), torch.randn(4, 2)]
