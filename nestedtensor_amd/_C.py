@@ -108,6 +108,25 @@ def ptr(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
+class _NoContext:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_CONTEXT = _NoContext()
+
+
+def on_device(device):
+    """Context that makes `device` the current HIP device for the launches inside
+    it; free when it already is (the usual case: one GPU per process)."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_CONTEXT
+    return torch.cuda.device(device)
+
+
 def current_stream(device):
     """hipStream_t of torch's current stream on `device`, as void*."""
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)

@@ -25,7 +25,7 @@ from . import _C
 
 class NestedTensorImpl:
     __slots__ = ("buffer", "sizes", "_opt_sizes", "_sizes_dev", "_offsets_dev",
-                 "_row_offsets_dev", "_max_sizes", "_attn_schedule", "_last_dim_rows", "channels_last")
+                 "_row_offsets_dev", "_max_sizes", "_attn_schedule", "_last_dim_rows", "_has_empty", "channels_last")
 
     def __init__(self, buffer, sizes, channels_last=False):
         """buffer: 1-D contiguous tensor; sizes: CPU int64 [B, D], or 0-d for an
@@ -48,6 +48,7 @@ class NestedTensorImpl:
         self._max_sizes = None
         self._attn_schedule = None
         self._last_dim_rows = None
+        self._has_empty = None
 
     # ---- host metadata ----------------------------------------------------
     @property
@@ -93,7 +94,9 @@ class NestedTensorImpl:
         return list(self._max_sizes)
 
     def has_empty_constituent(self):
-        return self.B > 0 and self.D > 0 and bool((self.sizes == 0).any())
+        if self._has_empty is None:
+            self._has_empty = self.B > 0 and self.D > 0 and bool((self.sizes == 0).any())
+        return self._has_empty
 
     def shapes(self):
         return [tuple(int(v) for v in row) for row in self.sizes] if self.sizes.dim() > 0 else []
@@ -181,6 +184,7 @@ class NestedTensorImpl:
                                self.channels_last if channels_last is None else channels_last)
         out._opt_sizes = self._opt_sizes
         out._max_sizes = self._max_sizes
+        out._has_empty = self._has_empty
         if buffer.device == self.buffer.device:
             out._sizes_dev = self._sizes_dev
             out._offsets_dev = self._offsets_dev
@@ -196,7 +200,7 @@ def device_offsets(sizes_dev, B, D):
     offsets = torch.empty(B + 1, dtype=torch.int64, device=dev)
     ws_bytes = _C.lib.nt_offsets_workspace_bytes(B)
     ws = torch.empty(max(ws_bytes, 8), dtype=torch.uint8, device=dev) if ws_bytes else None
-    with torch.cuda.device(dev):
+    with _C.on_device(dev):
         _C.check(_C.lib.nt_offsets_from_sizes(
             _C.ptr(sizes_dev), B, D, _C.ptr(offsets), _C.ptr(ws), ws_bytes,
             _C.current_stream(dev)))

@@ -120,7 +120,7 @@ def _compact(data, bmask, R, M, chunk_elems, total_kept, counts_dev):
     row_offsets = torch.empty(R + 1, dtype=torch.int64, device=dev)
     ws_bytes = _C.lib.nt_scan_workspace_bytes(R)
     ws = torch.empty(max(ws_bytes, 8), dtype=torch.uint8, device=dev) if ws_bytes else None
-    with torch.cuda.device(dev):
+    with _C.on_device(dev):
         stream = _C.current_stream(dev)
         _C.check(_C.lib.nt_exclusive_scan_i32(
             _C.ptr(counts_dev), R, _C.ptr(row_offsets), _C.ptr(ws), ws_bytes, stream))
@@ -134,7 +134,7 @@ def _row_counts(bmask, R, M):
     """Keep-count and is-a-prefix flag per row of a byte mask [R, M]."""
     counts = torch.empty(R, dtype=torch.int32, device=bmask.device)
     prefix = torch.empty(R, dtype=torch.uint8, device=bmask.device)
-    with torch.cuda.device(bmask.device):
+    with _C.on_device(bmask.device):
         _C.check(_C.lib.nt_mask_row_counts(
             _C.ptr(bmask), R, M, _C.ptr(counts), _C.ptr(prefix), _C.current_stream(bmask.device)))
     return counts, prefix
@@ -144,7 +144,7 @@ def _value_row_counts(tensor, padding, R, M):
     """The same for the mask ``tensor != padding`` without building it."""
     counts = torch.empty(R, dtype=torch.int32, device=tensor.device)
     prefix = torch.empty(R, dtype=torch.uint8, device=tensor.device)
-    with torch.cuda.device(tensor.device):
+    with _C.on_device(tensor.device):
         _C.check(_C.lib.nt_value_row_counts(
             _C.ptr(tensor), _C.ELEM_TYPE[tensor.dtype], float(padding), R, M, _C.ptr(counts),
             _C.ptr(prefix), _C.current_stream(tensor.device)))

@@ -65,9 +65,21 @@ def _elem_bytes(dtype):
     return n
 
 
+_PAD_BITS = {}
+
+
 def _pad_bits(padding, dtype):
     """The padding value converted the way the reference converts it,
     ``(T)(double)`` (masking.cpp:594,610), as raw bits."""
+    key = (repr(padding), dtype)
+    if key not in _PAD_BITS:
+        if len(_PAD_BITS) > 256:
+            _PAD_BITS.clear()
+        _PAD_BITS[key] = _pad_bits_uncached(padding, dtype)
+    return _PAD_BITS[key]
+
+
+def _pad_bits_uncached(padding, dtype):
     t = torch.tensor(padding, dtype=dtype)
     view = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()]
     return int(t.view(view).item()) & ((1 << (8 * t.element_size())) - 1)
@@ -118,7 +130,7 @@ def add_padding(impl, padding, with_mask=False, shape=None):
     out = torch.empty([B] + max_size, dtype=impl.buffer.dtype, device=impl.buffer.device)
     eb = _elem_bytes(impl.buffer.dtype)
     dev = impl.buffer.device
-    with torch.cuda.device(dev):
+    with _C.on_device(dev):
         if with_mask:
             mask = torch.empty([B] + max_size, dtype=torch.bool, device=dev)
             _C.check(_C.lib.nt_add_padding_mask(
@@ -219,7 +231,7 @@ def build_mask(impl, kept_dims):
         raise RuntimeError("masks over more than 3 constituent dimensions are not supported.")
     ext = impl.max_sizes()[:K]
     mask = torch.empty([impl.B] + ext, dtype=torch.bool, device=dev)
-    with torch.cuda.device(dev):
+    with _C.on_device(dev):
         _C.check(_C.lib.nt_build_mask(
             _C.ptr(mask), _C.ptr(impl.sizes_dev()), impl.B, impl.D, K, _C.i64_array(ext),
             _C.current_stream(dev)))
@@ -320,7 +332,7 @@ def from_padded_tensor(padded, target):
     eb = _elem_bytes(padded.dtype)
     if out.numel() == 0:
         return res
-    with torch.cuda.device(dev):
+    with _C.on_device(dev):
         _C.check(_C.lib.nt_remove_padding(
             _C.ptr(padded), _C.ptr(out), _C.ptr(res.offsets_dev()), _C.ptr(res.sizes_dev()),
             B, D, nrag, _C.i64_array(ext), eb, _C.current_stream(dev)))
@@ -337,7 +349,7 @@ def pack_device(tensors, offsets_dev, total, dtype, device):
     keep = [t.contiguous() for t in tensors]
     out = torch.empty(total, dtype=dtype, device=device)
     ptrs = torch.tensor([t.data_ptr() for t in keep], dtype=torch.int64).to(device)
-    with torch.cuda.device(device):
+    with _C.on_device(device):
         _C.check(_C.lib.nt_pack(
             _C.ptr(ptrs), _C.ptr(out), _C.ptr(offsets_dev), len(keep),
             _elem_bytes(dtype), _C.current_stream(device)))
@@ -373,7 +385,7 @@ def linear(x, weight, bias, activation=None):
     if bias is not None:
         bias = bias.contiguous()
     out = torch.empty((M, N), dtype=x.dtype, device=x.device)
-    with torch.cuda.device(x.device):
+    with _C.on_device(x.device):
         _C.check(_C.lib.nt_linear_act(
             _C.ptr(x), x.stride(0), _C.ptr(weight), _C.ptr(bias), _C.ptr(out), N, M, N, K,
             _ACTS[activation], _C.dtype_code(x.dtype), _C.current_stream(x.device)))
@@ -400,7 +412,7 @@ def activation(impl, kind):
     _C.require_device(buf, kind)
     out = torch.empty_like(buf)
     if buf.numel() > 0:
-        with torch.cuda.device(buf.device):
+        with _C.on_device(buf.device):
             _C.check(_C.lib.nt_activation_packed(_C.ptr(buf), _C.ptr(out), buf.numel(), _ACTS[kind],
                                                  _C.dtype_code(buf.dtype), _C.current_stream(buf.device)))
     return impl.with_buffer(out)
@@ -466,7 +478,7 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
         ldvt = (T_tokens + 72 + 7) // 8 * 8   # rows readable 72 elements past the last token
         qk = torch.empty((T_tokens, 2 * E), dtype=dtype, device=dev)
         vt = torch.empty((E, ldvt), dtype=dtype, device=dev)
-        with torch.cuda.device(dev):
+        with _C.on_device(dev):
             stream = _C.current_stream(dev)
             _C.check(_C.lib.nt_linear_qkv(
                 _C.ptr(xq), xq.stride(0), _C.ptr(W), _C.ptr(in_proj_bias), _C.ptr(qk), 2 * E,
@@ -489,7 +501,7 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
         vt = torch.empty((E, ldvt), dtype=dtype, device=dev)
         xv = value.buffer.reshape(-1, E)
         bv = None if b is None else b[2 * E:].contiguous()
-        with torch.cuda.device(dev):
+        with _C.on_device(dev):
             stream = _C.current_stream(dev)
             _C.check(_C.lib.nt_linear_transposed(
                 _C.ptr(xv), xv.stride(0), _C.ptr(W[2 * E:]), _C.ptr(bv), _C.ptr(vt), ldvt, T_kv, E, E,
@@ -512,7 +524,7 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
             v_t = linear(value.buffer.reshape(-1, E), W[2 * E:], None if b is None else b[2 * E:])
             qc = kc = vc = 0
             ldq = ldk = ldv = E
-        with torch.cuda.device(dev):
+        with _C.on_device(dev):
             _C.check(_C.lib.nt_varlen_attention(
                 _offset_ptr(q_t, qc), ldq, _offset_ptr(k_t, kc), ldk, _offset_ptr(v_t, vc), ldv,
                 _C.ptr(attn), E, _C.ptr(query.row_offsets_dev()), _C.ptr(key.row_offsets_dev()),
@@ -582,7 +594,7 @@ def layer_norm(impl, normalized_shape, weight=None, bias=None, eps=1e-5, residua
     rows = buf.numel() // n if n > 0 else 0
     weight = weight.contiguous() if weight is not None else None
     bias = bias.contiguous() if bias is not None else None
-    with torch.cuda.device(buf.device):
+    with _C.on_device(buf.device):
         _C.check(_C.lib.nt_layer_norm(_C.ptr(buf), _C.ptr(res_buf), _C.ptr(weight), _C.ptr(bias),
                                       _C.ptr(out), rows, n, float(eps), _C.dtype_code(buf.dtype),
                                       _C.current_stream(buf.device)))
@@ -618,7 +630,7 @@ def add(impl, other, alpha=1):
         raise RuntimeError("add: both operands must have the same dtype and device")
     out = torch.empty_like(buf)
     if buf.numel() > 0:
-        with torch.cuda.device(buf.device):
+        with _C.on_device(buf.device):
             _C.check(_C.lib.nt_add_packed(_C.ptr(buf), _C.ptr(b), float(alpha), _C.ptr(out), buf.numel(),
                                           period, _C.dtype_code(buf.dtype), _C.current_stream(buf.device)))
     return impl.with_buffer(out)
@@ -649,7 +661,7 @@ def softmax(impl, dim, dtype=None, log=False):
     if buf.numel() == 0:
         return impl.with_buffer(out)
     row_offsets, total_rows = impl.last_dim_rows()
-    with torch.cuda.device(buf.device):
+    with _C.on_device(buf.device):
         _C.check(_C.lib.nt_softmax_rows(_C.ptr(buf), _C.ptr(out), _C.ptr(impl.offsets_dev()),
                                         _C.ptr(row_offsets), B, total_rows, 1 if log else 0,
                                         _C.dtype_code(buf.dtype), _C.current_stream(buf.device)))
@@ -684,7 +696,7 @@ def mul(impl, other):
         raise RuntimeError("mul: both operands must have the same dtype and device")
     out = torch.empty_like(buf)
     if buf.numel() > 0:
-        with torch.cuda.device(buf.device):
+        with _C.on_device(buf.device):
             _C.check(_C.lib.nt_mul_packed(_C.ptr(buf), _C.ptr(b), scale, _C.ptr(out), buf.numel(), period,
                                           _C.dtype_code(buf.dtype), _C.current_stream(buf.device)))
     return impl.with_buffer(out)
@@ -819,7 +831,7 @@ def embedding(weight, indices, padding_idx=None, max_norm=None, norm_type=2.0,
     V, E = weight.shape
     out = torch.empty(idx.numel() * E, dtype=weight.dtype, device=weight.device)
     oob = torch.zeros(1, dtype=torch.int32, device=weight.device)
-    with torch.cuda.device(weight.device):
+    with _C.on_device(weight.device):
         _C.check(_C.lib.nt_gather_rows(_C.ptr(weight), V, E * weight.element_size(), _C.ptr(idx64),
                                        _C.ptr(out), idx.numel(), _C.ptr(oob),
                                        _C.current_stream(weight.device)))
@@ -871,7 +883,7 @@ def embedding_bag(input, weight, offsets=None, max_norm=None, norm_type=2, scale
     B = input.B
     out = torch.empty((B, E), dtype=weight.dtype, device=weight.device)
     oob = torch.zeros(1, dtype=torch.int32, device=weight.device)
-    with torch.cuda.device(weight.device):
+    with _C.on_device(weight.device):
         _C.check(_C.lib.nt_embedding_bag(_C.ptr(weight), E, V, _C.ptr(idx64), idx64.numel(),
                                          _C.ptr(input.offsets_dev()),
                                          _C.ptr(out), B, E, modes[mode], _C.dtype_code(weight.dtype),
@@ -891,7 +903,7 @@ def to_sparse_csr(impl):
     crow = impl.offsets_dev()
     col = torch.empty(buf.numel(), dtype=torch.int64, device=buf.device)
     mx = impl.max_sizes()
-    with torch.cuda.device(buf.device):
+    with _C.on_device(buf.device):
         _C.check(_C.lib.nt_ragged_arange(_C.ptr(crow), impl.B, mx[0] if mx else 0, _C.ptr(col),
                                          _C.current_stream(buf.device)))
     return torch.sparse_csr_tensor(crow, col, buf, size=(impl.B, mx[0] if mx else 0))
@@ -932,7 +944,7 @@ def to_packed_sequence(impl):
     # one upload for the three small index arrays
     meta = torch.cat([unsorted_indices, sorted_indices, step_starts]).to(dev)
     rank_dev, sorted_dev, starts_dev = meta[:B], meta[B:2 * B], meta[2 * B:]
-    with torch.cuda.device(dev):
+    with _C.on_device(dev):
         stream = _C.current_stream(dev)
         _C.check(_C.lib.nt_packed_sequence_index(_C.ptr(impl.row_offsets_dev()), _C.ptr(rank_dev),
                                                  _C.ptr(starts_dev), B, T, _C.ptr(index), stream))
@@ -971,7 +983,7 @@ def _transpose_constituents(impl, rows, cols, new_sizes):
     meta_dev = meta.to(buf.device)
     out = torch.empty_like(buf)
     if total_tiles:
-        with torch.cuda.device(buf.device):
+        with _C.on_device(buf.device):
             _C.check(_C.lib.nt_transpose_ragged(
                 _C.ptr(buf), _C.ptr(out), _C.ptr(impl.offsets_dev()), _C.ptr(meta_dev[0]),
                 _C.ptr(meta_dev[1]), _C.ptr(meta_dev[2]), B, total_tiles, tr, tc, buf.element_size(),
