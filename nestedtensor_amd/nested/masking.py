@@ -218,7 +218,7 @@ def _from_value_native(tensor, padding, nested_dim):
 
 
 # from this many mask rows on, the lowest mask level is summarised on the device
-_DEVICE_REDUCE_ROWS = 4096
+_DEVICE_REDUCE_ROWS = 32768
 
 
 def _from_rows(tensor, mask_dims, count_rows, byte_mask):
