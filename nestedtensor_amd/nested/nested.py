@@ -422,6 +422,7 @@ def _mul(input, other, *, out=None):
 
 
 def _softmax(input, dim=None, _stacklevel=3, dtype=None):
+    # torch.nn.functional.softmax(input, dim, _stacklevel, dtype)
     if dim is None:
         raise RuntimeError("softmax on a NestedTensor needs an explicit dim.")
     return ops.softmax(input, dim, dtype, log=False)
@@ -430,6 +431,15 @@ def _softmax(input, dim=None, _stacklevel=3, dtype=None):
 def _log_softmax(input, dim=None, _stacklevel=3, dtype=None):
     if dim is None:
         raise RuntimeError("log_softmax on a NestedTensor needs an explicit dim.")
+    return ops.softmax(input, dim, dtype, log=True)
+
+
+def _torch_softmax(input, dim, dtype=None):
+    # torch.softmax(input, dim, dtype=None) / Tensor.softmax: no _stacklevel argument
+    return ops.softmax(input, dim, dtype, log=False)
+
+
+def _torch_log_softmax(input, dim, dtype=None):
     return ops.softmax(input, dim, dtype, log=True)
 
 
@@ -534,11 +544,11 @@ _HANDLERS = {
     torch.unbind: _unbind,
     torch.Tensor.unbind: _unbind,
     torch.nn.functional.softmax: _softmax,
-    torch.softmax: _softmax,
-    torch.Tensor.softmax: _softmax,
+    torch.softmax: _torch_softmax,
+    torch.Tensor.softmax: _torch_softmax,
     torch.nn.functional.log_softmax: _log_softmax,
-    torch.log_softmax: _log_softmax,
-    torch.Tensor.log_softmax: _log_softmax,
+    torch.log_softmax: _torch_log_softmax,
+    torch.Tensor.log_softmax: _torch_log_softmax,
     torch.mul: _mul,
     torch.Tensor.mul: _mul,
     torch.Tensor.__mul__: _mul,

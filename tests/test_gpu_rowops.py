@@ -148,6 +148,8 @@ def test_softmax_last_dim(dtype, log):
     if dtype != torch.float32 and not log:
         up = torch.softmax(a, -1, dtype=torch.float32)          # at::softmax's dtype argument
         assert up.dtype == torch.float32
+        assert torch.equal(torch.softmax(a, -1, torch.float32)._impl.buffer, up._impl.buffer)   # positional
+        assert torch.equal(torch.nn.functional.softmax(a, -1, dtype=torch.float32)._impl.buffer, up._impl.buffer)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
