@@ -206,8 +206,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
     // lane fetches: slot p of row r holds piece p ^ ((r >> 1) & 7).  The compiler
     // does not see these loads (inline asm), so their completion is awaited by hand
     // before the barrier that publishes the tile.  The asm writes M0 (the LDS
-    // destination); nothing else in these kernels uses M0 (no dynamic register
-    // indexing, no LDS-direct builtin), which is why it is not saved.
+    // destination) and says so in its clobber list.
     static_assert(Cfg::kRowBytes == 128 && Cfg::kBM % 8 == 0, "1 KiB blocks of eight rows");
     constexpr int kN = Cfg::kPerThread;
     constexpr int kWaves = Cfg::kThreads / 64;
@@ -238,7 +237,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
             lds_base + (unsigned)(buf * Cfg::kDmaTileBytes + (i * kWaves + wave) * 1024));
         const char* src = gptr[i] + kt * Cfg::kRowBytes;
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                     :: "v"(src), "s"(dst) : "memory");
+                     :: "v"(src), "s"(dst) : "memory", "m0");
       }
     };
     const int sw = (l32 >> 1) & 7;
@@ -285,6 +284,13 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
       asm volatile("s_waitcnt vmcnt(%0)" :: "n"((kNB - 2) * kN) : "memory");
       __syncthreads();
       buf = buf + 1 == kNB ? 0 : buf + 1;
+    }
+    // The last kNB - 1 iterations issued clamped re-reads of the last K tile; up to
+    // (kNB - 2) * kN of them per lane may still be in flight, and their LDS
+    // destinations overlap the strips of the epilogue.  Drain them, workgroup-wide.
+    if (kNB > 2) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
     }
   } else {
     // Any K: element-wise tails, one K tile in registers ahead of the MFMAs, two
@@ -351,7 +357,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
   }
 
   // ---- epilogue ----------------------------------------------------------
-  // (the K loop ended with a barrier: the tile buffers are free)
+  // (the K loop ended with a barrier and no load into LDS is outstanding: the tile
+  // buffers are free)
   constexpr int kStripW = VT_OUT ? WM : WN;                    // 32-wide blocks per strip row
   constexpr int kStripRow = kStripW * 32 * (int)sizeof(T) + 16;
   constexpr int kCpr = kStripW * 32 * (int)sizeof(T) / 16;    // 16-byte pieces per strip row
