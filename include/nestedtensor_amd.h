@@ -62,6 +62,21 @@ int nt_offsets_from_sizes(const int64_t* sizes, int64_t B, int64_t D,
                           int64_t* offsets, void* workspace, size_t workspace_bytes,
                           void* stream);
 
+/* nt_offsets_from_sizes without a workspace argument and without any allocation.
+ * No counterpart in the reference: it exists for callers that cannot allocate
+ * device memory (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  The tile sums of the scan live in a 256 KiB array in
+ * the library's own device data segment (one copy per GPU, held until the
+ * process ends), which bounds B at nt_offsets_noalloc_max_B() = 67 108 864;
+ * larger B returns NT_ERR_UNSUPPORTED.  Results are bit-identical to
+ * nt_offsets_from_sizes.  All calls on one GPU share that array: calls that
+ * overlap on one GPU (different streams or threads) race on it; calls on one
+ * stream are ordered.  The first call on a device resolves the array's address
+ * (hipGetSymbolAddress) and should be made outside stream capture. */
+int64_t nt_offsets_noalloc_max_B(void);
+int nt_offsets_from_sizes_noalloc(const int64_t* sizes, int64_t B, int64_t D, int64_t* offsets,
+                                  void* stream);
+
 /* ---- packed <-> padded ------------------------------------------------- */
 
 /* padded[b, i_1..i_D] = inside(sizes[b]) ? packed[offsets[b] + lin(i)] : pad

@@ -9,6 +9,8 @@
 // tile sums by one workgroup, rescan with carry).
 #include "nt_common.h"
 
+#include <atomic>
+
 namespace nt {
 
 constexpr int kScanThreads = 256;
@@ -148,6 +150,47 @@ static int run_scan(Load load, int64_t n, int64_t* out, void* workspace, size_t 
   return check_launch("scan kernels");
 }
 
+// ---------------------------------------------------------------------------
+// The allocation-free variant of nt_offsets_from_sizes keeps its tile sums in
+// device memory that belongs to the library: a file-scope __device__ array.  In
+// host code the array's name is only a handle for hipGetSymbolAddress; the
+// address the kernels get is looked up once per device and cached here.  Every
+// GPU holds its own copy of the array (kNoAllocMaxTiles * 8 bytes = 256 KiB)
+// from the moment the code object is loaded there until the process ends.
+constexpr int64_t kNoAllocMaxTiles = 32768;
+constexpr int64_t kNoAllocMaxB = kNoAllocMaxTiles * kScanTile;   // 67 108 864 constituents
+static __device__ __align__(256) int64_t scratch[kNoAllocMaxTiles];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<int64_t*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device, or nullptr with the error
+// text set.  The first call on a device asks the runtime; later calls read the
+// cached pointer (threads that race on the first call store the same value).
+static int64_t* scratch_on_current_device() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    fail(NT_ERR_HIP, "offsets_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+    return nullptr;
+  }
+  if (dev < 0 || dev >= kMaxDevices) {
+    fail(NT_ERR_UNSUPPORTED, "offsets_noalloc: device index %d is not in [0, %d)", dev, kMaxDevices);
+    return nullptr;
+  }
+  int64_t* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p != nullptr) return p;
+  void* addr = nullptr;
+  e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || addr == nullptr) {
+    fail(NT_ERR_HIP, "offsets_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    return nullptr;
+  }
+  p = static_cast<int64_t*>(addr);
+  g_scratch_ptr[dev].store(p, std::memory_order_release);
+  return p;
+}
+
 }  // namespace nt
 
 using namespace nt;
@@ -165,6 +208,29 @@ extern "C" int nt_offsets_from_sizes(const int64_t* sizes, int64_t B, int64_t D,
   if (B > 0 && D > 0 && sizes == nullptr) return fail(NT_ERR_INVALID_ARGUMENT, "offsets: sizes is NULL");
   SizesProd load{sizes, D};
   return run_scan(load, B, offsets, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int64_t nt_offsets_noalloc_max_B(void) { return kNoAllocMaxB; }
+
+extern "C" int nt_offsets_from_sizes_noalloc(const int64_t* sizes, int64_t B, int64_t D,
+                                             int64_t* offsets, void* stream) {
+  if (D < 0) return fail(NT_ERR_INVALID_ARGUMENT, "offsets_noalloc: D must be >= 0");
+  if (B > 0 && D > 0 && sizes == nullptr) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "offsets_noalloc: sizes is NULL");
+  }
+  if (B > kNoAllocMaxB) {
+    return fail(NT_ERR_UNSUPPORTED,
+                "offsets_noalloc: B = %lld exceeds the built-in scratch (at most %lld constituents); "
+                "use nt_offsets_from_sizes with a caller-provided workspace",
+                (long long)B, (long long)kNoAllocMaxB);
+  }
+  // Nothing in the scratch has to start at zero: the first launch writes the
+  // sum of every tile before the second one reads it.
+  int64_t* ws = scratch_on_current_device();
+  if (ws == nullptr) return NT_ERR_HIP;
+  SizesProd load{sizes, D};
+  return run_scan(load, B, offsets, ws, (size_t)kNoAllocMaxTiles * sizeof(int64_t),
+                  (hipStream_t)stream);
 }
 
 extern "C" int nt_exclusive_scan_i32(const int32_t* in, int64_t n, int64_t* out, void* workspace,

@@ -1,0 +1,72 @@
+"""nt_offsets_from_sizes_noalloc, the entry point that allocates nothing: called
+through the C ABI and compared bit for bit with nt_offsets_from_sizes (which takes
+its scratch from the caller) and with the closed form cumsum(prod(sizes)), on
+calls in a row that share the library's built-in scratch, the later ones with
+smaller inputs."""
+
+import pytest
+import torch
+
+from nestedtensor_amd import _C
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda", 0)
+
+
+def _with_workspace(sizes_dev, B, D):
+    out = torch.empty(B + 1, dtype=torch.int64, device=DEV)
+    nbytes = _C.lib.nt_offsets_workspace_bytes(B)
+    ws = torch.empty(max(nbytes, 8), dtype=torch.uint8, device=DEV)
+    _C.check(_C.lib.nt_offsets_from_sizes(_C.ptr(sizes_dev), B, D, _C.ptr(out), _C.ptr(ws), nbytes,
+                                          _C.current_stream(DEV)))
+    return out
+
+
+def _noalloc(sizes_dev, B, D, out):
+    _C.check(_C.lib.nt_offsets_from_sizes_noalloc(_C.ptr(sizes_dev), B, D, _C.ptr(out),
+                                                  _C.current_stream(DEV)))
+
+
+def test_noalloc_offsets_match_workspace_variant_on_consecutive_calls():
+    # 300001 constituents = 147 tiles of the scan, then 5000 (3 tiles), then one
+    # tile, then the large one again: every call reuses the same built-in scratch
+    cases = [(300001, 2), (5000, 3), (100, 1), (300001, 2), (64, 0)]
+    inputs = []
+    for B, D in cases:
+        g = torch.Generator().manual_seed(B * 31 + D)
+        inputs.append(torch.randint(0, 50, (B, D), generator=g, dtype=torch.int64))
+    dev_inputs = [s.to(DEV) for s in inputs]
+    # outputs are allocated up front: the calls themselves allocate nothing
+    outs = [torch.full((B + 1,), -1, dtype=torch.int64, device=DEV) for B, _ in cases]
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated(DEV)
+    for (B, D), s, o in zip(cases, dev_inputs, outs):
+        _noalloc(s, B, D, o)
+    assert torch.cuda.memory_allocated(DEV) == before
+    torch.cuda.synchronize()
+    for (B, D), s_host, s, o in zip(cases, inputs, dev_inputs, outs):
+        exp = torch.cat([torch.zeros(1, dtype=torch.int64), s_host.prod(1).cumsum(0)])
+        assert torch.equal(o.cpu(), exp), (B, D)
+        assert torch.equal(o, _with_workspace(s, B, D)), (B, D)
+
+
+def test_noalloc_offsets_beyond_int32():
+    sizes = torch.full((4096, 2), 4096, dtype=torch.int64, device=DEV)
+    out = torch.empty(4097, dtype=torch.int64, device=DEV)
+    _noalloc(sizes, 4096, 2, out)
+    assert torch.equal(out.cpu(), torch.arange(4097, dtype=torch.int64) * (4096 * 4096))
+
+
+def test_noalloc_offsets_rejects_sizes_beyond_the_scratch():
+    limit = _C.lib.nt_offsets_noalloc_max_B()
+    assert limit == 32768 * 2048
+    sizes = torch.ones((8, 1), dtype=torch.int64, device=DEV)
+    out = torch.full((9,), 7, dtype=torch.int64, device=DEV)
+    rc = _C.lib.nt_offsets_from_sizes_noalloc(_C.ptr(sizes), limit + 1, 1, _C.ptr(out),
+                                              _C.current_stream(DEV))
+    assert rc == 2   # NT_ERR_UNSUPPORTED, nothing launched
+    assert b"exceeds the built-in scratch" in _C.lib.nt_last_error()
+    torch.cuda.synchronize()
+    assert bool((out == 7).all())
+    rc = _C.lib.nt_offsets_from_sizes_noalloc(None, 4, 1, _C.ptr(out), _C.current_stream(DEV))
+    assert rc == 1   # NT_ERR_INVALID_ARGUMENT
