@@ -67,13 +67,13 @@ int nt_offsets_from_sizes(const int64_t* sizes, int64_t B, int64_t D,
  * device memory (code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc).  The tile sums of the scan live in a 256 KiB array in
  * the library's own device data segment (one copy per GPU, held until the
- * process ends), which bounds B at nt_offsets_noalloc_max_B() = 67 108 864;
+ * process ends), which bounds B at nt_offsets_noalloc_max_count() = 67 108 864;
  * larger B returns NT_ERR_UNSUPPORTED.  Results are bit-identical to
  * nt_offsets_from_sizes.  All calls on one GPU share that array: calls that
  * overlap on one GPU (different streams or threads) race on it; calls on one
  * stream are ordered.  The first call on a device resolves the array's address
  * (hipGetSymbolAddress) and should be made outside stream capture. */
-int64_t nt_offsets_noalloc_max_B(void);
+int64_t nt_offsets_noalloc_max_count(void);
 int nt_offsets_from_sizes_noalloc(const int64_t* sizes, int64_t B, int64_t D, int64_t* offsets,
                                   void* stream);
 
@@ -188,7 +188,9 @@ int nt_linear_act(const void* A, int64_t lda, const void* W, const void* bias, v
  * over that sequence's own keys only:
  *   out[q_off[b] + i, h*hd + d] = sum_j softmax_j(scale * q_i . k_j) v_j[d]
  * q rows are q[(q_off[b] + i) * ldq + h*hd ...], k/v likewise with kv_off.
- * head_dim must be 64 for f16/bf16.  Replaces the padded chain of bt_min_mha
+ * f16 / bf16 with head_dim 64 run on the matrix pipe; any other head_dim, and
+ * f32, take a scalar kernel (one wavefront per query row and head), which is a
+ * parity path, not a fast one.  Replaces the padded chain of bt_min_mha
  * (nestedtensor/csrc/cuda/mha.cpp:59-105: to_padded_tensor, batched QK^T,
  * softmax_kernel_kernelLauncher of cuda/attention.h:25-33, PV,
  * from_padded_tensor) and the unwired add_QKV_bias_padding /
@@ -227,13 +229,16 @@ int nt_linear_transposed(const void* A, int64_t lda, const void* W, const void* 
  * self-attention on the output of nt_linear_qkv, q = QK, k = QK + E, ldq = ldk =
  * ldqk.  `schedule` is a device array of n_work int32[8] work items {first query
  * token, query length, first query row of the tile (multiple of 128), 0, first
- * key token, key length (>= 1), 0, 0}: one per 128-query tile of every sequence
+ * key token, key length, 0, 0}: one per 128-query tile of every sequence
  * (for cross-attention: of every query sequence, with the key sequence it
  * attends to), in the order they should start (longest key sequences first); a
  * workgroup is launched per (item, head), so no padded tile is ever issued.  The
  * rows of Vt must be readable up to 72 elements past the last key token
- * (ldvt >= total_kv_tokens + 72); what is stored there is ignored.  Output and
- * semantics as nt_varlen_attention. */
+ * (ldvt >= total_kv_tokens + 72); what is stored there is ignored.  An item
+ * with key length 0 writes zeros to its query rows, one with query length 0 does
+ * nothing; first tokens and lengths are int32 (at most 2^31 - 1 tokens in total)
+ * and must describe rows inside the buffers, the kernel cannot check them.
+ * Output and semantics as nt_varlen_attention. */
 int nt_varlen_attention_vt(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* vt,
                            int64_t ldvt, void* out, int64_t ldo, const int32_t* schedule,
                            int64_t n_work, int64_t num_heads, int64_t head_dim,

@@ -33,7 +33,7 @@ SIGNATURES = {
     "nt_last_error": (ctypes.c_char_p, []),
     "nt_offsets_workspace_bytes": (_size_t, [_i64]),
     "nt_offsets_from_sizes": (_int, [_c_void_p, _i64, _i64, _c_void_p, _c_void_p, _size_t, _c_void_p]),
-    "nt_offsets_noalloc_max_B": (_i64, []),
+    "nt_offsets_noalloc_max_count": (_i64, []),
     "nt_offsets_from_sizes_noalloc": (_int, [_c_void_p, _i64, _i64, _c_void_p, _c_void_p]),
     "nt_add_padding": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64,
                               ctypes.POINTER(_i64), _int, _u64, _c_void_p]),

@@ -35,11 +35,15 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 // max over the two lanes l and l ^ 32 without the LDS round trip of a shuffle:
 // v_permlane32_swap exchanges the upper half of one register with the lower half
-// of another, which leaves (lo, lo) in one and (hi, hi) in the other.
+// of another, which leaves (lo, lo) in one and (hi, hi) in the other.  Written as
+// inline asm: through the builtin, with the same value in both operands, the
+// compiler keeps only the first result and drops the maximum (the kernel then
+// sees the maximum of half of a row's keys).  The asm is opaque to the hazard
+// recognizer, hence the wait states around the swap.
 __device__ __forceinline__ float max_across_halves(float v) {
-  const unsigned b = __builtin_bit_cast(unsigned, v);
-  const auto r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
-  return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+  float lo = v, hi = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+  return fmaxf(lo, hi);
 }
 
 template <typename T> struct AttnT;
@@ -55,6 +59,12 @@ template <> struct AttnT<_Float16> {
     return r;
   }
   static constexpr uint32_t kOnePair = 0x3c003c00u;   // (1.0, 1.0)
+  // acc + lo + hi of a packed pair, in fp32 (v_dot2c_f32_f16)
+  static __device__ __forceinline__ float dot_ones(uint32_t pair, float acc) {
+    half2v h, one = {(_Float16)1.0f, (_Float16)1.0f};
+    __builtin_memcpy(&h, &pair, 4);
+    return __builtin_amdgcn_fdot2(h, one, acc, false);
+  }
   static __device__ __forceinline__ acc16 mma(Frag a, Frag b, acc16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
@@ -70,6 +80,11 @@ template <> struct AttnT<__bf16> {
     return r;
   }
   static constexpr uint32_t kOnePair = 0x3f803f80u;
+  static __device__ __forceinline__ float dot_ones(uint32_t pair, float acc) {   // v_dot2c_f32_bf16
+    bf16x2 h, one = {(__bf16)1.0f, (__bf16)1.0f};
+    __builtin_memcpy(&h, &pair, 4);
+    return __builtin_amdgcn_fdot2_f32_bf16(h, one, acc, false);
+  }
   static __device__ __forceinline__ acc16 mma(Frag a, Frag b, acc16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
@@ -283,28 +298,65 @@ __global__ __launch_bounds__(256) void varlen_attention_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Self-attention kernel of the fused layer: Q and K come row-major from the
-// [T, 2E] projection buffer, V comes TRANSPOSED (Vt[h*64 + d][token], written
-// that way by the QKV GEMM epilogue), so a V^T tile is 64 rows of 64
-// key-contiguous values and needs no transposition on its way into LDS.
+// Attention kernel of the fused layer: Q and K come row-major from the
+// projection buffers, V comes TRANSPOSED (Vt[h*HD + d][token], written that way by
+// the projection GEMM's epilogue), so a V^T tile is HD rows of 64 key-contiguous
+// values and needs no transposition on its way into LDS.
 //
-// LDS layout of the V^T tile: within each group of 16 keys the positions are
-// permuted (key = 8a + 4g + c  ->  position 8g + 4a + c) so that the eight keys a
-// lane group needs for one MFMA k-step -- the keys whose probabilities it
-// already holds in its score accumulators -- are one 16-byte read.
+// Work items {first query token, query length, first query row of the tile, 0,
+// first key token, key length, 0, 0} come from a schedule the host builds from
+// the nested size (longest sequences first, no item for a tile that does not
+// exist), so every workgroup that is launched has work and the long sequences
+// start first.  A workgroup is (item, head), head fastest: the items of ALL heads
+// of the long sequences are dispatched before any short item.
+//
+// What keeps the vector ALU work per score low:
+//
+//  * Q is multiplied by scale * log2(e) once, when its fragments are loaded, so
+//    the score accumulators are exponents of two as they stand;
+//  * the reference maximum of a query row is not subtracted with an instruction
+//    per score: the 32x32 blocks of S^T = K Q^T are accumulated onto a register
+//    block that holds -m_ref (the third MFMA operand), so S - m_ref falls out
+//    of the matrix pipe.  m_ref need not be the exact running maximum, softmax
+//    is invariant to it; it only has to keep 2^(S - m_ref) inside the range of
+//    the storage type.  It is set from the first tile and raised only when a
+//    tile's maximum exceeds it by more than kLazyMaxLog2 (wavefront-uniform
+//    branch, rare after the first tile), which is also the only place where the
+//    output accumulators are rescaled;
+//  * the denominators are sums of the ROUNDED probabilities (the ones that meet
+//    V), two per v_dot2c instruction, accumulated in fp32;
+//  * V^T tiles lie in LDS in key order (one 16-byte write per piece); the
+//    permutation that the PV product needs (the eight keys a lane group holds in
+//    its score accumulators must be one 16-byte run of a V^T row) is applied to
+//    the ROW order of the K tile instead, where it is free: a thread simply
+//    fetches another row.  LDS row rho = 16 ks + 8 a + 4 g + c of the K tile holds
+//    key 16 ks + 8 g + 4 a + c;
+//  * keys past L in the last tile: their K rows are copies of row L - 1 (valid
+//    memory, cannot raise the maximum), their scores are set to -inf after the
+//    maximum is taken and their V^T columns are zeroed on the way into LDS, so
+//    nothing of what follows the sequence in memory can reach the result.
+constexpr float kLazyMaxLog2 = 8.0f;
 
-// Work items {first token, length, first query row, 0} come from a schedule the
-// host builds from the nested size (longest sequences first, no item for a tile
-// that does not exist), so every workgroup that is launched has work and the
-// long sequences start first.
+template <typename T> struct QScale;
+template <> struct QScale<_Float16> {
+  static __device__ __forceinline__ half8 run(half8 v, float s) {
+    const _Float16 hs = (_Float16)s;
+    return v * hs;   // v_pk_mul_f16
+  }
+};
+template <> struct QScale<__bf16> {
+  static __device__ __forceinline__ bf16x8 run(bf16x8 v, float s) {
+    bf16x8 r;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r[j] = (__bf16)((float)v[j] * s);
+    return r;
+  }
+};
+
 #ifndef NT_ATTN_WAVES_PER_EU
 #define NT_ATTN_WAVES_PER_EU 3
 #endif
 
-// HD: head_dim, 32, 64 or 128.  Per key tile a workgroup stages 64 K rows of HD
-// elements and HD V^T rows of 64 keys; a wavefront holds HD / 16 Q fragments and
-// HD / 32 output accumulator blocks.  The benchmark shapes have HD = 64; 128 needs
-// about 200 registers per lane, so two wavefronts per SIMD there.
 template <typename T, int HD>
 __global__ __launch_bounds__(256, (HD > 64 ? 2 : NT_ATTN_WAVES_PER_EU)) void varlen_attention_vt_kernel(
     const T* __restrict__ Q, int64_t ldq, const T* __restrict__ K, int64_t ldk,
@@ -313,31 +365,34 @@ __global__ __launch_bounds__(256, (HD > 64 ? 2 : NT_ATTN_WAVES_PER_EU)) void var
   typedef AttnT<T> AT;
   typedef typename AT::Frag Frag;
 
-  constexpr int kKR = HD * 2 + 16;          // LDS bytes per K row (16 pad: conflict-free fragment reads)
-  constexpr int kQF = HD / 16;              // Q fragments = MFMA k-steps of the score product
-  constexpr int kDB = HD / 32;              // 32-row blocks of O^T
-  constexpr int kKPieces = HD / 8;          // 16-byte pieces per K row
+  constexpr int kKR = HD * 2 + 16;
+  constexpr int kQF = HD / 16;
+  constexpr int kDB = HD / 32;
+  constexpr int kKPieces = HD / 8;
   constexpr int kKRowsPerPass = 256 / kKPieces;
-  constexpr int kKP = kKTile / kKRowsPerPass;   // K pieces per thread and tile
-  constexpr int kVP = HD / 32;              // V^T pieces per thread and tile (8 per row, 32 rows a pass)
+  constexpr int kKP = kKTile / kKRowsPerPass;
+  constexpr int kVP = HD / 32;
   __shared__ __align__(16) char lds_k[2][kKTile * kKR];
-  __shared__ __align__(16) char lds_v[2][(HD + 1) * kVRow];   // row HD: ones (see below)
+  __shared__ __align__(16) char lds_v[2][HD * kVRow];
 
-  // Head fastest: the schedule lists the longest sequences first, and this way
-  // their items of ALL heads are dispatched before any short item (with the
-  // item index fastest, the long items of the last heads would start last and
-  // run alone at the end).
   const int h = (int)(blockIdx.x % num_heads);
-  // item: {first query token, query length, first query row of this tile, 0,
-  //        first key token, key length, 0, 0}; self-attention lists the same
-  //        sequence twice, cross-attention the two sequences of the pair
   const int4 item = schedule[2 * (blockIdx.x / num_heads)];
   const int4 item_kv = schedule[2 * (blockIdx.x / num_heads) + 1];
   const int64_t q_begin = item.x;
   const int Lq = item.y;
   const int q0 = item.z;
-  const int64_t begin = item_kv.x;   // of the keys
-  const int L = item_kv.y;           // number of keys
+  const int64_t begin = item_kv.x;
+  const int L = item_kv.y;
+  if (L <= 0 || Lq <= 0) {   // uniform.  No keys: zeros, as in varlen_attention_kernel
+    for (int i = threadIdx.x; i < kQTile * (HD / 8); i += 256) {
+      const int row = q0 + i / (HD / 8);
+      if (Lq > 0 && row < Lq) {
+        const u32x4 z = {0, 0, 0, 0};
+        __builtin_memcpy(reinterpret_cast<char*>(O + (q_begin + row) * ldo + h * HD + (i % (HD / 8)) * 8), &z, 16);
+      }
+    }
+    return;
+  }
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -349,13 +404,14 @@ __global__ __launch_bounds__(256, (HD > 64 ? 2 : NT_ATTN_WAVES_PER_EU)) void var
   const bool wave_active = (q0 + wave * 32) < Lq;
   Frag qf[kQF];
   {
-    // rows past Lq read the last row; their results are never stored
     const int qr = q_row < Lq ? q_row : Lq - 1;
     const T* qp = Q + (q_begin + qr) * ldq + h * HD + g * 8;
 #pragma unroll
     for (int s = 0; s < kQF; ++s) {
       u32x4 v = load16_unaligned(reinterpret_cast<const char*>(qp + s * 16));
-      __builtin_memcpy(&qf[s], &v, 16);
+      Frag f;
+      __builtin_memcpy(&f, &v, 16);
+      qf[s] = QScale<T>::run(f, scale_log2e);
     }
   }
 
@@ -364,21 +420,24 @@ __global__ __launch_bounds__(256, (HD > 64 ? 2 : NT_ATTN_WAVES_PER_EU)) void var
   for (int i = 0; i < kDB; ++i)
 #pragma unroll
     for (int e = 0; e < 16; ++e) o_acc[i][e] = 0.0f;
-  float m_run = -INFINITY;
+  acc16 negm;           // -m_ref in every element
+#pragma unroll
+  for (int e = 0; e < 16; ++e) negm[e] = 0.0f;
+  float l_run = 0.0f;   // this lane's share of the row's denominator
 
   const int ntiles = (L + kKTile - 1) / kKTile;
   const T* kbase = K + begin * ldk + h * HD;
   const T* vbase = Vt + (int64_t)h * HD * ldvt + begin;
 
-  // Each thread moves HD / 32 16-byte pieces of a K tile and as many of a V^T tile.
-  // The loads are unconditional and unmasked (clamped addresses), so that the
-  // wavefront only waits for them where the data is stored to LDS.  All per-thread
-  // addressing is set up once; a step only advances pointers.
-  const int r0 = tid >> 3;      // V^T: row of piece 0 (piece i: r0 + 32 i), keys 8 cc .. 8 cc + 7
+  const int r0 = tid >> 3;
   const int cc = tid & 7;
-  const int kr0 = tid / kKPieces;   // K: row of piece 0 (piece i: kr0 + i * kKRowsPerPass)
-  const int kc = tid % kKPieces;    //    elements 8 kc .. 8 kc + 7 of the row
-  u32x4 rk[kKP], rv[kVP];
+  const int kr0 = tid / kKPieces;
+  const int kc = tid % kKPieces;
+  // one tile of K and V^T pieces on its way from global memory to LDS
+  struct Stage {
+    u32x4 k[kKP], v[kVP];
+  };
+  Stage st;
   const char* k_last = reinterpret_cast<const char*>(kbase + (int64_t)(L - 1) * ldk + kc * 8);
   const int64_t k_step = (int64_t)kKTile * ldk * (int64_t)sizeof(T);
   const char* v_ptr[kVP];
@@ -386,39 +445,30 @@ __global__ __launch_bounds__(256, (HD > 64 ? 2 : NT_ATTN_WAVES_PER_EU)) void var
   for (int i = 0; i < kVP; ++i) {
     v_ptr[i] = reinterpret_cast<const char*>(vbase + (int64_t)(r0 + i * 32) * ldvt + cc * 8);
   }
-  auto gload_k = [&](int t_in) {
+  auto gload = [&](Stage& sg, int t_in) {
     const int t = t_in < ntiles ? t_in : ntiles - 1;   // past the end: re-read, never used
     const char* tile = reinterpret_cast<const char*>(kbase + kc * 8) + t * k_step;
 #pragma unroll
     for (int i = 0; i < kKP; ++i) {
+      // LDS row `row` holds the key with bits 2 and 3 of the row index exchanged;
       // rows past L read row L - 1 (a valid key: it cannot raise the row maximum)
       const int row = kr0 + i * kKRowsPerPass;
-      const int kr = t * kKTile + row;
-      const char* src = tile + (int64_t)row * ldk * (int64_t)sizeof(T);
-      rk[i] = load16_unaligned(kr < L ? src : k_last);
+      const int key = (row & ~12) | ((row & 4) << 1) | ((row & 8) >> 1);
+      const int kr = t * kKTile + key;
+      const char* src = tile + (int64_t)key * ldk * (int64_t)sizeof(T);
+      sg.k[i] = load16_unaligned(kr < L ? src : k_last);
     }
-  };
-  auto gload_v = [&](int t_in) {
-    const int t = t_in < ntiles ? t_in : ntiles - 1;
-    // V^T piece: keys key0 .. key0+7 of row d, read where it lies (the rows of Vt
+    // V^T piece: keys 8 cc .. 8 cc + 7 of row d, read where it lies (the rows of Vt
     // are readable 72 elements past the last token)
 #pragma unroll
     for (int i = 0; i < kVP; ++i) {
-      rv[i] = load16_unaligned(v_ptr[i] + t * (kKTile * (int)sizeof(T)));
+      sg.v[i] = load16_unaligned(v_ptr[i] + t * (kKTile * (int)sizeof(T)));
     }
   };
-  auto lstore_k = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < kKP; ++i) {
-      store16(&lds_k[buf][(kr0 + i * kKRowsPerPass) * kKR + kc * 16], rk[i]);
-    }
-  };
-  // piece cc = keys 8cc .. 8cc+7 = (ks = cc/2, a = cc%2); its low half (g = 0)
-  // goes to position 16ks + 4a, its high half (g = 1) to 16ks + 8 + 4a.
-  const int v_lo = (16 * (cc >> 1) + 4 * (cc & 1)) * 2;
-  // keys at or past L are zeroed in the last tile: a probability must not meet
-  // a NaN there, and the ones row must not count them
-  uint32_t vm[4];
+  // V^T columns of keys at or past L are zeroed in the last tile: their
+  // probabilities are zero (below), and 0 * x must not meet a NaN or an infinity
+  // in whatever follows the sequence in memory
+  u32x4 vm;
   {
     int nv = L - ((ntiles - 1) * kKTile + cc * 8);
     nv = nv > 8 ? 8 : (nv < 0 ? 0 : nv);
@@ -427,158 +477,165 @@ __global__ __launch_bounds__(256, (HD > 64 ? 2 : NT_ATTN_WAVES_PER_EU)) void var
       vm[j] = nv >= 2 * j + 2 ? 0xffffffffu : (nv == 2 * j + 1 ? 0x0000ffffu : 0u);
     }
   }
-  // Row 64 of a V^T buffer: 1 for every valid key.  Multiplied with P^T by the
-  // matrix pipe it yields the softmax denominators, and because it is zero past L
-  // (like the V^T columns) the keys of a partial tile need no masking of their
-  // scores.  Full tiles share the all-ones row written here once; the last tile
-  // writes its own masked row.
-  if (r0 == 0) {
-    const uint64_t ones = ((uint64_t)AT::kOnePair << 32) | AT::kOnePair;
+  auto lstore = [&](const Stage& sg, int buf, int t) {
 #pragma unroll
-    for (int b2 = 0; b2 < 2; ++b2) {
-      char* row = &lds_v[b2][HD * kVRow + v_lo];
-      *reinterpret_cast<uint64_t*>(row) = ones;
-      *reinterpret_cast<uint64_t*>(row + 16) = ones;
+    for (int i = 0; i < kKP; ++i) {
+      store16(&lds_k[buf][(kr0 + i * kKRowsPerPass) * kKR + kc * 16], sg.k[i]);
     }
-  }
-  auto lstore_v = [&](int buf, int t) {
-    if (t < ntiles - 1) {   // uniform: a full tile, nothing to mask
+    if (t < ntiles - 1) {   // uniform: a full tile
 #pragma unroll
-      for (int i = 0; i < kVP; ++i) {
-        char* row = &lds_v[buf][(r0 + i * 32) * kVRow + v_lo];
-        *reinterpret_cast<uint64_t*>(row) = ((uint64_t)rv[i].y << 32) | rv[i].x;
-        *reinterpret_cast<uint64_t*>(row + 16) = ((uint64_t)rv[i].w << 32) | rv[i].z;
-      }
+      for (int i = 0; i < kVP; ++i) store16(&lds_v[buf][(r0 + i * 32) * kVRow + cc * 16], sg.v[i]);
       return;
     }
 #pragma unroll
-    for (int i = 0; i < kVP; ++i) {
-      char* row = &lds_v[buf][(r0 + i * 32) * kVRow + v_lo];
-      const uint64_t lo = ((uint64_t)(rv[i].y & vm[1]) << 32) | (rv[i].x & vm[0]);
-      const uint64_t hi = ((uint64_t)(rv[i].w & vm[3]) << 32) | (rv[i].z & vm[2]);
-      *reinterpret_cast<uint64_t*>(row) = lo;
-      *reinterpret_cast<uint64_t*>(row + 16) = hi;
-    }
-    if (r0 == 0) {
-      char* row = &lds_v[buf][HD * kVRow + v_lo];
-      const uint64_t lo = ((uint64_t)(AT::kOnePair & vm[1]) << 32) | (AT::kOnePair & vm[0]);
-      const uint64_t hi = ((uint64_t)(AT::kOnePair & vm[3]) << 32) | (AT::kOnePair & vm[2]);
-      *reinterpret_cast<uint64_t*>(row) = lo;
-      *reinterpret_cast<uint64_t*>(row + 16) = hi;
-    }
+    for (int i = 0; i < kVP; ++i) store16(&lds_v[buf][(r0 + i * 32) * kVRow + cc * 16], sg.v[i] & vm);
   };
+  const int n_last = L - (ntiles - 1) * kKTile;   // keys of the last tile, 1..64
 
-  // S^T tile of K tile in lds_k[buf]:
-  // s[kb][e] = score(key = 64 t + 32 kb + 8 (e/4) + 4 g + e%4, q = l32)
-  auto scores = [&](acc16 (&sa)[2], int buf) {
+  // The body of a tile is written in the order it should issue, and fenced so
+  // that it does: matrix instructions execute in the background while the
+  // wavefront goes on issuing vector instructions, but only if the two kinds
+  // alternate in the instruction stream (the scheduler would otherwise group
+  // all exponentials in front of all PV products).  NT_FENCE keeps the
+  // scheduler from moving anything across it.
+#define NT_FENCE() __builtin_amdgcn_sched_barrier(0)
+  auto tile = [&](int buf, bool first, bool partial) {
+    // S^T - m_ref: s[kb][e] belongs to LDS row 32 kb + 8 (e/4) + 4 g + e%4 of the K tile
+    const char* krow = &lds_k[buf][l32 * kKR + g * 16];
+    Frag kf[2][kQF];
+    auto read_k = [&](int kb, int s0, int s1) {
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+      for (int s = s0; s < s1; ++s)
+        kf[kb][s] = *reinterpret_cast<const Frag*>(krow + kb * 32 * kKR + s * 32);
+    };
+    read_k(0, 0, kQF);
+    read_k(1, 0, kQF / 2);
+    NT_FENCE();
+    acc16 sa[2];
 #pragma unroll
-      for (int e = 0; e < 16; ++e) sa[kb][e] = 0.0f;
-      const char* krow = &lds_k[buf][(kb * 32 + l32) * kKR + g * 16];
+    for (int s = 0; s < kQF; ++s) sa[0] = AT::mma(kf[0][s], qf[s], s == 0 ? negm : sa[0]);
+    read_k(1, kQF / 2, kQF);
 #pragma unroll
-      for (int s = 0; s < kQF; ++s) {
-        Frag kf = *reinterpret_cast<const Frag*>(krow + s * 32);
-        sa[kb] = AT::mma(kf, qf[s], sa[kb]);
-      }
-    }
-  };
-
-  // Online softmax of one tile's scores, then O^T += V^T P^T and the
-  // denominators l += 1^T P^T from lds_v[vbuf].
-  //
-  // Keys past L in a partial tile: their K rows are copies of row L - 1, so they
-  // cannot raise the row maximum; their V^T columns and their entries of the ones
-  // row are zero, so they add nothing to O or l.  No score is ever masked.
-  acc16 l_acc;
-#pragma unroll
-  for (int e = 0; e < 16; ++e) l_acc[e] = 0.0f;
-  auto softmax_pv = [&](acc16 (&sa)[2], int vbuf) {
+    for (int s = 0; s < kQF / 2; ++s) sa[1] = AT::mma(kf[1][s], qf[s], s == 0 ? negm : sa[1]);
+    NT_FENCE();
+    // the maximum of the first block while the second one is in the matrix pipe
     float m_tile = sa[0][0];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+    for (int e = 1; e < 16; ++e) m_tile = fmaxf(m_tile, sa[0][e]);
+    NT_FENCE();
 #pragma unroll
-      for (int e = 0; e < 16; ++e) m_tile = fmaxf(m_tile, sa[kb][e]);
+    for (int s = kQF / 2; s < kQF; ++s) sa[1] = AT::mma(kf[1][s], qf[s], sa[1]);
+    NT_FENCE();
+    // V^T fragments of k-step 0 travel while the maximum is finished
+    Frag vf[2][kDB];
+    const char* vrow = &lds_v[buf][l32 * kVRow + g * 16];
+    auto read_v = [&](int ks) {
+#pragma unroll
+      for (int db = 0; db < kDB; ++db)
+        vf[ks & 1][db] = *reinterpret_cast<const Frag*>(vrow + db * 32 * kVRow + ks * 32);
+    };
+    read_v(0);
+    NT_FENCE();
+#pragma unroll
+    for (int e = 0; e < 16; ++e) m_tile = fmaxf(m_tile, sa[1][e]);
     m_tile = max_across_halves(m_tile);
-    const float m_new = fmaxf(m_run, m_tile);   // finite: every tile holds a valid key
-    // raw v_exp_f32: arguments are <= 0, results in [0, 1]
-    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
-    const float m_scaled = m_new * scale_log2e;
-    m_run = m_new;
-    // the running maxima settle after the first tiles; then alpha is 1 in
-    // every lane and the multiplications are skipped (wavefront-uniform)
-    if (__any(alpha != 1.0f)) {
+    if (partial) {
+      // last tile, fewer than 64 keys: the K rows past L are copies of row L - 1
+      // (they cannot have raised the maximum); their probabilities become zero
 #pragma unroll
-      for (int i = 0; i < kDB; ++i)
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
-      l_acc[0] *= alpha;   // every element of l_acc holds the same sum; [0] is the one read
-    }
-    Frag pf[4];   // P^T as B-operand: k-step ks = 2 kb + half uses sa[kb][8 half .. +8]
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        uint32_t w[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float p0 =
-              __builtin_amdgcn_exp2f(fmaf(sa[kb][half * 8 + 2 * j], scale_log2e, -m_scaled));
-          const float p1 =
-              __builtin_amdgcn_exp2f(fmaf(sa[kb][half * 8 + 2 * j + 1], scale_log2e, -m_scaled));
-          w[j] = AT::cvt2(p0, p1);
+        for (int e = 0; e < 16; ++e) {
+          // key of LDS row 32 kb + 8 (e/4) + 4 g + e%4: bits 2 and 3 exchanged
+          const int key = 32 * kb + 16 * (e >> 3) + 8 * g + 4 * ((e >> 2) & 1) + (e & 3);
+          if (key >= n_last) sa[kb][e] = -INFINITY;
         }
-        __builtin_memcpy(&pf[kb * 2 + half], w, 16);
+    }
+    if (first || __any(m_tile > kLazyMaxLog2)) {   // wavefront-uniform
+      // raise (first tile: set) the reference maximum of every row by delta
+      const float delta = first ? m_tile : fmaxf(m_tile, 0.0f);
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sa[kb][e] -= delta;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) negm[e] -= delta;
+      if (!first) {
+        const float alpha = __builtin_amdgcn_exp2f(-delta);
+#pragma unroll
+        for (int i = 0; i < kDB; ++i)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+        l_run *= alpha;
       }
     }
+    // the compiler must not see that the elements of negm are equal: it would
+    // rebuild the block from one register in front of every use
+    asm volatile("" : "+v"(negm));
+    // probabilities of k-step ks = 2 kb + half: sa[kb][8 half .. 8 half + 8)
+    float pr[8];
+    uint32_t pw[4][4];
+    auto exps = [&](int ks, int j0, int j1) {
+#pragma unroll
+      for (int j = j0; j < j1; ++j) pr[j] = __builtin_amdgcn_exp2f(sa[ks >> 1][(ks & 1) * 8 + j]);
+    };
+    auto cvts = [&](int ks) {
+      // the denominator sums the rounded probabilities, the ones that meet V
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        pw[ks][j] = AT::cvt2(pr[2 * j], pr[2 * j + 1]);
+        l_run = AT::dot_ones(pw[ks][j], l_run);
+      }
+    };
+    exps(0, 0, 8);
+    cvts(0);
+    NT_FENCE();
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
+      if (ks < 3) read_v(ks + 1);
+      Frag pf;
+      __builtin_memcpy(&pf, pw[ks], 16);
+      NT_FENCE();
 #pragma unroll
-      for (int db = 0; db < kDB; ++db) {
-        const char* vrow = &lds_v[vbuf][(db * 32 + l32) * kVRow + g * 16];
-        Frag vf = *reinterpret_cast<const Frag*>(vrow + ks * 32);
-        o_acc[db] = AT::mma(vf, pf[ks], o_acc[db]);
+      for (int m = 0; m < kDB; ++m) {
+        o_acc[m] = AT::mma(vf[ks & 1][m], pf, o_acc[m]);
+        NT_FENCE();
+        if (ks < 3) {
+          // the next k-step's eight exponentials, spread over this one's matrix instructions
+          exps(ks + 1, 8 * m / kDB, 8 * (m + 1) / kDB);
+          if (m == kDB - 1) cvts(ks + 1);
+          NT_FENCE();
+        }
       }
-      // all 32 rows of this A-operand are the ones row: every lane gets l[q]
-      Frag of = *reinterpret_cast<const Frag*>(&lds_v[vbuf][HD * kVRow + g * 16 + ks * 32]);
-      l_acc = AT::mma(of, pf[ks], l_acc);
     }
   };
-
   // Tile t + 1 travels global -> registers while tile t is computed, and goes
   // registers -> LDS (the other buffer) after the compute, before the barrier.
-  // Wavefronts of other workgroups on the SIMD (three fit) fill the matrix pipe
-  // while this one runs its softmax, and the other way round.
-  gload_k(0);
-  gload_v(0);
-  lstore_k(0);
-  lstore_v(0, 0);
+  // (Giving the loads two tiles of time to arrive, with a second register set,
+  // was measured: no change.)
+  gload(st, 0);
+  lstore(st, 0, 0);
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
     const int buf = t & 1;
-    gload_k(t + 1);   // past the end: re-reads the last tile
-    gload_v(t + 1);
+    gload(st, t + 1);   // past the end: re-reads the last tile
     // keep the loads above the MFMA / softmax work (the scheduler would sink them)
     __builtin_amdgcn_sched_barrier(0);
-    if (wave_active) {
-      acc16 sa[2];
-      scores(sa, buf);
-      softmax_pv(sa, buf);
-    }
-    lstore_k(buf ^ 1);          // past the end: harmless, the buffer is not read again
-    lstore_v(buf ^ 1, t + 1);
+    if (wave_active) tile(buf, t == 0, t == ntiles - 1 && n_last < kKTile);
+    lstore(st, buf ^ 1, t + 1);   // past the end: harmless, the buffer is not read again
     __syncthreads();
   }
 
-  if (!wave_active || q_row >= Lq) return;
-  const float l_tot = l_acc[0];
+  if (!wave_active) return;
+  // lanes l and l ^ 32 hold the two halves of a row's keys
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  if (q_row >= Lq) return;
   const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
   T* op = O + (q_begin + q_row) * ldo + h * HD;
 #pragma unroll
   for (int db = 0; db < kDB; ++db) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      // d = 32 db + 8 r + 4 g + (0..3)
       uint32_t w0 = AT::cvt2(o_acc[db][r * 4 + 0] * inv, o_acc[db][r * 4 + 1] * inv);
       uint32_t w1 = AT::cvt2(o_acc[db][r * 4 + 2] * inv, o_acc[db][r * 4 + 3] * inv);
       uint64_t bits = ((uint64_t)w1 << 32) | w0;

@@ -206,7 +206,12 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
     // lane fetches: slot p of row r holds piece p ^ ((r >> 1) & 7).  The compiler
     // does not see these loads (inline asm), so their completion is awaited by hand
     // before the barrier that publishes the tile.  The asm writes M0 (the LDS
-    // destination) and says so in its clobber list.
+    // destination).  M0 cannot be declared as a clobber: the compiler treats it as a
+    // reserved register, warns and ignores the entry.  The s_mov and the load that
+    // reads M0 sit in one asm statement, so the compiler cannot put anything
+    // between them; in the other direction the rule for this file is that nothing
+    // makes the compiler keep a value of its own in M0 across these statements (no
+    // LDS-direct builtin, no dynamic register indexing, no sendmsg).
     static_assert(Cfg::kRowBytes == 128 && Cfg::kBM % 8 == 0, "1 KiB blocks of eight rows");
     constexpr int kN = Cfg::kPerThread;
     constexpr int kWaves = Cfg::kThreads / 64;
@@ -237,7 +242,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
             lds_base + (unsigned)(buf * Cfg::kDmaTileBytes + (i * kWaves + wave) * 1024));
         const char* src = gptr[i] + kt * Cfg::kRowBytes;
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                     :: "v"(src), "s"(dst) : "memory", "m0");
+                     :: "v"(src), "s"(dst) : "memory");
       }
     };
     const int sw = (l32 >> 1) & 7;

@@ -197,18 +197,30 @@ extern "C" int nt_value_row_counts(const void* data, int elem_type, double paddi
   if (R == 0) return NT_OK;
   if (!counts || (M > 0 && !data)) return fail(NT_ERR_INVALID_ARGUMENT, "value_row_counts: NULL pointer");
   hipStream_t s = (hipStream_t)stream;
+  // `tensor != padding` as torch evaluates it: a floating tensor compares in its
+  // own type, i.e. against the padding ROUNDED to that type (0.1 is not a half);
+  // an integer tensor compares exactly against an integral padding, and in fp32
+  // (torch's promotion of integer tensor and floating scalar) against any other.
+  const bool integral = padding == (double)(int64_t)padding && padding >= -9.2e18 && padding <= 9.2e18;
+  const int64_t ipad = integral ? (int64_t)padding : 0;
+#define NT_INT_CASE(TYPE)                                                                          \
+  if (integral) return launch_row_counts(data, R, M, NotEqual<TYPE, int64_t>{ipad}, counts, prefix, s); \
+  return launch_row_counts(data, R, M, NotEqual<TYPE, float>{(float)padding}, counts, prefix, s);
   switch (elem_type) {
     case NT_F32: return launch_row_counts(data, R, M, NotEqual<float, float>{(float)padding}, counts, prefix, s);
-    case NT_F16: return launch_row_counts(data, R, M, NotEqual<_Float16, float>{(float)padding}, counts, prefix, s);
-    case NT_BF16: return launch_row_counts(data, R, M, NotEqual<__bf16, float>{(float)padding}, counts, prefix, s);
+    case NT_F16:
+      return launch_row_counts(data, R, M, NotEqual<_Float16, float>{(float)(_Float16)padding}, counts, prefix, s);
+    case NT_BF16:
+      return launch_row_counts(data, R, M, NotEqual<__bf16, float>{(float)(__bf16)(float)padding}, counts, prefix, s);
     case NT_F64: return launch_row_counts(data, R, M, NotEqual<double, double>{padding}, counts, prefix, s);
-    case NT_I8: return launch_row_counts(data, R, M, NotEqual<int8_t, double>{padding}, counts, prefix, s);
-    case NT_U8: return launch_row_counts(data, R, M, NotEqual<uint8_t, double>{padding}, counts, prefix, s);
-    case NT_I16: return launch_row_counts(data, R, M, NotEqual<int16_t, double>{padding}, counts, prefix, s);
-    case NT_I32: return launch_row_counts(data, R, M, NotEqual<int32_t, double>{padding}, counts, prefix, s);
-    case NT_I64: return launch_row_counts(data, R, M, NotEqual<int64_t, double>{padding}, counts, prefix, s);
+    case NT_I8: NT_INT_CASE(int8_t)
+    case NT_U8: NT_INT_CASE(uint8_t)
+    case NT_I16: NT_INT_CASE(int16_t)
+    case NT_I32: NT_INT_CASE(int32_t)
+    case NT_I64: NT_INT_CASE(int64_t)
     default: return fail(NT_ERR_INVALID_ARGUMENT, "value_row_counts: unknown element type %d", elem_type);
   }
+#undef NT_INT_CASE
 }
 
 extern "C" int nt_compact_rows(const void* data, const uint8_t* mask, const int64_t* row_offsets,

@@ -210,7 +210,7 @@ extern "C" int nt_offsets_from_sizes(const int64_t* sizes, int64_t B, int64_t D,
   return run_scan(load, B, offsets, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
-extern "C" int64_t nt_offsets_noalloc_max_B(void) { return kNoAllocMaxB; }
+extern "C" int64_t nt_offsets_noalloc_max_count(void) { return kNoAllocMaxB; }
 
 extern "C" int nt_offsets_from_sizes_noalloc(const int64_t* sizes, int64_t B, int64_t D,
                                              int64_t* offsets, void* stream) {

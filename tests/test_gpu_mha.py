@@ -393,3 +393,119 @@ def test_min_mha_under_hip_graph_replays():
         exp = layer()._impl.buffer
         torch.cuda.synchronize()
         assert torch.equal(got, exp), "replay %d differs from the eager layer" % rep
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("K", [128, 320, 512, 896])
+def test_linear_k_tile_counts_on_the_256x128_shape(K, dtype):
+    # K = 2, 5, 8, 14 tiles of 64: every residue of the three-buffer ring of the
+    # 256 x 128 tile shape (N = 128 admits no other shape), whose last iterations
+    # re-read the final K tile into a buffer the epilogue then reuses
+    from nestedtensor_amd import ops
+    M, N = 700, 128
+    g = torch.Generator().manual_seed(K)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) * K ** -0.5).to(dtype)
+    b = torch.randn(N, generator=g).to(dtype)
+    xd, wd, bd = x.to(DEV), w.to(DEV), b.to(DEV)
+    exp = x.float() @ w.float().t() + b.float()
+    first = ops.linear(xd, wd, bd)
+    for _ in range(5):     # the same launch again and again: no run may differ
+        assert torch.equal(ops.linear(xd, wd, bd), first)
+    tol = 2e-2 if dtype == torch.float16 else 6e-2
+    assert (first.float().cpu() - exp).abs().max().item() <= tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("order", ["rising", "falling", "spike"])
+def test_attention_reference_maximum_moves(dtype, order):
+    """Scores that grow along the keys by far more than the slack the kernel allows
+    its reference maximum (2^8): the maximum is raised and the accumulators are
+    rescaled on every tile ("rising"), never after the first ("falling"), or once in
+    the middle ("spike")."""
+    H, hd = 2, 64
+    E = H * hd
+    L = 300
+    g = torch.Generator().manual_seed(5)
+    u = torch.randn(E, generator=g)
+    u = u / u.norm() * 8.0
+    amp = torch.linspace(0.2, 3.0, L)
+    if order == "falling":
+        amp = amp.flip(0)
+    elif order == "spike":
+        amp = torch.full((L,), 0.3)
+        amp[170] = 3.0
+    x = (amp[:, None] * u[None, :] + 0.05 * torch.randn(L, E, generator=g)).to(dtype)
+    short = (0.5 * torch.randn(40, E, generator=g)).to(dtype)
+    # identity-like projections keep q . k ~ amp_i amp_j |u|^2 / H per head
+    W_in = torch.cat([torch.eye(E), torch.eye(E), torch.eye(E)]).to(dtype)
+    b_in = torch.zeros(3 * E, dtype=dtype)
+    W_out = torch.eye(E).to(dtype)
+    b_out = torch.zeros(E, dtype=dtype)
+    xs = [x, short]
+    got = run_min_mha(H, hd, xs, W_in, b_in, W_out, b_out, dtype)
+    ref = oracle.ref_nested_tensor(xs, dtype=dtype)
+    exp = oracle.min_mha(H, hd, 0.0, False, ref, ref, ref, W_in, b_in, hd ** -0.5, W_out, b_out)
+    # the reference rounds q * scaling and the scores to the storage type, which
+    # at scores of this size (up to ~36) moves its own result; compare with the
+    # float64 answer as well
+    ref64 = oracle.ref_nested_tensor([p.double() for p in xs], dtype=torch.float64)
+    exp64 = oracle.min_mha(H, hd, 0.0, False, ref64, ref64, ref64, W_in.double(), b_in.double(),
+                           hd ** -0.5, W_out.double(), b_out.double())
+    gotf = got._impl.buffer.float().cpu()
+    e64 = torch.cat([p.reshape(-1) for p in exp64]).float()
+    e = torch.cat([p.reshape(-1) for p in exp]).float()
+    assert torch.isfinite(gotf).all()
+    err64 = (gotf - e64).abs().max().item()
+    ref_err64 = (e - e64).abs().max().item()
+    assert err64 <= max(HALF_ABS, ref_err64 + HALF_ABS / 4), (err64, ref_err64)
+
+
+def test_attention_vt_items_without_keys_or_queries():
+    # through the C ABI: a work item with key length 0 writes zeros to its query
+    # rows, one with query length 0 writes nothing
+    from nestedtensor_amd import _C
+    H, hd = 2, 64
+    E = H * hd
+    T = 200
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(T, E, generator=g).half().to(DEV)
+    k = torch.randn(T, E, generator=g).half().to(DEV)
+    ldvt = T + 72
+    vt = torch.randn(E, ldvt, generator=g).half().to(DEV)
+    out = torch.full((T, E), 7.0, dtype=torch.float16, device=DEV)
+    # item 0: queries 0..129 (two tiles) without keys; item 2: no queries; item 3: a real one
+    sched = torch.tensor([[0, 130, 0, 0, 0, 0, 0, 0],
+                          [0, 130, 128, 0, 0, 0, 0, 0],
+                          [130, 0, 0, 0, 130, 20, 0, 0],
+                          [150, 50, 0, 0, 150, 50, 0, 0]], dtype=torch.int32, device=DEV)
+    _C.check(_C.lib.nt_varlen_attention_vt(_C.ptr(q), E, _C.ptr(k), E, _C.ptr(vt), ldvt, _C.ptr(out), E,
+                                           _C.ptr(sched), 4, H, hd, T, 0.125, _C.dtype_code(torch.float16),
+                                           _C.current_stream(DEV)))
+    torch.cuda.synchronize()
+    o = out.float().cpu()
+    assert (o[:130] == 0).all()
+    assert (o[130:150] == 7).all()
+    qs, ks, vs = q[150:].float().cpu(), k[150:].float().cpu(), vt[:, 150:200].float().cpu().t()
+    for h in range(H):
+        sl = slice(h * hd, (h + 1) * hd)
+        p = torch.softmax(qs[:, sl] @ ks[:, sl].t() * 0.125, dim=-1)
+        assert (o[150:, sl] - p @ vs[:, sl]).abs().max().item() <= HALF_ABS
+
+
+# (num_heads, batch_size, seq_len_, head_size): the four largest shapes of
+# test/test_nested_tensor_functional.py:1155-1160
+REF_SHAPES_LARGE = [(16, 128, 50, 16), (16, 256, 50, 16), (4, 256, 50, 256), (16, 256, 50, 64)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("H,B,Lmax,hd", REF_SHAPES_LARGE)
+def test_min_mha_reference_shapes_large(dtype, H, B, Lmax, hd):
+    random.seed(H * 1000 + B)
+    lens = [random.randint(1, Lmax) for _ in range(B)]
+    E = H * hd
+    xs, W_in, b_in, W_out, b_out = make_case(E, lens, 19, dtype, w_std=E ** -0.5, bias_std=0.1)
+    got = run_min_mha(H, hd, xs, W_in, b_in, W_out, b_out, dtype)
+    ref = oracle.ref_nested_tensor(xs, dtype=dtype)
+    exp = oracle.min_mha(H, hd, 0.0, False, ref, ref, ref, W_in, b_in, hd ** -0.5, W_out, b_out)
+    check(got, exp, dtype)

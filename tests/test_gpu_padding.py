@@ -555,3 +555,28 @@ def test_from_padded_value_non_prefix_takes_compaction_path():
     got2 = nt.nested_tensor_from_padded_tensor(t2.to(DEV))
     assert got2.nested_size().unbind() == exp2.nested_size()
     bits_equal(got2._impl.buffer, exp2.buffer)
+
+
+@pytest.mark.parametrize("dtype,padding", [(torch.float16, 0.1), (torch.bfloat16, 0.1), (torch.bfloat16, 1e-3),
+                                           (torch.float32, 0.1), (torch.int64, -1), (torch.int32, 0.5)])
+def test_from_padded_tensor_compares_in_the_tensors_own_type(dtype, padding):
+    # `tensor != padding` rounds the padding to the tensor's type first: 0.1 as a
+    # half is 0.0999755859375, and elements holding exactly that are padding
+    B, L, E = 6, 9, 4
+    g = torch.Generator().manual_seed(77)
+    lens = [int(v) for v in torch.randint(1, L + 1, (B,), generator=g)]
+    lens[0] = L
+    if dtype.is_floating_point:
+        pad_t = torch.tensor(padding, dtype=dtype)
+        padded = pad_t.expand(B, L, E).clone()
+        for b, n in enumerate(lens):
+            padded[b, :n] = torch.randn(n, E, generator=g).to(dtype) + 3.0
+    else:
+        padded = torch.full((B, L, E), int(padding) if float(padding).is_integer() else 0, dtype=dtype)
+        for b, n in enumerate(lens):
+            padded[b, :n] = torch.randint(1 << 40 if dtype == torch.int64 else 5, (1 << 40) + 50 if dtype == torch.int64 else 90,
+                                          (n, E), generator=g).to(dtype)
+    mask = padded != padding          # torch's own comparison, on the host
+    got = nt.nested_tensor_from_padded_tensor(padded.to(DEV), padding=padding)
+    exp = oracle.nested_tensor_from_tensor_mask(padded, mask)
+    nt_matches(got, exp.unbind(), dtype)

@@ -58,7 +58,7 @@ def test_noalloc_offsets_beyond_int32():
 
 
 def test_noalloc_offsets_rejects_sizes_beyond_the_scratch():
-    limit = _C.lib.nt_offsets_noalloc_max_B()
+    limit = _C.lib.nt_offsets_noalloc_max_count()
     assert limit == 32768 * 2048
     sizes = torch.ones((8, 1), dtype=torch.int64, device=DEV)
     out = torch.full((9,), 7, dtype=torch.int64, device=DEV)
