@@ -96,6 +96,23 @@ def _load():
 
 lib = _load()
 
+OPS_PATH = os.path.join(_HERE, "_torch_ops.so")
+
+
+def _load_ops():
+    """The operator layer: the C++ torch extension that registers the
+    ``nestedtensor`` operator library (csrc/torch_ops.cpp).  No fallback either."""
+    if not os.path.exists(OPS_PATH):
+        raise ImportError(
+            "nestedtensor_amd: %s is missing. Build it with `make -C %s` "
+            "(or __graft_entry__.build()); there is no fallback path."
+            % (OPS_PATH, os.path.join(_HERE, "csrc")))
+    torch.ops.load_library(OPS_PATH)
+    return torch.ops.nestedtensor
+
+
+ops = _load_ops()
+
 
 def check(rc):
     if rc != NT_OK:

@@ -1,0 +1,725 @@
+// Operator layer of nestedtensor_amd as a C++ torch extension.
+//
+// The reference registers its operators from C++ with TORCH_LIBRARY_IMPL on its
+// own dispatch key and a custom TensorImpl (nestedtensor/csrc/masking.cpp:652-675,
+// csrc/mha.cpp:71-74, csrc/cuda/mha.cpp:109-113, csrc/py_init.cpp:132-216).  That
+// key belongs to torch core now, so a nested tensor crosses the dispatcher in
+// lowered form: (packed buffer, sizes[B, D], offsets[B + 1]).  This file
+//
+//   * defines the schemas of the reference's operators (same names, same argument
+//     order; their `Tensor nt` argument is the Python wrapper, which
+//     __torch_function__ lowers before the dispatcher sees it), and
+//   * defines and implements, for the HIP device key, the lowered operators that
+//     do the work: host code here only validates, sizes outputs, allocates them
+//     from torch's caching allocator and calls the C ABI of
+//     include/nestedtensor_amd.h on torch's current stream.
+//
+// Nothing here computes on the host except nested sizes (integers): converting a
+// dense tensor + mask to a nested tensor needs the per-row keep-counts on the
+// host to size its output, which is one device-to-host copy into pinned memory.
+#include <ATen/ATen.h>
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/library.h>
+
+#include <cstring>
+#include <tuple>
+#include <vector>
+
+#include "../../include/nestedtensor_amd.h"
+
+namespace {
+
+using at::Tensor;
+
+inline void check(int rc) {
+  if (rc != NT_OK) {
+    const char* msg = nt_last_error();
+    TORCH_CHECK(false, "nestedtensor_amd: ", (msg && *msg) ? msg : "error", " (code ", rc, ")");
+  }
+}
+
+inline void require_device(const Tensor& t, const char* what) {
+  TORCH_CHECK(t.is_cuda(), "nestedtensor_amd: ", what, " runs on the HIP device only; got a tensor on ",
+              t.device(), ". Move the nested tensor with .to('cuda') first.");
+}
+
+inline void* stream_of(const Tensor& t) {
+  return static_cast<void*>(c10::hip::getCurrentHIPStream(t.device().index()).stream());
+}
+
+inline int elem_bytes(at::ScalarType st) {
+  const int n = static_cast<int>(c10::elementSize(st));
+  // masking.cpp:622 returns an uninitialised tensor for other dtypes; raise instead.
+  TORCH_CHECK(n == 1 || n == 2 || n == 4 || n == 8, "Input datatype ", st, " is not supported.");
+  return n;
+}
+
+inline int elem_type(at::ScalarType st) {
+  switch (st) {
+    case at::kFloat: return NT_F32;
+    case at::kHalf: return NT_F16;
+    case at::kBFloat16: return NT_BF16;
+    case at::kDouble: return NT_F64;
+    case at::kChar: return NT_I8;
+    case at::kByte: return NT_U8;
+    case at::kShort: return NT_I16;
+    case at::kInt: return NT_I32;
+    case at::kLong: return NT_I64;
+    default: return -1;
+  }
+}
+
+inline int dtype_code(at::ScalarType st) {
+  switch (st) {
+    case at::kFloat: return NT_F32;
+    case at::kHalf: return NT_F16;
+    case at::kBFloat16: return NT_BF16;
+    default: TORCH_CHECK(false, "nestedtensor_amd: dtype ", st, " is not supported by this op");
+  }
+}
+
+// The padding value converted the way the reference converts it, (T)(double)
+// (masking.cpp:594,610), as raw bits in the low bytes.
+uint64_t pad_bits(double padding, at::ScalarType st) {
+  uint64_t bits = 0;
+  switch (st) {
+    case at::kFloat: { const float v = static_cast<float>(padding); std::memcpy(&bits, &v, 4); break; }
+    case at::kDouble: std::memcpy(&bits, &padding, 8); break;
+    case at::kHalf: { const c10::Half v(static_cast<float>(padding)); bits = v.x; break; }
+    case at::kBFloat16: { const c10::BFloat16 v(static_cast<float>(padding)); bits = v.x; break; }
+    case at::kBool: bits = padding != 0.0 ? 1 : 0; break;
+    case at::kChar: case at::kByte: bits = static_cast<uint64_t>(static_cast<int64_t>(padding)) & 0xffu; break;
+    case at::kShort: bits = static_cast<uint64_t>(static_cast<int64_t>(padding)) & 0xffffu; break;
+    case at::kInt: bits = static_cast<uint64_t>(static_cast<int64_t>(padding)) & 0xffffffffu; break;
+    case at::kLong: bits = static_cast<uint64_t>(static_cast<int64_t>(padding)); break;
+    default: TORCH_CHECK(false, "Input datatype ", st, " is not supported.");
+  }
+  return bits;
+}
+
+// ---- metadata ---------------------------------------------------------------
+
+// offsets[b] = sum_{c<b} prod_k sizes[c, k] on the device (nt_offsets_from_sizes).
+Tensor offsets_from_sizes(const Tensor& sizes_dev) {
+  require_device(sizes_dev, "device metadata");
+  TORCH_CHECK(sizes_dev.scalar_type() == at::kLong && sizes_dev.dim() == 2 && sizes_dev.is_contiguous(),
+              "offsets_from_sizes: sizes must be a contiguous int64 [B, D] tensor");
+  const int64_t B = sizes_dev.size(0), D = sizes_dev.size(1);
+  c10::hip::HIPGuard guard(sizes_dev.device().index());
+  Tensor offsets = at::empty({B + 1}, sizes_dev.options());
+  const size_t ws_bytes = nt_offsets_workspace_bytes(B);
+  Tensor ws;
+  if (ws_bytes) ws = at::empty({static_cast<int64_t>(ws_bytes)}, sizes_dev.options().dtype(at::kByte));
+  check(nt_offsets_from_sizes(sizes_dev.const_data_ptr<int64_t>(), B, D, offsets.data_ptr<int64_t>(),
+                              ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, stream_of(sizes_dev)));
+  return offsets;
+}
+
+// ---- packed <-> padded --------------------------------------------------------
+
+struct PadArgs {
+  int64_t B, D;
+  std::vector<int64_t> out_shape;
+};
+
+PadArgs pad_args(const Tensor& buffer, const Tensor& sizes_dev, const Tensor& offsets_dev,
+                 at::IntArrayRef padded_sizes, int64_t n_ragged, const char* what) {
+  require_device(buffer, what);
+  TORCH_CHECK(sizes_dev.dim() == 2 && sizes_dev.scalar_type() == at::kLong && sizes_dev.is_contiguous() &&
+                  sizes_dev.device() == buffer.device(),
+              what, ": sizes must be a contiguous int64 [B, D] tensor on the buffer's device");
+  PadArgs a;
+  a.B = sizes_dev.size(0);
+  a.D = sizes_dev.size(1);
+  TORCH_CHECK(offsets_dev.numel() == a.B + 1 && offsets_dev.scalar_type() == at::kLong &&
+                  offsets_dev.is_contiguous() && offsets_dev.device() == buffer.device(),
+              what, ": offsets must be a contiguous int64 [B + 1] tensor on the buffer's device");
+  TORCH_CHECK(static_cast<int64_t>(padded_sizes.size()) == a.D, what, ": one padded extent per constituent dim");
+  TORCH_CHECK(n_ragged >= 1 && n_ragged <= 3, what, " supports at most 3 irregular dimensions.");
+  a.out_shape.reserve(a.D + 1);
+  a.out_shape.push_back(a.B);
+  for (int64_t v : padded_sizes) a.out_shape.push_back(v);
+  return a;
+}
+
+// to_padded_tensor (masking.cpp:558-625) on the lowered form.
+Tensor add_padding(const Tensor& buffer, const Tensor& sizes_dev, const Tensor& offsets_dev,
+                   at::IntArrayRef padded_sizes, int64_t n_ragged, double padding) {
+  const PadArgs a = pad_args(buffer, sizes_dev, offsets_dev, padded_sizes, n_ragged, "to_padded_tensor");
+  c10::hip::HIPGuard guard(buffer.device().index());
+  Tensor out = at::empty(a.out_shape, buffer.options());
+  check(nt_add_padding(buffer.const_data_ptr(), out.data_ptr(), offsets_dev.const_data_ptr<int64_t>(),
+                       sizes_dev.const_data_ptr<int64_t>(), a.B, a.D, n_ragged, padded_sizes.data(),
+                       elem_bytes(buffer.scalar_type()), pad_bits(padding, buffer.scalar_type()),
+                       stream_of(buffer)));
+  return out;
+}
+
+// to_tensor_mask when the mask keeps every dim of the data, and pad_nt
+// (masking.cpp:138-179, 251-296): data and mask in one launch.
+std::tuple<Tensor, Tensor> add_padding_mask(const Tensor& buffer, const Tensor& sizes_dev,
+                                            const Tensor& offsets_dev, at::IntArrayRef padded_sizes,
+                                            int64_t n_ragged, double padding) {
+  const PadArgs a = pad_args(buffer, sizes_dev, offsets_dev, padded_sizes, n_ragged, "to_tensor_mask");
+  c10::hip::HIPGuard guard(buffer.device().index());
+  Tensor out = at::empty(a.out_shape, buffer.options());
+  Tensor mask = at::empty(a.out_shape, buffer.options().dtype(at::kBool));
+  check(nt_add_padding_mask(buffer.const_data_ptr(), out.data_ptr(), static_cast<uint8_t*>(mask.data_ptr()),
+                            offsets_dev.const_data_ptr<int64_t>(), sizes_dev.const_data_ptr<int64_t>(), a.B,
+                            a.D, n_ragged, padded_sizes.data(), elem_bytes(buffer.scalar_type()),
+                            pad_bits(padding, buffer.scalar_type()), stream_of(buffer)));
+  return std::make_tuple(out, mask);
+}
+
+// from_padded_tensor (masking.cpp:459-509) on the lowered form: the entries of
+// `padded` inside the nested size, packed.  total_numel = offsets[B] as the host knows it.
+Tensor remove_padding(const Tensor& padded_in, const Tensor& sizes_dev, const Tensor& offsets_dev,
+                      int64_t total_numel, int64_t n_ragged) {
+  require_device(padded_in, "from_padded_tensor");
+  const Tensor padded = padded_in.contiguous();
+  const PadArgs a = pad_args(padded, sizes_dev, offsets_dev, padded.sizes().slice(1), n_ragged,
+                             "from_padded_tensor");
+  TORCH_CHECK(padded.size(0) == a.B, "Target size has a different batch size than the padded Tensor.");
+  c10::hip::HIPGuard guard(padded.device().index());
+  Tensor out = at::empty({total_numel}, padded.options());
+  if (total_numel == 0) return out;
+  const at::IntArrayRef ext = padded.sizes().slice(1);
+  check(nt_remove_padding(padded.const_data_ptr(), out.data_ptr(), offsets_dev.const_data_ptr<int64_t>(),
+                          sizes_dev.const_data_ptr<int64_t>(), a.B, a.D, n_ragged, ext.data(),
+                          elem_bytes(padded.scalar_type()), stream_of(padded)));
+  return out;
+}
+
+// Bool mask over [B, ext...] from the nested size (nt_build_mask): to_mask, and the
+// collapsed mask of to_tensor_mask (masking.cpp:322-457).
+Tensor build_mask(const Tensor& sizes_dev, at::IntArrayRef ext) {
+  require_device(sizes_dev, "to_tensor_mask");
+  TORCH_CHECK(sizes_dev.dim() == 2 && sizes_dev.scalar_type() == at::kLong && sizes_dev.is_contiguous(),
+              "build_mask: sizes must be a contiguous int64 [B, D] tensor");
+  const int64_t B = sizes_dev.size(0), D = sizes_dev.size(1), K = static_cast<int64_t>(ext.size());
+  TORCH_CHECK(K >= 1 && K <= 3 && K <= D, "masks over more than 3 constituent dimensions are not supported.");
+  std::vector<int64_t> shape;
+  shape.push_back(B);
+  for (int64_t v : ext) shape.push_back(v);
+  c10::hip::HIPGuard guard(sizes_dev.device().index());
+  Tensor mask = at::empty(shape, sizes_dev.options().dtype(at::kBool));
+  check(nt_build_mask(static_cast<uint8_t*>(mask.data_ptr()), sizes_dev.const_data_ptr<int64_t>(), B, D, K,
+                      ext.data(), stream_of(sizes_dev)));
+  return mask;
+}
+
+// ---- dense + mask -> nested ----------------------------------------------------
+
+// Result of a dense -> nested conversion in lowered form.  sizes is a host int64
+// [B, D] tensor (0-d for an empty nested tensor, EfficientSizeNode.h:8-12);
+// sizes_dev / offsets_dev are its device mirror and the element offsets when the
+// conversion had to build them anyway (undefined tensors otherwise).
+struct Lowered {
+  Tensor buffer, sizes, sizes_dev, offsets_dev;
+};
+
+Lowered empty_nt() {
+  // nested_tensor([]): Packed.h:77-79, EfficientSizeNode.h:10-12
+  return {at::ones({0}, at::kFloat), at::zeros({}, at::kLong), Tensor(), Tensor()};
+}
+
+Tensor sizes_from_shapes(const std::vector<std::vector<int64_t>>& shapes) {
+  const int64_t n = static_cast<int64_t>(shapes.size());
+  const int64_t d = static_cast<int64_t>(shapes[0].size());
+  for (const auto& s : shapes) {
+    TORCH_CHECK(static_cast<int64_t>(s.size()) == d, "Given Tensor / NestedTensor constiuent of dimension ",
+                s.size(), " doesn't match another constiuent of dimension ", d, ". ");
+  }
+  Tensor sizes = at::empty({n, d}, at::kLong);
+  int64_t* p = sizes.data_ptr<int64_t>();
+  for (const auto& s : shapes)
+    for (int64_t v : s) *p++ = v;
+  return sizes;
+}
+
+// Every tensor[i] is a constituent, whole (masking.cpp:228-232).
+Lowered keep_all(const Tensor& tensor) {
+  const int64_t B = tensor.size(0);
+  if (B == 0) return empty_nt();
+  std::vector<int64_t> shape(tensor.sizes().begin() + 1, tensor.sizes().end());
+  Tensor sizes = at::empty({B, static_cast<int64_t>(shape.size())}, at::kLong);
+  int64_t* p = sizes.data_ptr<int64_t>();
+  for (int64_t b = 0; b < B; ++b)
+    for (int64_t v : shape) *p++ = v;
+  return {tensor.contiguous().reshape({-1}).clone(), sizes, Tensor(), Tensor()};
+}
+
+Tensor as_byte_mask(const Tensor& mask) {
+  if (mask.scalar_type() == at::kBool) return mask.contiguous().view(at::kByte);
+  if (mask.scalar_type() == at::kByte) return mask.contiguous();
+  return mask.ne(0).contiguous().view(at::kByte);
+}
+
+// Pinned staging memory for the one device-to-host copy of a conversion; grows,
+// never shrinks, one per host thread.
+Tensor& pinned_staging(int64_t bytes) {
+  static thread_local Tensor buf;
+  if (!buf.defined() || buf.numel() < bytes) {
+    int64_t cap = 1 << 16;
+    while (cap < bytes) cap <<= 1;
+    buf = at::empty({cap}, at::TensorOptions().dtype(at::kByte).pinned_memory(true));
+  }
+  return buf;
+}
+
+// Device keep-counts (int32) and is-a-prefix flags (uint8) of R rows in ONE
+// device buffer [4 R bytes of counts | R bytes of flags], so that both reach the
+// host in one copy.
+struct RowStats {
+  Tensor raw;           // device, uint8 [5 R]
+  int32_t* counts_dev;
+  uint8_t* prefix_dev;
+};
+
+RowStats alloc_row_stats(const Tensor& like, int64_t R) {
+  RowStats s;
+  s.raw = at::empty({5 * R + 16}, like.options().dtype(at::kByte));
+  s.counts_dev = reinterpret_cast<int32_t*>(s.raw.data_ptr());
+  s.prefix_dev = static_cast<uint8_t*>(s.raw.data_ptr()) + 4 * R;
+  return s;
+}
+
+// Scan the per-row keep-counts and move the kept chunks (nt_exclusive_scan_i32,
+// nt_compact_rows).  Returns the packed 1-D buffer.
+Tensor compact(const Tensor& data, const Tensor& bmask, int64_t R, int64_t M, int64_t chunk_elems,
+               int64_t total_kept, const int32_t* counts_dev) {
+  Tensor out = at::empty({total_kept * chunk_elems}, data.options());
+  if (total_kept == 0 || chunk_elems == 0) return out;
+  Tensor row_offsets = at::empty({R + 1}, data.options().dtype(at::kLong));
+  const size_t ws_bytes = nt_scan_workspace_bytes(R);
+  Tensor ws;
+  if (ws_bytes) ws = at::empty({static_cast<int64_t>(ws_bytes)}, data.options().dtype(at::kByte));
+  void* stream = stream_of(data);
+  check(nt_exclusive_scan_i32(counts_dev, R, row_offsets.data_ptr<int64_t>(), ws_bytes ? ws.data_ptr() : nullptr,
+                              ws_bytes, stream));
+  check(nt_compact_rows(data.const_data_ptr(), static_cast<const uint8_t*>(bmask.const_data_ptr()),
+                        row_offsets.const_data_ptr<int64_t>(), R, M,
+                        chunk_elems * static_cast<int64_t>(data.element_size()), out.data_ptr(), stream));
+  return out;
+}
+
+// Upload sizes[B, D] and the element offsets computed from them in one copy.
+void upload_meta(const Tensor& sizes, const Tensor& like, Tensor* sizes_dev, Tensor* offsets_dev, int64_t* total) {
+  const int64_t B = sizes.size(0), D = sizes.size(1);
+  const int64_t n = B * D + B + 1;
+  Tensor& stage = pinned_staging(n * 8);
+  int64_t* h = reinterpret_cast<int64_t*>(stage.data_ptr());
+  const int64_t* s = sizes.const_data_ptr<int64_t>();
+  std::memcpy(h, s, static_cast<size_t>(B * D) * 8);
+  int64_t* off = h + B * D;
+  int64_t acc = 0;
+  for (int64_t b = 0; b < B; ++b) {
+    off[b] = acc;
+    int64_t prod = 1;
+    for (int64_t k = 0; k < D; ++k) prod *= s[b * D + k];
+    acc += prod;
+  }
+  off[B] = acc;
+  *total = acc;
+  Tensor meta = at::empty({n}, like.options().dtype(at::kLong));
+  hipStream_t stream = c10::hip::getCurrentHIPStream(like.device().index()).stream();
+  C10_HIP_CHECK(hipMemcpyAsync(meta.data_ptr(), h, static_cast<size_t>(n) * 8, hipMemcpyHostToDevice, stream));
+  // the staging buffer is reused by the next conversion of this thread: the copy
+  // must have left it
+  C10_HIP_CHECK(hipStreamSynchronize(stream));
+  *sizes_dev = meta.narrow(0, 0, B * D).view({B, D});
+  *offsets_dev = meta.narrow(0, B * D, B + 1);
+}
+
+// General case of nt_from_tensor_mask (masking.cpp:203-222) for a mask over the
+// first `mask_dims` dims of `tensor`.  Rows = everything but the last mask dim.
+// `count_rows` fills device (counts, prefix flags); `byte_mask` materialises the
+// mask, which only the non-prefix path needs.
+template <class CountRows, class ByteMask>
+Lowered from_rows(const Tensor& tensor, int64_t mask_dims, CountRows count_rows, ByteMask byte_mask) {
+  const int64_t B = tensor.size(0);
+  const at::IntArrayRef shape = tensor.sizes();
+  const int64_t M = shape[mask_dims - 1];
+  int64_t R = 1;
+  for (int64_t k = 0; k + 1 < mask_dims; ++k) R *= shape[k];
+  std::vector<int64_t> rest(shape.begin() + mask_dims, shape.end());
+  int64_t chunk = 1;
+  for (int64_t v : rest) chunk *= v;
+  // count_shape = [B] + shape[1 : mask_dims - 1]; per constituent rows_per = R / B
+  const int64_t levels = mask_dims - 1;            // mask dims below the batch dim
+  const int64_t rows_per = B > 0 ? R / B : 0;
+
+  TORCH_CHECK(R <= (int64_t(1) << 26), "nested_tensor_from_tensor_mask: ", R,
+              " mask rows exceed what this conversion stages on the host (67 108 864)");
+  c10::hip::HIPGuard guard(tensor.device().index());
+  RowStats st = alloc_row_stats(tensor, R);
+  count_rows(R, M, st.counts_dev, st.prefix_dev);
+  // one device-to-host copy: the row counts and the "row keeps a prefix" flags
+  Tensor& stage = pinned_staging(5 * R + 16);
+  hipStream_t stream = c10::hip::getCurrentHIPStream(tensor.device().index()).stream();
+  if (R > 0) {
+    C10_HIP_CHECK(hipMemcpyAsync(stage.data_ptr(), st.raw.const_data_ptr(), static_cast<size_t>(5 * R),
+                                 hipMemcpyDeviceToHost, stream));
+    C10_HIP_CHECK(hipStreamSynchronize(stream));
+  }
+  const int32_t* counts = reinterpret_cast<const int32_t*>(stage.data_ptr());
+  const uint8_t* prefix = static_cast<const uint8_t*>(stage.data_ptr()) + 4 * R;
+
+  // Nested size from the counts: at every mask level the extent is the number of
+  // children that keep anything (masking.cpp:203-222); the selection must be
+  // rectangular or at::stack would have thrown.  `leading`: the kept children
+  // come first at every level.
+  bool leading = true;
+  for (int64_t r = 0; r < R; ++r) leading = leading && prefix[r] != 0;
+  std::vector<int64_t> total(B, 0);
+  std::vector<std::vector<int64_t>> extents(B, std::vector<int64_t>(levels, 0));   // outermost first
+  std::vector<uint8_t> alive, next;
+  for (int64_t b = 0; b < B; ++b) {
+    const int32_t* c = counts + b * rows_per;
+    int64_t sum = 0, mx = 0;
+    for (int64_t r = 0; r < rows_per; ++r) {
+      sum += c[r];
+      if (c[r] > mx) mx = c[r];
+    }
+    total[b] = sum;
+    extents[b][levels - 1] = mx;
+    // walk the mask levels upwards: alive[i] = child i keeps anything
+    alive.assign(rows_per, 0);
+    for (int64_t r = 0; r < rows_per; ++r) alive[r] = c[r] > 0;
+    int64_t n = rows_per;
+    for (int64_t lev = levels - 2; lev >= 0; --lev) {
+      const int64_t width = shape[lev + 1];      // children per parent at this level
+      const int64_t parents = n / width;
+      next.assign(parents, 0);
+      int64_t mxc = 0;
+      for (int64_t p = 0; p < parents; ++p) {
+        int64_t cnt = 0;
+        for (int64_t i = 0; i < width; ++i) {
+          const uint8_t a = alive[p * width + i];
+          if (i > 0 && a > alive[p * width + i - 1]) leading = false;
+          cnt += a;
+        }
+        next[p] = cnt > 0;
+        if (cnt > mxc) mxc = cnt;
+      }
+      extents[b][lev] = mxc;
+      alive.swap(next);
+      n = parents;
+    }
+  }
+  std::vector<std::vector<int64_t>> shapes(B);
+  int64_t kept_total = 0;
+  for (int64_t b = 0; b < B; ++b) {
+    int64_t prod = 1;
+    for (int64_t v : extents[b]) prod *= v;
+    TORCH_CHECK(prod == total[b], "stack expects each tensor to be equal size: the mask does not select "
+                                  "a rectangular block in every constituent.");
+    kept_total += total[b];
+    if (total[b] != 0) {
+      shapes[b] = extents[b];
+      shapes[b].insert(shapes[b].end(), rest.begin(), rest.end());
+    } else {
+      shapes[b].assign(shape.begin() + 1, shape.begin() + mask_dims - 1);
+      shapes[b].push_back(0);
+    }
+  }
+  if (B == 0) return empty_nt();
+  Tensor sizes = sizes_from_shapes(shapes);
+  if (leading) {
+    // Every constituent keeps a leading box: this is the length-based un-pad
+    // (nt_remove_padding) with the nested size just derived.
+    const int64_t D = sizes.size(1);
+    TORCH_CHECK(D == tensor.dim() - 1, "Target size has different dimension as input padded Tensor.");
+    Tensor sizes_dev, offsets_dev;
+    int64_t numel = 0;
+    upload_meta(sizes, tensor, &sizes_dev, &offsets_dev, &numel);
+    // dims up to the last one that differs between constituents, or from the
+    // padded extent, are walked as ragged
+    int64_t n_ragged = 1;
+    const int64_t* s = sizes.const_data_ptr<int64_t>();
+    for (int64_t k = 0; k < D; ++k) {
+      bool regular = true;
+      for (int64_t b = 0; b < B && regular; ++b) regular = s[b * D + k] == shape[k + 1];
+      if (!regular) n_ragged = k + 1;
+    }
+    TORCH_CHECK(n_ragged <= 3, "from_padded_tensor supports at most 3 irregular dimensions.");
+    Tensor out = remove_padding(tensor, sizes_dev, offsets_dev, numel, n_ragged);
+    return {out, sizes, sizes_dev, offsets_dev};
+  }
+  Tensor buf = compact(tensor, byte_mask(), R, M, chunk, kept_total, st.counts_dev);
+  return {buf, sizes, Tensor(), Tensor()};
+}
+
+// nt_from_tensor_mask (masking.cpp:181-249) at nested_dim 1.
+Lowered from_mask(const Tensor& tensor_in, const Tensor& mask_in, int64_t nested_dim) {
+  TORCH_CHECK(nested_dim == 1, "Only nested_dim of 1 is currently supported.");
+  // masking.cpp:228-234: an empty mask or a single true keeps everything, a single
+  // false keeps nothing.
+  if (mask_in.numel() == 0) return keep_all(tensor_in);
+  if (mask_in.numel() == 1) {
+    return mask_in.reshape({-1})[0].item<bool>() ? keep_all(tensor_in) : empty_nt();
+  }
+  TORCH_CHECK(tensor_in.device() == mask_in.device(), "tensor and mask must be on the same device.");
+  require_device(tensor_in, "nested_tensor_from_tensor_mask");
+  TORCH_CHECK(mask_in.dim() <= tensor_in.dim(), "Mask has more dimensions than the data tensor.");
+  const int64_t B = tensor_in.size(0);
+  TORCH_CHECK_INDEX(mask_in.size(0) >= B, "index ", mask_in.size(0), " is out of bounds for dimension 0 with size ", B);
+  const Tensor mask = mask_in.narrow(0, 0, B);
+  const Tensor tensor = tensor_in.contiguous();
+  const Tensor bmask = as_byte_mask(mask);
+  int64_t inner_numel = 1;
+  for (int64_t k = 1; k < mask.dim(); ++k) inner_numel *= mask.size(k);
+  c10::hip::HIPGuard guard(tensor.device().index());
+
+  if (inner_numel == 1) {
+    // One mask value per constituent (masking.cpp:186-201 on mask[i]): true keeps
+    // tensor[i] whole; false drops it (0-d mask[i]) or leaves an empty constituent
+    // of shape [1, .., 1, 0].
+    const int64_t row_elems = B > 0 ? tensor[0].numel() : 0;
+    Tensor keep_host = mask.reshape({B}).to(at::kBool).cpu();
+    const bool* keep = keep_host.const_data_ptr<bool>();
+    int64_t kept = 0;
+    for (int64_t b = 0; b < B; ++b) kept += keep[b];
+    RowStats st = alloc_row_stats(tensor, 1);
+    check(nt_mask_row_counts(static_cast<const uint8_t*>(bmask.const_data_ptr()), 1, B, st.counts_dev,
+                             st.prefix_dev, stream_of(tensor)));
+    Tensor buf = compact(tensor, bmask, 1, B, row_elems, kept, st.counts_dev);
+    std::vector<int64_t> full(tensor.sizes().begin() + 1, tensor.sizes().end());
+    if (mask.dim() == 1) {
+      if (kept == 0) return empty_nt();
+      std::vector<std::vector<int64_t>> shapes(kept, full);
+      return {buf, sizes_from_shapes(shapes), Tensor(), Tensor()};
+    }
+    std::vector<int64_t> empty_shape(mask.dim() - 2, 1);
+    empty_shape.push_back(0);
+    std::vector<std::vector<int64_t>> shapes;
+    for (int64_t b = 0; b < B; ++b) shapes.push_back(keep[b] ? full : empty_shape);
+    if (shapes.empty()) return empty_nt();
+    return {buf, sizes_from_shapes(shapes), Tensor(), Tensor()};
+  }
+  for (int64_t k = 1; k < mask.dim(); ++k) {
+    TORCH_CHECK(tensor.size(k) == mask.size(k), "Mask of shape ", mask.sizes(),
+                " does not match the leading dimensions of the data tensor ", tensor.sizes(), ".");
+  }
+  return from_rows(
+      tensor, mask.dim(),
+      [&](int64_t R, int64_t M, int32_t* counts, uint8_t* prefix) {
+        check(nt_mask_row_counts(static_cast<const uint8_t*>(bmask.const_data_ptr()), R, M, counts, prefix,
+                                 stream_of(tensor)));
+      },
+      [&]() { return bmask; });
+}
+
+// nested_tensor_from_padded_tensor (nested/masking.py:12-14) on the device: the
+// mask `tensor != padding` has the dims of the data and is never materialised
+// unless the selection is not a leading box.
+Lowered from_value(const Tensor& tensor_in, double padding, int64_t nested_dim) {
+  TORCH_CHECK(nested_dim == 1, "Only nested_dim of 1 is currently supported.");
+  require_device(tensor_in, "nested_tensor_from_padded_tensor");
+  const int et = elem_type(tensor_in.scalar_type());
+  TORCH_CHECK(et >= 0, "Input datatype ", tensor_in.scalar_type(), " is not supported.");
+  const Tensor tensor = tensor_in.contiguous();
+  return from_rows(
+      tensor, tensor.dim(),
+      [&](int64_t R, int64_t M, int32_t* counts, uint8_t* prefix) {
+        check(nt_value_row_counts(tensor.const_data_ptr(), et, padding, R, M, counts, prefix, stream_of(tensor)));
+      },
+      [&]() { return as_byte_mask(tensor.ne(padding)); });
+}
+
+std::tuple<Tensor, Tensor> nt_from_tensor_mask_op(const Tensor& tensor, const Tensor& mask, int64_t nested_dim) {
+  Lowered r = from_mask(tensor, mask, nested_dim);
+  return std::make_tuple(r.buffer, r.sizes);
+}
+
+std::tuple<Tensor, Tensor, Tensor, Tensor> from_tensor_mask_lowered(const Tensor& tensor, const Tensor& mask,
+                                                                    int64_t nested_dim) {
+  Lowered r = from_mask(tensor, mask, nested_dim);
+  return std::make_tuple(r.buffer, r.sizes, r.sizes_dev.defined() ? r.sizes_dev : at::empty({0}, at::kLong),
+                         r.offsets_dev.defined() ? r.offsets_dev : at::empty({0}, at::kLong));
+}
+
+std::tuple<Tensor, Tensor> nt_from_padded_tensor_op(const Tensor& tensor, double padding, int64_t nested_dim) {
+  Lowered r = from_value(tensor, padding, nested_dim);
+  return std::make_tuple(r.buffer, r.sizes);
+}
+
+std::tuple<Tensor, Tensor, Tensor, Tensor> from_padded_value_lowered(const Tensor& tensor, double padding,
+                                                                     int64_t nested_dim) {
+  Lowered r = from_value(tensor, padding, nested_dim);
+  return std::make_tuple(r.buffer, r.sizes, r.sizes_dev.defined() ? r.sizes_dev : at::empty({0}, at::kLong),
+                         r.offsets_dev.defined() ? r.offsets_dev : at::empty({0}, at::kLong));
+}
+
+// merge_tensor_mask (masking.cpp:12-43) on a dense (tensor, mask) pair, any
+// device: the last mask dim is dropped while every one of its rows is all ones
+// or all zeros; stops at mask_dim, and refuses a mask_dim it cannot reach.
+std::tuple<Tensor, Tensor> merge_tensor_mask(const Tensor& tensor, const Tensor& mask_in,
+                                             c10::optional<int64_t> mask_dim) {
+  Tensor mask = mask_in;
+  while (true) {
+    if (mask_dim.has_value() && mask.dim() == *mask_dim) return std::make_tuple(tensor, mask);
+    if (mask.dim() == 0) return std::make_tuple(tensor, mask);
+    const int64_t last = mask.size(-1);
+    Tensor collapsed = mask.sum(-1);
+    const int64_t uniform = collapsed.eq(last).logical_or(collapsed.eq(0)).sum().item<int64_t>();
+    if (uniform == collapsed.numel()) {
+      mask = collapsed.to(at::kBool);
+      continue;
+    }
+    TORCH_CHECK(!(mask_dim.has_value() && *mask_dim != mask.dim()),
+                "Mask dimension is too small to represent data tensor.");
+    return std::make_tuple(tensor.contiguous(), mask.contiguous());
+  }
+}
+
+// ---- packed projections and nested multi-head attention -------------------------
+
+// y = act(x @ weight.T + bias) on a 2-D row-major view (nt_linear_act): the packed
+// fast path of NestedTensor_matmul (matmul.cpp:13-41) with the packed bias add
+// (BinaryOps.cpp:97-107) and, optionally, relu / gelu (activation.cpp:11-19, 34-46)
+// in the GEMM epilogue.  act: 0 none, 1 relu, 2 gelu.
+Tensor linear_packed(const Tensor& x, const Tensor& weight_in, const c10::optional<Tensor>& bias_in, int64_t act) {
+  require_device(x, "linear");
+  TORCH_CHECK(x.dim() == 2 && weight_in.dim() == 2 && x.stride(1) == 1, "linear: x must be a 2-D row-major view");
+  TORCH_CHECK(act >= 0 && act <= 2, "linear: activation must be None, 'relu' or 'gelu'");
+  const int64_t M = x.size(0), K = x.size(1), N = weight_in.size(0);
+  TORCH_CHECK(weight_in.size(1) == K, "linear: weight of shape ", weight_in.sizes(),
+              " does not match input feature size ", K);
+  const Tensor weight = weight_in.contiguous();
+  Tensor bias;
+  if (bias_in.has_value() && bias_in->defined()) bias = bias_in->contiguous();
+  TORCH_CHECK(weight.scalar_type() == x.scalar_type() && (!bias.defined() || bias.scalar_type() == x.scalar_type()),
+              "linear: input, weight and bias must have the same dtype");
+  c10::hip::HIPGuard guard(x.device().index());
+  Tensor out = at::empty({M, N}, x.options());
+  check(nt_linear_act(x.const_data_ptr(), x.stride(0), weight.const_data_ptr(),
+                      bias.defined() ? bias.const_data_ptr() : nullptr, out.data_ptr(), N, M, N, K,
+                      static_cast<int>(act), dtype_code(x.scalar_type()), stream_of(x)));
+  return out;
+}
+
+// Self-attention layer on the packed token buffer x [T, E] (min_mha, mha.cpp:18-69;
+// bt_min_mha, cuda/mha.cpp:22-107, passes no out bias): fused QKV projection with V
+// written transposed, attention over each sequence's own keys, output projection.
+// `schedule` is the device work list of nt_varlen_attention_vt.
+Tensor mha_self_packed(const Tensor& x, const Tensor& schedule, int64_t num_heads, int64_t head_dim,
+                       const Tensor& in_proj_weight, const c10::optional<Tensor>& in_proj_bias, double scaling,
+                       const Tensor& out_proj_weight, const c10::optional<Tensor>& out_proj_bias) {
+  require_device(x, "multi-head attention");
+  const int64_t E = num_heads * head_dim;
+  TORCH_CHECK(x.dim() == 2 && x.size(1) == E && x.stride(1) == 1, "mha: x must be a [T, num_heads * head_dim] view");
+  const at::ScalarType st = x.scalar_type();
+  TORCH_CHECK(st == at::kHalf || st == at::kBFloat16, "mha_self_packed: dtype must be float16 or bfloat16");
+  TORCH_CHECK(head_dim == 32 || head_dim == 64 || head_dim == 128, "mha_self_packed: head_dim must be 32, 64 or 128");
+  const Tensor W = in_proj_weight.contiguous();
+  TORCH_CHECK(W.dim() == 2 && W.size(0) == 3 * E && W.size(1) == E,
+              "in_proj_weight must have shape [3 * embed_dim, embed_dim].");
+  Tensor b_in, b_out;
+  if (in_proj_bias.has_value() && in_proj_bias->defined()) b_in = in_proj_bias->contiguous();
+  if (out_proj_bias.has_value() && out_proj_bias->defined()) b_out = out_proj_bias->contiguous();
+  const Tensor Wo = out_proj_weight.contiguous();
+  TORCH_CHECK(W.scalar_type() == st && Wo.scalar_type() == st && (!b_in.defined() || b_in.scalar_type() == st) &&
+                  (!b_out.defined() || b_out.scalar_type() == st),
+              "linear: input, weight and bias must have the same dtype");
+  TORCH_CHECK(Wo.dim() == 2 && Wo.size(1) == E, "linear: weight of shape ", Wo.sizes(),
+              " does not match input feature size ", E);
+  TORCH_CHECK(schedule.scalar_type() == at::kInt && schedule.dim() == 2 && schedule.size(1) == 8 &&
+                  schedule.is_contiguous() && schedule.device() == x.device(),
+              "mha: schedule must be a contiguous int32 [n_work, 8] tensor on the input's device");
+  const int64_t T = x.size(0), N = Wo.size(0);
+  const int64_t ldvt = (T + 72 + 7) / 8 * 8;   // rows readable 72 elements past the last token
+  c10::hip::HIPGuard guard(x.device().index());
+  void* stream = stream_of(x);
+  const int dt = dtype_code(st);
+  Tensor qk = at::empty({T, 2 * E}, x.options());
+  Tensor vt = at::empty({E, ldvt}, x.options());
+  Tensor attn = at::empty({T, E}, x.options());
+  Tensor out = at::empty({T, N}, x.options());
+  if (T == 0) return out;
+  check(nt_linear_qkv(x.const_data_ptr(), x.stride(0), W.const_data_ptr(), b_in.defined() ? b_in.const_data_ptr() : nullptr,
+                      qk.data_ptr(), 2 * E, vt.data_ptr(), ldvt, T, E, E, dt, stream));
+  const char* kptr = static_cast<const char*>(qk.const_data_ptr()) + E * static_cast<int64_t>(x.element_size());
+  check(nt_varlen_attention_vt(qk.const_data_ptr(), 2 * E, kptr, 2 * E, vt.const_data_ptr(), ldvt, attn.data_ptr(), E,
+                               schedule.const_data_ptr<int32_t>(), schedule.size(0), num_heads, head_dim, T,
+                               static_cast<float>(scaling), dt, stream));
+  check(nt_linear_act(attn.const_data_ptr(), E, Wo.const_data_ptr(), b_out.defined() ? b_out.const_data_ptr() : nullptr,
+                      out.data_ptr(), N, T, N, E, 0, dt, stream));
+  return out;
+}
+
+}  // namespace
+
+// Schemas.  The first block are the reference's operators, names and argument
+// order as in nestedtensor/csrc/masking.cpp:652-675, csrc/mha.cpp:72,
+// csrc/cuda/mha.cpp:110-111 and csrc/py_init.cpp:132-216; a `Tensor nt` argument
+// is the Python NestedTensor wrapper, lowered by its __torch_function__.  The
+// second block are the lowered operators implemented in this file.
+TORCH_LIBRARY(nestedtensor, m) {
+  m.def("to_padded_tensor(Tensor nt, float padding) -> Tensor");
+  m.def("to_tensor_mask(Tensor nt, int? mask_dim) -> (Tensor, Tensor)");
+  m.def("to_mask(Tensor nt, int? mask_dim) -> Tensor");
+  m.def("nt_from_tensor_mask(Tensor tensor, Tensor mask, int nested_dim) -> (Tensor, Tensor)");
+  m.def("get_max_size(Tensor nt) -> int[]");
+  m.def("pad_nt(Tensor nt, int[] shape) -> (Tensor, Tensor)");
+  m.def("merge_tensor_mask(Tensor tensor, Tensor mask, int? mask_dim=None) -> (Tensor, Tensor)");
+  m.def("min_mha(int num_heads, int head_dim, float dropout_p, bool training, Tensor query, "
+        "Tensor key, Tensor value, Tensor in_proje_weight, Tensor? in_proj_bias, float scaling, "
+        "Tensor out_proj_weight, Tensor out_proj_bias) -> Tensor");
+  m.def("bt_min_mha(int num_heads, int head_dim, float dropout_p, bool training, Tensor query, "
+        "Tensor key, Tensor value, Tensor attr_kernel, Tensor attr_bias, float scaling, "
+        "Tensor out_proj_weight, Tensor out_proj_bias) -> Tensor");
+  m.def("is_nested_tensor_impl(Tensor tensor) -> bool");
+  m.def("nested_dim(Tensor tensor) -> int");
+  m.def("to_nested_tensor(Tensor tensor, int? dim) -> Tensor");
+  m.def("sizes(Tensor tensor) -> int?[]");
+  m.def("len(Tensor self) -> int");
+  m.def("get_dim(Tensor self) -> int");
+  m.def("get_numel(Tensor self) -> int");
+  m.def("get_is_contiguous(Tensor self, MemoryFormat memory_format) -> bool");
+  m.def("make_contiguous(Tensor self) -> Tensor");
+  m.def("to_tensor_list(Tensor tensor) -> Tensor[]");
+  m.def("transpose_nhwc_nchw(Tensor self) -> Tensor");
+  m.def("transpose_nchw_nhwc(Tensor self) -> Tensor");
+  m.def("to_sparse_csr(Tensor tensor) -> Tensor");
+  // no counterpart among the reference's ops (it builds the mask in Python,
+  // nestedtensor/nested/masking.py:12-14); same lowered return convention as
+  // nt_from_tensor_mask: (packed buffer, sizes[B, D]), sizes 0-d for an empty result
+  m.def("nt_from_padded_tensor(Tensor tensor, float padding, int nested_dim) -> (Tensor, Tensor)");
+
+  m.def("offsets_from_sizes(Tensor sizes) -> Tensor");
+  m.def("add_padding(Tensor buffer, Tensor sizes, Tensor offsets, int[] padded_sizes, int n_ragged, "
+        "float padding) -> Tensor");
+  m.def("add_padding_mask(Tensor buffer, Tensor sizes, Tensor offsets, int[] padded_sizes, int n_ragged, "
+        "float padding) -> (Tensor, Tensor)");
+  m.def("remove_padding(Tensor padded, Tensor sizes, Tensor offsets, int total_numel, int n_ragged) -> Tensor");
+  m.def("build_mask(Tensor sizes, int[] extents) -> Tensor");
+  m.def("from_tensor_mask_lowered(Tensor tensor, Tensor mask, int nested_dim) -> (Tensor, Tensor, Tensor, Tensor)");
+  m.def("from_padded_value_lowered(Tensor tensor, float padding, int nested_dim) -> (Tensor, Tensor, Tensor, Tensor)");
+  m.def("linear_packed(Tensor x, Tensor weight, Tensor? bias, int act) -> Tensor");
+  m.def("mha_self_packed(Tensor x, Tensor schedule, int num_heads, int head_dim, Tensor in_proj_weight, "
+        "Tensor? in_proj_bias, float scaling, Tensor out_proj_weight, Tensor? out_proj_bias) -> Tensor");
+}
+
+// "CUDA" is the dispatch key of the HIP device on PyTorch-ROCm.
+TORCH_LIBRARY_IMPL(nestedtensor, CUDA, m) {
+  m.impl("offsets_from_sizes", offsets_from_sizes);
+  m.impl("add_padding", add_padding);
+  m.impl("add_padding_mask", add_padding_mask);
+  m.impl("remove_padding", remove_padding);
+  m.impl("build_mask", build_mask);
+  m.impl("from_padded_value_lowered", from_padded_value_lowered);
+  m.impl("nt_from_padded_tensor", nt_from_padded_tensor_op);
+  m.impl("linear_packed", linear_packed);
+  m.impl("mha_self_packed", mha_self_packed);
+}
+
+// Operators on plain tensors of any device: merge_tensor_mask is host logic over
+// torch reductions; nt_from_tensor_mask answers the trivial masks (empty, one
+// element) for any device and raises for host tensors otherwise.
+TORCH_LIBRARY_IMPL(nestedtensor, CompositeExplicitAutograd, m) {
+  m.impl("merge_tensor_mask", merge_tensor_mask);
+  m.impl("nt_from_tensor_mask", nt_from_tensor_mask_op);
+  m.impl("from_tensor_mask_lowered", from_tensor_mask_lowered);
+}

@@ -176,6 +176,14 @@ class NestedTensorImpl:
         self._attn_schedule = (kv.sizes, sched)      # holds kv.sizes, so the identity test stays valid
         return sched
 
+    def adopt_device_metadata(self, sizes_dev, offsets_dev):
+        """Take over device copies of the nested size and of the element offsets
+        that a conversion has already built for this nested size."""
+        if sizes_dev.device == self.buffer.device and tuple(sizes_dev.shape) == tuple(self.sizes.shape):
+            self._sizes_dev = sizes_dev
+            if offsets_dev.numel() == self.B + 1:
+                self._offsets_dev = offsets_dev
+
     def with_buffer(self, buffer, channels_last=None):
         """Same nested size over another buffer (in the same layout unless
         channels_last says otherwise); shares the cached metadata when the
@@ -194,14 +202,9 @@ class NestedTensorImpl:
         return out
 
 
+_offsets_from_sizes = _C.ops.offsets_from_sizes.default
+
+
 def device_offsets(sizes_dev, B, D):
     """offsets[b] = sum_{c<b} prod_k sizes[c, k] on the device (nt_offsets_from_sizes)."""
-    dev = sizes_dev.device
-    offsets = torch.empty(B + 1, dtype=torch.int64, device=dev)
-    ws_bytes = _C.lib.nt_offsets_workspace_bytes(B)
-    ws = torch.empty(max(ws_bytes, 8), dtype=torch.uint8, device=dev) if ws_bytes else None
-    with _C.on_device(dev):
-        _C.check(_C.lib.nt_offsets_from_sizes(
-            _C.ptr(sizes_dev), B, D, _C.ptr(offsets), _C.ptr(ws), ws_bytes,
-            _C.current_stream(dev)))
-    return offsets
+    return _offsets_from_sizes(sizes_dev.reshape(B, D))

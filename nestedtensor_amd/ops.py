@@ -18,71 +18,28 @@ import torch
 from . import _C
 from .impl import NestedTensorImpl
 
-# ---------------------------------------------------------------------------
-# schemas (same names and argument order as the reference)
+# The schemas (same names and argument order as the reference) and the lowered
+# operators that do the work live in the C++ extension csrc/torch_ops.cpp
+# (TORCH_LIBRARY(nestedtensor, ...)), loaded by _C.  Overloads are resolved once.
+_add_padding = _C.ops.add_padding.default
+_add_padding_mask = _C.ops.add_padding_mask.default
+_remove_padding = _C.ops.remove_padding.default
+_build_mask = _C.ops.build_mask.default
+_linear_packed = _C.ops.linear_packed.default
+_mha_self_packed = _C.ops.mha_self_packed.default
 
-_lib = torch.library.Library("nestedtensor", "DEF")
-_SCHEMAS = [
-    # nestedtensor/csrc/masking.cpp:652-675
-    "to_padded_tensor(Tensor nt, float padding) -> Tensor",
-    "to_tensor_mask(Tensor nt, int? mask_dim) -> (Tensor, Tensor)",
-    "to_mask(Tensor nt, int? mask_dim) -> Tensor",
-    "nt_from_tensor_mask(Tensor tensor, Tensor mask, int nested_dim) -> (Tensor, Tensor)",
-    "get_max_size(Tensor nt) -> int[]",
-    "pad_nt(Tensor nt, int[] shape) -> (Tensor, Tensor)",
-    "merge_tensor_mask(Tensor tensor, Tensor mask, int? mask_dim=None) -> (Tensor, Tensor)",
-    # nestedtensor/csrc/mha.cpp:72, nestedtensor/csrc/cuda/mha.cpp:110-111
-    "min_mha(int num_heads, int head_dim, float dropout_p, bool training, Tensor query, "
-    "Tensor key, Tensor value, Tensor in_proje_weight, Tensor? in_proj_bias, float scaling, "
-    "Tensor out_proj_weight, Tensor out_proj_bias) -> Tensor",
-    "bt_min_mha(int num_heads, int head_dim, float dropout_p, bool training, Tensor query, "
-    "Tensor key, Tensor value, Tensor attr_kernel, Tensor attr_bias, float scaling, "
-    "Tensor out_proj_weight, Tensor out_proj_bias) -> Tensor",
-    # nestedtensor/csrc/py_init.cpp:132-216
-    "is_nested_tensor_impl(Tensor tensor) -> bool",
-    "nested_dim(Tensor tensor) -> int",
-    "to_nested_tensor(Tensor tensor, int? dim) -> Tensor",
-    "sizes(Tensor tensor) -> int?[]",
-    "len(Tensor self) -> int",
-    "get_dim(Tensor self) -> int",
-    "get_numel(Tensor self) -> int",
-    "get_is_contiguous(Tensor self, MemoryFormat memory_format) -> bool",
-    "make_contiguous(Tensor self) -> Tensor",
-    "to_tensor_list(Tensor tensor) -> Tensor[]",
-    "transpose_nhwc_nchw(Tensor self) -> Tensor",
-    "transpose_nchw_nhwc(Tensor self) -> Tensor",
-    "to_sparse_csr(Tensor tensor) -> Tensor",
-]
-for _s in _SCHEMAS:
-    _lib.define(_s)
+
+_ELEM_BYTES = {}
 
 
 def _elem_bytes(dtype):
-    n = torch.empty((), dtype=dtype).element_size()
+    n = _ELEM_BYTES.get(dtype)
+    if n is None:
+        n = _ELEM_BYTES[dtype] = torch.empty((), dtype=dtype).element_size()
     if n not in (1, 2, 4, 8):
         # masking.cpp:622 returns an uninitialised tensor for other dtypes; raise instead.
         raise RuntimeError("Input datatype %s is not supported." % dtype)
     return n
-
-
-_PAD_BITS = {}
-
-
-def _pad_bits(padding, dtype):
-    """The padding value converted the way the reference converts it,
-    ``(T)(double)`` (masking.cpp:594,610), as raw bits."""
-    key = (repr(padding), dtype)
-    if key not in _PAD_BITS:
-        if len(_PAD_BITS) > 256:
-            _PAD_BITS.clear()
-        _PAD_BITS[key] = _pad_bits_uncached(padding, dtype)
-    return _PAD_BITS[key]
-
-
-def _pad_bits_uncached(padding, dtype):
-    t = torch.tensor(padding, dtype=dtype)
-    view = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()]
-    return int(t.view(view).item()) & ((1 << (8 * t.element_size())) - 1)
 
 
 def _n_ragged(impl):
@@ -127,22 +84,11 @@ def add_padding(impl, padding, with_mask=False, shape=None):
         max_size = shape
     if nrag > 3:
         raise RuntimeError("to_padded_tensor supports at most 3 irregular dimensions.")
-    out = torch.empty([B] + max_size, dtype=impl.buffer.dtype, device=impl.buffer.device)
-    eb = _elem_bytes(impl.buffer.dtype)
-    dev = impl.buffer.device
-    with _C.on_device(dev):
-        if with_mask:
-            mask = torch.empty([B] + max_size, dtype=torch.bool, device=dev)
-            _C.check(_C.lib.nt_add_padding_mask(
-                _C.ptr(impl.buffer), _C.ptr(out), _C.ptr(mask), _C.ptr(impl.offsets_dev()),
-                _C.ptr(impl.sizes_dev()), B, D, nrag, _C.i64_array(max_size), eb,
-                _pad_bits(padding, impl.buffer.dtype), _C.current_stream(dev)))
-            return out, mask
-        _C.check(_C.lib.nt_add_padding(
-            _C.ptr(impl.buffer), _C.ptr(out), _C.ptr(impl.offsets_dev()), _C.ptr(impl.sizes_dev()),
-            B, D, nrag, _C.i64_array(max_size), eb, _pad_bits(padding, impl.buffer.dtype),
-            _C.current_stream(dev)))
-    return out
+    _elem_bytes(impl.buffer.dtype)
+    if with_mask:
+        return _add_padding_mask(impl.buffer, impl.sizes_dev(), impl.offsets_dev(), max_size, nrag,
+                                 float(padding))
+    return _add_padding(impl.buffer, impl.sizes_dev(), impl.offsets_dev(), max_size, nrag, float(padding))
 
 
 def pad_nt(impl, shape):
@@ -229,13 +175,7 @@ def build_mask(impl, kept_dims):
     K = kept_dims - 1
     if K > 3:
         raise RuntimeError("masks over more than 3 constituent dimensions are not supported.")
-    ext = impl.max_sizes()[:K]
-    mask = torch.empty([impl.B] + ext, dtype=torch.bool, device=dev)
-    with _C.on_device(dev):
-        _C.check(_C.lib.nt_build_mask(
-            _C.ptr(mask), _C.ptr(impl.sizes_dev()), impl.B, impl.D, K, _C.i64_array(ext),
-            _C.current_stream(dev)))
-    return mask
+    return _build_mask(impl.sizes_dev(), impl.max_sizes()[:K])
 
 
 def _check_mask_dim(impl, mask_dim):
@@ -326,17 +266,14 @@ def from_padded_tensor(padded, target):
             nrag = max(nrag, k + 1)
     if nrag > 3:
         raise RuntimeError("from_padded_tensor supports at most 3 irregular dimensions.")
-    dev = padded.device
-    out = torch.empty(target.numel(), dtype=padded.dtype, device=dev)
-    res = target.with_buffer(out)
-    eb = _elem_bytes(padded.dtype)
-    if out.numel() == 0:
-        return res
-    with _C.on_device(dev):
-        _C.check(_C.lib.nt_remove_padding(
-            _C.ptr(padded), _C.ptr(out), _C.ptr(res.offsets_dev()), _C.ptr(res.sizes_dev()),
-            B, D, nrag, _C.i64_array(ext), eb, _C.current_stream(dev)))
-    return res
+    _elem_bytes(padded.dtype)
+    total = target.numel()
+    if total == 0:
+        return target.with_buffer(torch.empty(0, dtype=padded.dtype, device=padded.device))
+    if target.buffer.device != padded.device:
+        target = target.with_buffer(torch.empty(0, dtype=padded.dtype, device=padded.device))
+    out = _remove_padding(padded, target.sizes_dev(), target.offsets_dev(), total, nrag)
+    return target.with_buffer(out)
 
 
 # ---------------------------------------------------------------------------
@@ -379,17 +316,7 @@ def linear(x, weight, bias, activation=None):
     if weight.size(1) != K:
         raise RuntimeError("linear: weight of shape %s does not match input feature size %d"
                            % (tuple(weight.shape), K))
-    weight = weight.contiguous()
-    if weight.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
-        raise RuntimeError("linear: input, weight and bias must have the same dtype")
-    if bias is not None:
-        bias = bias.contiguous()
-    out = torch.empty((M, N), dtype=x.dtype, device=x.device)
-    with _C.on_device(x.device):
-        _C.check(_C.lib.nt_linear_act(
-            _C.ptr(x), x.stride(0), _C.ptr(weight), _C.ptr(bias), _C.ptr(out), N, M, N, K,
-            _ACTS[activation], _C.dtype_code(x.dtype), _C.current_stream(x.device)))
-    return out
+    return _linear_packed(x, weight, bias, _ACTS[activation])
 
 
 def linear_nt(impl, weight, bias=None, activation=None):
@@ -474,20 +401,11 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
         raise RuntimeError("linear: input, weight and bias must have the same dtype")
     if fused:
         # self-attention, head_dim 32 / 64 / 128: Q|K row-major + V transposed straight out of
-        # the projection GEMM, attention reads both without any re-layout pass
-        ldvt = (T_tokens + 72 + 7) // 8 * 8   # rows readable 72 elements past the last token
-        qk = torch.empty((T_tokens, 2 * E), dtype=dtype, device=dev)
-        vt = torch.empty((E, ldvt), dtype=dtype, device=dev)
-        with _C.on_device(dev):
-            stream = _C.current_stream(dev)
-            _C.check(_C.lib.nt_linear_qkv(
-                _C.ptr(xq), xq.stride(0), _C.ptr(W), _C.ptr(in_proj_bias), _C.ptr(qk), 2 * E,
-                _C.ptr(vt), ldvt, T_tokens, E, E, _C.dtype_code(dtype), stream))
-            sched = query.attention_schedule()
-            _C.check(_C.lib.nt_varlen_attention_vt(
-                _C.ptr(qk), 2 * E, _offset_ptr(qk, E), 2 * E, _C.ptr(vt), ldvt, _C.ptr(attn), E,
-                _C.ptr(sched), sched.size(0), num_heads, head_dim, T_tokens,
-                float(scaling), _C.dtype_code(dtype), stream))
+        # the projection GEMM, attention reads both without any re-layout pass, then the
+        # output projection: three launches, issued by one call into the extension
+        out = _mha_self_packed(xq, query.attention_schedule(), num_heads, head_dim, W, in_proj_bias,
+                               float(scaling), out_proj_weight, out_proj_bias)
+        return query.with_buffer(out.reshape(-1))
     elif mfma_path and bool((key.sizes[:, 0] > 0).all()):
         # cross-attention (or an embedding size the fused projection does not tile),
         # head_dim 32 / 64 / 128: three projections (the value one written

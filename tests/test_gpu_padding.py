@@ -248,13 +248,8 @@ def test_reference_round_trip_literal_on_device():
     bits_equal(data3, exp)
 
 
-@pytest.mark.parametrize("device_reduce", [False, True])
 @pytest.mark.parametrize("mask_dims", [2, 3, 4])
-def test_from_tensor_mask_random_boxes_vs_literal_walk(mask_dims, device_reduce, monkeypatch):
-    # device_reduce: take the path of masks with many rows, where the lowest mask level is
-    # summarised on the device before the counts cross to the host
-    from nestedtensor_amd.nested import masking as _masking
-    monkeypatch.setattr(_masking, "_DEVICE_REDUCE_ROWS", 1 if device_reduce else 1 << 60)
+def test_from_tensor_mask_random_boxes_vs_literal_walk(mask_dims):
     g = torch.Generator().manual_seed(100 + mask_dims)
     for trial in range(8):
         B = 4
@@ -276,10 +271,7 @@ def test_from_tensor_mask_random_boxes_vs_literal_walk(mask_dims, device_reduce,
         nt_matches(res, exp, torch.float32)
 
 
-@pytest.mark.parametrize("device_reduce", [False, True])
-def test_from_tensor_mask_literals_both_reduction_paths(device_reduce, monkeypatch):
-    from nestedtensor_amd.nested import masking as _masking
-    monkeypatch.setattr(_masking, "_DEVICE_REDUCE_ROWS", 1 if device_reduce else 1 << 60)
+def test_from_tensor_mask_literals_and_subset_selections():
     for name, tensor, mask, parts, dtype in FROM_TENSOR_MASK:
         res = nt.nested_tensor_from_tensor_mask(tensor.to(DEV), mask.to(DEV))
         nt_matches(res, parts, dtype)
