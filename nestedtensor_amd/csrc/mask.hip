@@ -14,7 +14,7 @@
 
 namespace nt {
 
-constexpr int kRowsPerBlock = 4;  // one wavefront per row, 4 rows per workgroup
+constexpr int kRowsPerBlock = 4;  // wavefronts per workgroup of the row kernels
 
 // Predicates: a mask byte is kept if non-zero; a data element is kept if it
 // differs from the padding value with the comparison of its type (so NaN != x is
@@ -31,66 +31,94 @@ struct NotEqual {
 };
 
 // counts[r] = kept entries of row r; prefix[r] = 1 iff the kept entries are
-// exactly the first counts[r] entries of the row.  One wavefront per row; a lane
-// looks at VEC consecutive entries per step (16 bytes; one entry for short
-// rows); ballots over the lanes' "full / non-empty / is a prefix" flags decide
-// prefix-ness without any serial scan.
-template <typename P, int VEC>
+// exactly the first counts[r] entries of the row.  A wavefront takes NR
+// consecutive rows and walks them together, so that NR loads per lane are in
+// flight at a time (one row per wavefront left the memory system mostly idle: a
+// 16-byte load, then a long chain of ballots and shuffles); a lane looks at VEC
+// consecutive entries per step (16 bytes; one entry for short rows); ballots over
+// the lanes' "full / non-empty / is a prefix" flags decide prefix-ness without
+// any serial scan.  The results of a workgroup's 4 * NR rows leave through LDS as
+// two contiguous stores: the destination may be pinned host memory.
+template <typename P, int VEC, int NR>
 __global__ __launch_bounds__(kWave * kRowsPerBlock) void row_counts_kernel(
     const typename P::type* __restrict__ data, int64_t R, int64_t M, P pred,
     int32_t* __restrict__ counts, uint8_t* __restrict__ prefix) {
   typedef typename P::type T;
+  __shared__ int32_t s_count[kRowsPerBlock * NR];
+  __shared__ uint8_t s_prefix[kRowsPerBlock * NR];
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
-  if (row >= R) return;
-  const T* m = data + row * M;
-  int32_t count = 0;
-  bool is_prefix = true;
-  bool ended = false;   // an entry that is not kept has been seen (wave-uniform)
+  const int wave = threadIdx.x / kWave;
+  const int64_t block_row0 = (int64_t)blockIdx.x * (kRowsPerBlock * NR);
+  const int64_t row0 = block_row0 + wave * NR;
+  int32_t count[NR];
+  bool is_prefix[NR], ended[NR];   // ended: an entry that is not kept has been seen (wave-uniform)
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    count[r] = 0;
+    is_prefix[r] = true;
+    ended[r] = false;
+  }
   for (int64_t base = 0; base < M; base += (int64_t)kWave * VEC) {
     const int64_t i0 = base + (int64_t)lane * VEC;
-    T v[VEC];
-    if (VEC == 1) {
-      if (i0 < M) v[0] = m[i0];
-    } else {
-      if (i0 + VEC <= M) {
+    T v[NR][VEC];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+      if (row0 + r >= R) continue;
+      const T* m = data + (row0 + r) * M;
+      if (VEC == 1) {
+        if (i0 < M) v[r][0] = m[i0];
+      } else if (i0 + VEC <= M) {
         // any alignment: the part runs in unaligned-access mode
         u32x4 raw = load16_unaligned(reinterpret_cast<const char*>(m + i0));
-        __builtin_memcpy(v, &raw, 16);
+        __builtin_memcpy(v[r], &raw, 16);
       } else {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
-          if (i0 + j < M) v[j] = m[i0 + j];
+          if (i0 + j < M) v[r][j] = m[i0 + j];
         }
       }
     }
-    uint32_t flags = 0;
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      if (i0 + j < M && pred(v[j])) flags |= 1u << j;
-    }
-    const int cnt = __popc(flags);
-    count += cnt;
     // entries of this lane that exist (the last lanes of the last step hold fewer)
-    int64_t here = M - i0;
+    const int64_t here = M - i0;
     const int exist = here >= VEC ? VEC : (here > 0 ? (int)here : 0);
-    const uint64_t full = __ballot(cnt == exist && exist > 0);
-    const uint64_t nonempty = __ballot(cnt > 0);
-    const uint64_t lane_ok = __ballot(flags == ((1u << cnt) - 1u));
     const uint64_t present = __ballot(exist > 0);
-    const int q = __popcll(nonempty);
-    const uint64_t low_q = q >= 64 ? ~0ull : ((1ull << q) - 1ull);
-    const uint64_t low_qm1 = q == 0 ? 0ull : (low_q >> 1);
-    bool ok = (lane_ok == ~0ull) && (nonempty == low_q) && ((full & low_qm1) == low_qm1);
-    if (ended && nonempty != 0) ok = false;
-    is_prefix = is_prefix && ok;
-    if (full != present) ended = true;
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+      if (row0 + r >= R) continue;
+      uint32_t flags = 0;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        if (j < exist && pred(v[r][j])) flags |= 1u << j;
+      }
+      const int cnt = __popc(flags);
+      count[r] += cnt;
+      const uint64_t full = __ballot(cnt == exist && exist > 0);
+      const uint64_t nonempty = __ballot(cnt > 0);
+      const uint64_t lane_ok = __ballot(flags == ((1u << cnt) - 1u));
+      const int q = __popcll(nonempty);
+      const uint64_t low_q = q >= 64 ? ~0ull : ((1ull << q) - 1ull);
+      const uint64_t low_qm1 = q == 0 ? 0ull : (low_q >> 1);
+      bool ok = (lane_ok == ~0ull) && (nonempty == low_q) && ((full & low_qm1) == low_qm1);
+      if (ended[r] && nonempty != 0) ok = false;
+      is_prefix[r] = is_prefix[r] && ok;
+      if (full != present) ended[r] = true;
+    }
   }
 #pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) count += __shfl_xor(count, off, kWave);
-  if (lane == 0) {
-    counts[row] = count;
-    if (prefix) prefix[row] = is_prefix ? 1 : 0;
+  for (int r = 0; r < NR; ++r) {
+    int c = count[r];
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) c += __shfl_xor(c, off, kWave);
+    if (lane == 0) {
+      s_count[wave * NR + r] = c;
+      s_prefix[wave * NR + r] = is_prefix[r] ? 1 : 0;
+    }
+  }
+  __syncthreads();
+  const int t = threadIdx.x;
+  if (t < kRowsPerBlock * NR && block_row0 + t < R) {
+    counts[block_row0 + t] = s_count[t];
+    if (prefix) prefix[block_row0 + t] = s_prefix[t];
   }
 }
 
@@ -98,18 +126,23 @@ template <typename P>
 static int launch_row_counts(const void* data, int64_t R, int64_t M, P pred, int32_t* counts,
                              uint8_t* prefix, hipStream_t stream) {
   typedef typename P::type T;
-  const int64_t blocks = (R + kRowsPerBlock - 1) / kRowsPerBlock;
-  if (blocks > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "row_counts: too many rows");
   constexpr int kVec = 16 / sizeof(T);
-  dim3 grid((unsigned)blocks), block(kWave * kRowsPerBlock);
   const T* d = static_cast<const T*>(data);
-  // short rows: one entry per lane keeps more lanes busy than 16 bytes per lane
-  if (M * (int64_t)sizeof(T) >= 256) {
-    hipLaunchKernelGGL((row_counts_kernel<P, kVec>), grid, block, 0, stream, d, R, M, pred, counts,
-                       prefix);
+  // short rows: one entry per lane keeps more lanes busy than 16 bytes per lane;
+  // few rows: one row per wavefront spreads them over more CUs
+  const bool vec = M * (int64_t)sizeof(T) >= 256;
+  const int nr = R >= 8192 ? 4 : 1;
+  const int64_t blocks = (R + kRowsPerBlock * nr - 1) / (kRowsPerBlock * nr);
+  if (blocks > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "row_counts: too many rows");
+  dim3 grid((unsigned)blocks), block(kWave * kRowsPerBlock);
+  if (vec && nr == 4) {
+    hipLaunchKernelGGL((row_counts_kernel<P, kVec, 4>), grid, block, 0, stream, d, R, M, pred, counts, prefix);
+  } else if (vec) {
+    hipLaunchKernelGGL((row_counts_kernel<P, kVec, 1>), grid, block, 0, stream, d, R, M, pred, counts, prefix);
+  } else if (nr == 4) {
+    hipLaunchKernelGGL((row_counts_kernel<P, 1, 4>), grid, block, 0, stream, d, R, M, pred, counts, prefix);
   } else {
-    hipLaunchKernelGGL((row_counts_kernel<P, 1>), grid, block, 0, stream, d, R, M, pred, counts,
-                       prefix);
+    hipLaunchKernelGGL((row_counts_kernel<P, 1, 1>), grid, block, 0, stream, d, R, M, pred, counts, prefix);
   }
   return check_launch("row_counts_kernel");
 }

@@ -16,6 +16,7 @@
 //
 // All index math is int64: the largest configuration holds 1.7e10 elements.
 #include "nt_common.h"
+#include <stdlib.h>
 
 // Tuning knobs of the row kernels (compile-time).
 #ifndef NT_ROW_UNROLL
@@ -168,19 +169,25 @@ __device__ __forceinline__ void move_row(char* d, const char* s, int64_t valid, 
   }
 }
 
-// WAVE_ROWS: rows of at most 1 KiB -- every wavefront of the workgroup takes a row
-// of its own (4 rows per workgroup) instead of 192 lanes idling on one row.
-template <int EB, int MODE, bool WAVE_ROWS>
-__global__ __launch_bounds__(256) void row_kernel(RowParams p) {
-  constexpr int kT = WAVE_ROWS ? 64 : 256;
-  const int64_t row = WAVE_ROWS ? row_index() * 4 + (threadIdx.x >> 6) : row_index();
-  if (row >= p.nrows) return;
+// One row of work, decoded: bytes [0, valid) of d come from s, bytes [valid, total)
+// are padding (kOnes: ones / zeros, s unused).
+struct RowDesc {
+  char* d;
+  const char* s;
+  int64_t valid, total;
+};
+
+// Decode row `row` (scalar arithmetic, uniform over the lanes that share the row).
+// Returns false when the row has nothing to move.
+template <int EB, int MODE>
+__device__ __forceinline__ bool decode_row(const RowParams& p, int64_t row, RowDesc& r) {
   if (MODE == kPack) {
     const int64_t off = p.offsets[row];
     const int64_t n = (p.offsets[row + 1] - off) * EB;
-    move_row<EB, kUnpad, kT>(p.dst + off * EB, reinterpret_cast<const char*>(p.srcs[row]), n, n,
-                             p.pad);
-    return;
+    r.d = p.dst + off * EB;
+    r.s = reinterpret_cast<const char*>(p.srcs[row]);
+    r.valid = r.total = n;
+    return n > 0;
   }
   int64_t b, src_off = 0, last;
   bool inside = true;
@@ -197,9 +204,9 @@ __global__ __launch_bounds__(256) void row_kernel(RowParams p) {
   } else {
     const int64_t plane = p.M0 * p.M1;
     b = row / plane;
-    const int64_t r = row - b * plane;
-    const int64_t i0 = r / p.M1;
-    const int64_t i1 = r - i0 * p.M1;
+    const int64_t rr = row - b * plane;
+    const int64_t i0 = rr / p.M1;
+    const int64_t i1 = rr - i0 * p.M1;
     const int64_t* sz = p.sizes + b * p.D;
     inside = (i0 < sz[0]) && (i1 < sz[1]);
     last = sz[2];
@@ -209,22 +216,397 @@ __global__ __launch_bounds__(256) void row_kernel(RowParams p) {
   const int64_t row_bytes = Mlast * p.inner * EB;
   const int64_t valid = inside ? last * p.inner * EB : 0;
   if (MODE == kOnes) {
-    move_row<EB, kOnes, kT>(p.dst + row * row_bytes, nullptr, valid, row_bytes, p.pad);
-  } else {
-    const int64_t packed_byte = (p.offsets[b] + src_off * p.inner) * EB;
-    if (MODE == kPad || MODE == kPadMask) {
-      move_row<EB, kPad, kT>(p.dst + row * row_bytes, p.src + packed_byte, valid, row_bytes, p.pad);
-      if (MODE == kPadMask) {
-        // the same workgroups write the row's mask bytes: ones over the valid prefix
-        const u32x4 zero = {0u, 0u, 0u, 0u};
-        move_row<1, kOnes, kT>(p.mask + row * (row_bytes / EB), nullptr, valid / EB, row_bytes / EB, zero);
+    r.d = p.dst + row * row_bytes;
+    r.s = nullptr;
+    r.valid = valid;
+    r.total = row_bytes;
+    return true;
+  }
+  const int64_t packed_byte = (p.offsets[b] + src_off * p.inner) * EB;
+  if (MODE == kPad || MODE == kPadMask) {
+    r.d = p.dst + row * row_bytes;
+    r.s = p.src + packed_byte;
+    r.valid = valid;
+    r.total = row_bytes;
+    return true;
+  }
+  r.d = p.dst + packed_byte;      // kUnpad
+  r.s = p.src + row * row_bytes;
+  r.valid = r.total = valid;
+  return valid > 0;
+}
+
+// WAVE_ROWS: rows of at most 1 KiB -- every wavefront of the workgroup takes a row
+// of its own (4 rows per workgroup) instead of 192 lanes idling on one row.
+template <int EB, int MODE, bool WAVE_ROWS>
+__global__ __launch_bounds__(256) void row_kernel(RowParams p) {
+  constexpr int kT = WAVE_ROWS ? 64 : 256;
+  const int64_t row = WAVE_ROWS ? row_index() * 4 + (threadIdx.x >> 6) : row_index();
+  if (row >= p.nrows) return;
+  RowDesc r;
+  if (!decode_row<EB, MODE>(p, row, r)) return;
+  constexpr int kMove = MODE == kPack ? kUnpad : (MODE == kPadMask ? kPad : MODE);
+  move_row<EB, kMove, kT>(r.d, r.s, r.valid, r.total, p.pad);
+  if (MODE == kPadMask) {
+    // the same workgroups write the row's mask bytes: ones over the valid prefix
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    move_row<1, kOnes, kT>(p.mask + (r.d - p.dst) / EB, nullptr, r.valid / EB, r.total / EB, zero);
+  }
+}
+
+// NR short rows (one 16-byte chunk per lane covers a row) moved together by a
+// lane group of kT lanes: the chunks of all of them are in flight at once.
+template <int EB, int MODE, int kT, int NR>
+__device__ __forceinline__ void move_rows(const RowDesc (&r)[NR], const bool (&on)[NR], const RowParams& p,
+                                          const int tid) {
+  constexpr int kMove = MODE == kPadMask ? kPad : MODE;
+  // whole 16-byte chunks of the destination rows: all loads first, then all stores
+  u32x4 v[NR];
+  int state[NR];
+  int64_t pos[NR], head[NR], tail_start[NR];
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    state[i] = 0;
+    if (!on[i]) continue;
+    int64_t h = (int64_t)((0 - (uintptr_t)r[i].d) & 15);
+    if (h > r[i].total) h = r[i].total;
+    const int64_t nvec = (r[i].total - h) >> 4;
+    head[i] = h;
+    tail_start[i] = h + (nvec << 4);
+    pos[i] = h + ((int64_t)tid << 4);
+    if (tid >= nvec) continue;
+    if (pos[i] + 16 <= r[i].valid) {
+      state[i] = 1;
+      if (kMove == kOnes) {
+        v[i] = u32x4{0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};
+      } else {
+        v[i] = load16_unaligned(r[i].s + pos[i]);
       }
+    } else if (pos[i] >= r[i].valid) {
+      state[i] = 1;
+      v[i] = p.pad;
     } else {
-      if (valid > 0) {
-        move_row<EB, kUnpad, kT>(p.dst + packed_byte, p.src + row * row_bytes, valid, valid, p.pad);
+      state[i] = 2;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    if (state[i] == 1) {
+#if NT_ROW_STREAM_STORE
+      store16_stream(r[i].d + pos[i], v[i]);
+#else
+      store16(r[i].d + pos[i], v[i]);
+#endif
+    } else if (state[i] == 2) {
+      // the one chunk that straddles the valid / padding boundary
+#pragma unroll
+      for (int k = 0; k < 16; k += EB) move_elem<EB, kMove>(r[i].d, r[i].s, pos[i] + k, r[i].valid, p.pad);
+    }
+  }
+  // unaligned edges of the destination rows: fewer than 32 bytes each
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    if (!on[i]) continue;
+    const int64_t nedge = (head[i] + (r[i].total - tail_start[i])) / EB;
+    if (tid < nedge) {
+      int64_t e = (int64_t)tid * EB;
+      if (e >= head[i]) e = tail_start[i] + (e - head[i]);
+      move_elem<EB, kMove>(r[i].d, r[i].s, e, r[i].valid, p.pad);
+    }
+  }
+  if (MODE == kPadMask) {
+    // mask bytes of the same rows: ones over the valid prefix.  Rows here are at
+    // most kT chunks of data, so a mask row is at most kT * 16 / EB bytes.
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      if (!on[i]) continue;
+      char* m = p.mask + (r[i].d - p.dst) / EB;
+      const int64_t mv = r[i].valid / EB, mt = r[i].total / EB;
+      int64_t h = (int64_t)((0 - (uintptr_t)m) & 15);
+      if (h > mt) h = mt;
+      const int64_t nvec = (mt - h) >> 4;
+      const int64_t ts = h + (nvec << 4);
+      const int64_t mp = h + ((int64_t)tid << 4);
+      if (tid < nvec) {
+        if (mp + 16 <= mv) {
+          store16_stream(m + mp, u32x4{0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u});
+        } else if (mp >= mv) {
+          store16_stream(m + mp, u32x4{0u, 0u, 0u, 0u});
+        } else {
+#pragma unroll
+          for (int k = 0; k < 16; ++k) m[mp + k] = (mp + k) < mv ? 1 : 0;
+        }
+      }
+      const int64_t nedge = h + (mt - ts);
+      if (tid < nedge) {
+        int64_t e = tid;
+        if (e >= h) e = ts + (e - h);
+        m[e] = e < mv ? 1 : 0;
       }
     }
   }
+}
+
+// Short rows, nrag == 1 (every row is a constituent of its own): a lane group --
+// the workgroup, or one wavefront for rows of at most 1 KiB -- takes NR
+// consecutive rows.  A row of a few KiB per workgroup leaves a CU with too few
+// bytes in flight to cover the latency of the row decode (dependent scalar
+// loads) and of the copy itself.
+template <int EB, int MODE, int kT, int NR>
+__global__ __launch_bounds__(256) void row_batch_kernel(RowParams p) {
+  constexpr int kGroups = 256 / kT;
+  const int tid = threadIdx.x & (kT - 1);
+  const int64_t group = ((int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x) * kGroups + (threadIdx.x / kT);
+  const int64_t row0 = group * NR;
+  if (row0 >= p.nrows) return;
+  // Row decode in three steps so that the size-table and offset loads of all NR
+  // rows are in flight together (one memory round trip, not NR): coordinates of
+  // the first row by division and of the others by increment, then every load,
+  // then the arithmetic on what was loaded.
+  int64_t cb[NR], c0[NR], c1[NR];
+  {
+    int64_t b, i0 = 0, i1 = 0;
+    if (p.nrag == 1) {
+      b = row0;
+    } else if (p.nrag == 2) {
+      b = row0 / p.M0;
+      i0 = row0 - b * p.M0;
+    } else {
+      const int64_t plane = p.M0 * p.M1;
+      b = row0 / plane;
+      const int64_t rr = row0 - b * plane;
+      i0 = rr / p.M1;
+      i1 = rr - i0 * p.M1;
+    }
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      cb[i] = b;
+      c0[i] = i0;
+      c1[i] = i1;
+      if (p.nrag == 1) {
+        ++b;
+      } else if (p.nrag == 2) {
+        if (++i0 == p.M0) { i0 = 0; ++b; }
+      } else {
+        if (++i1 == p.M1) {
+          i1 = 0;
+          if (++i0 == p.M0) { i0 = 0; ++b; }
+        }
+      }
+    }
+  }
+  int64_t sz0[NR], sz1[NR], sz2[NR], off[NR];
+  bool on[NR];
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    on[i] = row0 + i < p.nrows;
+    const int64_t bb = on[i] ? cb[i] : 0;
+    const int64_t* sz = p.sizes + bb * p.D;
+    sz0[i] = sz[0];
+    sz1[i] = p.nrag > 1 ? sz[1] : 0;
+    sz2[i] = p.nrag > 2 ? sz[2] : 0;
+    off[i] = MODE == kOnes ? 0 : p.offsets[bb];
+  }
+  const int64_t Mlast = p.nrag == 1 ? p.M0 : (p.nrag == 2 ? p.M1 : p.M2);
+  const int64_t row_bytes = Mlast * p.inner * EB;
+  RowDesc r[NR];
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    int64_t last, src_off = 0;
+    bool inside = true;
+    if (p.nrag == 1) {
+      last = sz0[i];
+    } else if (p.nrag == 2) {
+      inside = c0[i] < sz0[i];
+      last = sz1[i];
+      src_off = c0[i] * last;
+    } else {
+      inside = (c0[i] < sz0[i]) && (c1[i] < sz1[i]);
+      last = sz2[i];
+      src_off = (c0[i] * sz1[i] + c1[i]) * last;
+    }
+    const int64_t valid = inside ? last * p.inner * EB : 0;
+    const int64_t packed_byte = (off[i] + src_off * p.inner) * EB;
+    const int64_t padded_byte = (row0 + i) * row_bytes;
+    if (MODE == kUnpad) {
+      r[i].d = p.dst + packed_byte;
+      r[i].s = p.src + padded_byte;
+      r[i].valid = r[i].total = valid;
+      on[i] = on[i] && valid > 0;
+    } else {
+      r[i].d = p.dst + padded_byte;
+      r[i].s = MODE == kOnes ? nullptr : p.src + packed_byte;
+      r[i].valid = valid;
+      r[i].total = row_bytes;
+    }
+  }
+  move_rows<EB, MODE, kT, NR>(r, on, p, tid);
+}
+
+// Short rows, nrag >= 2: the rows of one constituent (and, with three ragged dims,
+// of one index of the first) share their entry of the size table and their
+// offset, so a lane group that walks `rows_per_group` consecutive rows decodes
+// once (two divisions, one round trip to the tables) and then only adds strides;
+// the rows are moved two at a time.  With one row per workgroup the decode was
+// most of a workgroup's life: 4.4 TB/s on 16 fp32 images [3, H, W] against
+// 5.9 TB/s this way.
+template <int EB, int MODE, int kT>
+__global__ __launch_bounds__(256) void row_group_kernel(RowParams p, int rows_per_group) {
+  constexpr int kGroups = 256 / kT;
+  const int tid = threadIdx.x & (kT - 1);
+  const int64_t group = ((int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x) * kGroups + (threadIdx.x / kT);
+  const int64_t row0 = group * rows_per_group;
+  if (row0 >= p.nrows) return;
+  const int64_t count = p.nrows - row0 < rows_per_group ? p.nrows - row0 : rows_per_group;
+  // coordinates of the first row: (b, i0) for two ragged dims, (b, i0, i1) for three
+  int64_t b, i0, i1 = 0;
+  if (p.nrag == 2) {
+    b = row0 / p.M0;
+    i0 = row0 - b * p.M0;
+  } else {
+    const int64_t plane = p.M0 * p.M1;
+    b = row0 / plane;
+    const int64_t rr = row0 - b * plane;
+    i0 = rr / p.M1;
+    i1 = rr - i0 * p.M1;
+  }
+  const int64_t Mlast = p.nrag == 2 ? p.M1 : p.M2;
+  const int64_t row_bytes = Mlast * p.inner * EB;
+  int64_t cur_b = -1, sz0 = 0, sz1 = 0, sz2 = 0, off = 0;
+  for (int64_t j = 0; j < count; j += 2) {
+    RowDesc r[2];
+    bool on[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      on[u] = j + u < count;
+      if (on[u] && b != cur_b) {   // uniform; once per constituent
+        const int64_t* sz = p.sizes + b * p.D;
+        sz0 = sz[0];
+        sz1 = sz[1];
+        sz2 = p.nrag > 2 ? sz[2] : 0;
+        off = MODE == kOnes ? 0 : p.offsets[b];
+        cur_b = b;
+      }
+      int64_t last, src_off;
+      bool inside;
+      if (p.nrag == 2) {
+        inside = i0 < sz0;
+        last = sz1;
+        src_off = i0 * last;
+      } else {
+        inside = (i0 < sz0) && (i1 < sz1);
+        last = sz2;
+        src_off = (i0 * sz1 + i1) * last;
+      }
+      const int64_t valid = inside ? last * p.inner * EB : 0;
+      const int64_t packed_byte = (off + src_off * p.inner) * EB;
+      const int64_t padded_byte = (row0 + j + u) * row_bytes;
+      if (MODE == kUnpad) {
+        r[u].d = p.dst + packed_byte;
+        r[u].s = p.src + padded_byte;
+        r[u].valid = r[u].total = valid;
+        on[u] = on[u] && valid > 0;
+      } else {
+        r[u].d = p.dst + padded_byte;
+        r[u].s = MODE == kOnes ? nullptr : p.src + packed_byte;
+        r[u].valid = valid;
+        r[u].total = row_bytes;
+      }
+      // next row
+      if (p.nrag == 2) {
+        if (++i0 == p.M0) { i0 = 0; ++b; }
+      } else if (++i1 == p.M1) {
+        i1 = 0;
+        if (++i0 == p.M0) { i0 = 0; ++b; }
+      }
+    }
+    move_rows<EB, MODE, kT, 2>(r, on, p, tid);
+  }
+}
+
+// Mask of a nested size without any row structure on the store side.  grid.y
+// walks the planes -- one per constituent (two mask dims below the batch dim) or
+// per (constituent, index of the first dim) (three) -- whose entry of the size
+// table every lane of the workgroup shares; the lanes take the 16-byte chunks of
+// the flat mask that overlap the plane, find the row of a chunk's first byte with
+// one 32-bit division and set ones up to each row's length (a chunk may run over
+// several rows).  The chunk that two planes share is written byte-wise by both,
+// each its own bytes.  This runs at the speed of a plain fill; the row-by-row
+// kernels spend more scalar work per row than a 1 KiB store is worth.
+template <int PER>
+__global__ __launch_bounds__(256) void mask_plane_kernel(char* mask, const int64_t* sizes, int64_t D, int K,
+                                                         unsigned M0, unsigned rows, unsigned Mlast) {
+  const int64_t plane = (int64_t)blockIdx.y + (int64_t)blockIdx.z * 65535;
+  int64_t b = plane;
+  bool inside0 = true;
+  if (K == 3) {
+    b = plane / M0;
+    inside0 = (plane - b * M0) < sizes[b * D];
+  }
+  const int64_t* sz = sizes + b * D + (K - 2);
+  const unsigned nrow = inside0 ? (unsigned)min((int64_t)rows, sz[0]) : 0u;   // rows that hold anything
+  const unsigned len = (unsigned)min(sz[1], (int64_t)Mlast);
+  const int64_t plane_bytes = (int64_t)rows * Mlast;
+  const int64_t ps = plane * plane_bytes, pe = ps + plane_bytes;
+  const int64_t g0 = ps >> 4;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int64_t g = g0 + (int64_t)blockIdx.x * (256 * PER) + k * 256 + threadIdx.x;
+    const int64_t byte0 = g << 4;
+    if (byte0 >= pe) break;
+    const int64_t lo = byte0 > ps ? byte0 : ps;
+    const int64_t hi = byte0 + 16 < pe ? byte0 + 16 : pe;
+    const unsigned rel = (unsigned)(lo - ps);
+    unsigned row = rel / Mlast;
+    unsigned col = rel - row * Mlast;
+    unsigned bits = 0;                       // bit j: byte byte0 + j is valid
+    unsigned pos = (unsigned)(lo - byte0);
+    const unsigned end = (unsigned)(hi - byte0);
+    while (pos < end) {
+      const unsigned n = min(end - pos, Mlast - col);
+      if (row < nrow && col < len) {
+        const unsigned v = min(len - col, n);
+        bits |= ((1u << v) - 1u) << pos;
+      }
+      pos += n;
+      ++row;
+      col = 0;
+    }
+    if (end - (unsigned)(lo - byte0) == 16u) {
+      u32x4 v;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const unsigned nib = (bits >> (4 * w)) & 0xfu;
+        v[w] = (nib * 0x00204081u) & 0x01010101u;   // bit i of the nibble -> byte i
+      }
+      __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(mask + byte0));
+    } else {
+      for (unsigned j = (unsigned)(lo - byte0); j < end; ++j) mask[byte0 + j] = (bits >> j) & 1u;
+    }
+  }
+}
+
+// Launches mask_plane_kernel when its conditions hold; *done says whether it did.
+static int try_mask_planes(char* mask, const int64_t* sizes, int64_t B, int64_t D, int64_t K,
+                           const int64_t* ext, hipStream_t stream, bool* done) {
+  *done = false;
+  if (K < 2 || K > 3) return NT_OK;
+  const int64_t Mlast = ext[K - 1], rows = ext[K - 2];
+  const int64_t planes = K == 3 ? B * ext[0] : B;
+  if (Mlast == 0 || rows == 0 || planes == 0 || reinterpret_cast<uintptr_t>(mask) % 16 != 0) return NT_OK;
+  if (Mlast >= ((int64_t)1 << 31) || rows * Mlast >= ((int64_t)1 << 31) || planes > (int64_t)65535 * 65535 ||
+      (K == 3 && ext[0] >= ((int64_t)1 << 31))) {
+    return NT_OK;
+  }
+  if (planes * rows * Mlast < ((int64_t)1 << 20)) return NT_OK;   // tiny masks: the row kernels do
+  constexpr int PER = 4;
+  const int64_t chunks = (rows * Mlast + 15) / 16 + 1;     // a plane may start and end inside a chunk
+  const int64_t gx = (chunks + 256 * PER - 1) / (256 * PER);
+  dim3 grid((unsigned)gx, (unsigned)(planes < 65535 ? planes : 65535), (unsigned)((planes + 65534) / 65535));
+  hipLaunchKernelGGL((mask_plane_kernel<PER>), grid, dim3(256), 0, stream, mask, sizes, D, (int)K,
+                     (unsigned)(K == 3 ? ext[0] : 1), (unsigned)rows, (unsigned)Mlast);
+  *done = true;
+  return check_launch("mask_plane_kernel");
 }
 
 static u32x4 replicate_pad(int eb, uint64_t bits) {
@@ -282,11 +664,52 @@ static int launch_rows_t(int eb, const RowParams& p, int64_t max_row_bytes, hipS
   return check_launch("row_kernel");
 }
 
+#ifndef NT_ROW_GROUP
+#define NT_ROW_GROUP 4           // rows per lane group of row_group_kernel (measured: 2 and 8 are 8-10 % slower)
+#endif
+
+// Short rows: see row_batch_kernel (nrag == 1) and row_group_kernel.
+template <int MODE, int kT>
+static int launch_batch(int eb, const RowParams& p, hipStream_t stream) {
+  static int rpg_env = -1;
+  if (rpg_env < 0) { const char* e = getenv("NT_ROW_GROUP_RT"); rpg_env = e ? atoi(e) : 0; }
+  const int rpg = p.nrag == 1 ? 2 : (rpg_env > 0 ? rpg_env : NT_ROW_GROUP);
+  const int64_t groups = (p.nrows + rpg - 1) / rpg;
+  const int64_t wgs = (groups + (256 / kT) - 1) / (256 / kT);
+  const int64_t gx = wgs < 65535 ? wgs : 65535;
+  const int64_t gy = (wgs + gx - 1) / gx;
+  if (gy > 65535) return fail(NT_ERR_UNSUPPORTED, "row count %lld exceeds the grid limit", (long long)p.nrows);
+  dim3 grid((unsigned)gx, (unsigned)gy, 1), block(256, 1, 1);
+#define NT_BATCH_CASE(EB)                                                                             \
+  if (p.nrag == 1) {                                                                                  \
+    hipLaunchKernelGGL((row_batch_kernel<EB, MODE, kT, 2>), grid, block, 0, stream, p);               \
+  } else {                                                                                            \
+    hipLaunchKernelGGL((row_group_kernel<EB, MODE, kT>), grid, block, 0, stream, p, rpg);             \
+  }                                                                                                   \
+  break;
+  switch (eb) {
+    case 1: NT_BATCH_CASE(1)
+    case 2: NT_BATCH_CASE(2)
+    case 4: NT_BATCH_CASE(4)
+    case 8: NT_BATCH_CASE(8)
+    default: return fail(NT_ERR_INVALID_ARGUMENT, "elem_bytes must be 1, 2, 4 or 8, got %d", eb);
+  }
+#undef NT_BATCH_CASE
+  return check_launch("row_group_kernel");
+}
+
 template <int MODE>
 static int launch_rows(int eb, const RowParams& p, int64_t max_row_bytes, hipStream_t stream) {
   if (p.nrows == 0 || max_row_bytes == 0) return NT_OK;
   if (p.nrows > 0x7fffffffLL) {
     return fail(NT_ERR_UNSUPPORTED, "row count %lld exceeds the grid limit", (long long)p.nrows);
+  }
+  static int use_batch = -1;
+  if (use_batch < 0) { const char* e = getenv("NT_ROW_BATCH_RT"); use_batch = (e && atoi(e) == 1) ? 0 : 1; }
+  if (MODE != kPack && p.nrows >= 4096 && use_batch) {
+    // many short rows: several rows per lane group, all of their chunks in flight
+    if (max_row_bytes <= 1024) return launch_batch<MODE, 64>(eb, p, stream);
+    if (max_row_bytes <= 4096) return launch_batch<MODE, 256>(eb, p, stream);
   }
   if (max_row_bytes <= 1024 && MODE != kPack) return launch_rows_t<MODE, true>(eb, p, max_row_bytes, stream);
   return launch_rows_t<MODE, false>(eb, p, max_row_bytes, stream);
@@ -356,6 +779,15 @@ extern "C" int nt_add_padding_mask(const void* packed, void* padded, uint8_t* ma
   p.offsets = offsets;
   p.sizes = sizes;
   p.pad = replicate_pad(elem_bytes, pad_bits);
+  {
+    // mask[b, i...] = all_k(i_k < sizes[b, k]) over every dim of the size table:
+    // written at fill speed by a launch of its own where that kernel applies,
+    // which beats carrying the mask along in the data kernel
+    bool done = false;
+    rc = try_mask_planes(p.mask, sizes, B, D, D, padded_sizes_host, (hipStream_t)stream, &done);
+    if (rc != NT_OK) return rc;
+    if (done) return launch_rows<kPad>(elem_bytes, p, max_row_elems * elem_bytes, (hipStream_t)stream);
+  }
   return launch_rows<kPadMask>(elem_bytes, p, max_row_elems * elem_bytes, (hipStream_t)stream);
 }
 
@@ -387,6 +819,9 @@ extern "C" int nt_build_mask(uint8_t* mask, const int64_t* sizes, int64_t B, int
   if (rc != NT_OK) return rc;
   if (B == 0 || max_row_elems == 0) return NT_OK;
   if (!mask || !sizes) return fail(NT_ERR_INVALID_ARGUMENT, "NULL pointer");
+  bool done = false;
+  rc = try_mask_planes(reinterpret_cast<char*>(mask), sizes, B, D, K, mask_sizes_host, (hipStream_t)stream, &done);
+  if (rc != NT_OK || done) return rc;
   p.dst = reinterpret_cast<char*>(mask);
   p.sizes = sizes;
   p.pad = replicate_pad(1, 0);

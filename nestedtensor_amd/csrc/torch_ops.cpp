@@ -209,6 +209,68 @@ Tensor build_mask(const Tensor& sizes_dev, at::IntArrayRef ext) {
   return mask;
 }
 
+// ---- list of device tensors -> packed -------------------------------------------
+
+// impl::pack (Packed.h:75-98) with the checks of _verify_variables
+// (creation.cpp:28-171) for constituents that already live on the device: one
+// gather launch (nt_pack) instead of B copy_ calls.  The nested size, the element
+// offsets computed from it and the table of source pointers reach the device in
+// one copy from pinned memory.  Returns (buffer, sizes, sizes_dev, offsets_dev).
+std::tuple<Tensor, Tensor, Tensor, Tensor> pack_device(at::TensorList tensors) {
+  static const char* hint =
+      "To form a valid NestedTensor all Tensor / NestedTensor constiuents of the given list must be "
+      "of the same dimension, layout, device, scalar type and either all or none require gradients.";
+  TORCH_CHECK(!tensors.empty(), "pack_device: empty list");
+  const Tensor& first = tensors[0];
+  require_device(first, "nested_tensor (device constituents)");
+  const int64_t B = static_cast<int64_t>(tensors.size()), D = first.dim();
+  for (const Tensor& t : tensors) {
+    TORCH_CHECK(t.dim() == first.dim(), "Given Tensor / NestedTensor constiuent of dimension ", t.dim(),
+                " doesn't match another constiuent of dimension ", first.dim(), ". ", hint);
+    TORCH_CHECK(t.layout() == first.layout(), "Given Tensor / NestedTensor constiuent of layout ", t.layout(),
+                " doesn't match another constiuent of layout ", first.layout(), ". ", hint);
+    TORCH_CHECK(t.device() == first.device(), "Given Tensor / NestedTensor constiuent of device ", t.device(),
+                " doesn't match another constiuent of device ", first.device(), ". ");
+    TORCH_CHECK(t.scalar_type() == first.scalar_type(), "Given Tensor / NestedTensor constiuent of scalar type ",
+                t.scalar_type(), " doesn't match another constiuent of scalar type ", first.scalar_type(), ". ");
+    TORCH_CHECK(t.requires_grad() == first.requires_grad(),
+                "Given Tensor / NestedTensor constiuent requires gradient in contrast to another constiuent. ", hint);
+  }
+  const int eb = elem_bytes(first.scalar_type());
+  c10::hip::HIPGuard guard(first.device().index());
+  std::vector<Tensor> keep;
+  keep.reserve(B);
+  for (const Tensor& t : tensors) keep.push_back(t.contiguous());
+  Tensor sizes = at::empty({B, D}, at::kLong);
+  int64_t* sp = sizes.data_ptr<int64_t>();
+  const int64_t n = B * D + (B + 1) + B;
+  Tensor host = at::empty({n}, at::TensorOptions().dtype(at::kLong).pinned_memory(true));
+  int64_t* h = host.data_ptr<int64_t>();
+  int64_t* off = h + B * D;
+  int64_t* ptrs = off + B + 1;
+  int64_t acc = 0;
+  for (int64_t b = 0; b < B; ++b) {
+    const at::IntArrayRef shape = keep[b].sizes();
+    for (int64_t k = 0; k < D; ++k) sp[b * D + k] = h[b * D + k] = shape[k];
+    off[b] = acc;
+    acc += keep[b].numel();
+    ptrs[b] = reinterpret_cast<int64_t>(keep[b].const_data_ptr());
+  }
+  off[B] = acc;
+  Tensor meta = at::empty({n}, first.options().dtype(at::kLong));
+  meta.copy_(host, /*non_blocking=*/true);
+  Tensor sizes_dev = meta.narrow(0, 0, B * D).view({B, D});
+  Tensor offsets_dev = meta.narrow(0, B * D, B + 1);
+  Tensor buffer = at::empty({acc}, first.options());
+  if (acc > 0) {
+    check(nt_pack(reinterpret_cast<const void* const*>(meta.const_data_ptr<int64_t>() + B * D + B + 1),
+                  buffer.data_ptr(), offsets_dev.const_data_ptr<int64_t>(), B, eb, stream_of(first)));
+  }
+  // `keep` may hold temporaries; torch's caching allocator reuses their blocks
+  // only for later work on this same stream
+  return std::make_tuple(buffer, sizes, sizes_dev, offsets_dev);
+}
+
 // ---- dense + mask -> nested ----------------------------------------------------
 
 // Result of a dense -> nested conversion in lowered form.  sizes is a host int64
@@ -268,21 +330,33 @@ Tensor& pinned_staging(int64_t bytes) {
   return buf;
 }
 
-// Device keep-counts (int32) and is-a-prefix flags (uint8) of R rows in ONE
-// device buffer [4 R bytes of counts | R bytes of flags], so that both reach the
-// host in one copy.
-struct RowStats {
-  Tensor raw;           // device, uint8 [5 R]
-  int32_t* counts_dev;
-  uint8_t* prefix_dev;
-};
-
-RowStats alloc_row_stats(const Tensor& like, int64_t R) {
-  RowStats s;
-  s.raw = at::empty({5 * R + 16}, like.options().dtype(at::kByte));
-  s.counts_dev = reinterpret_cast<int32_t*>(s.raw.data_ptr());
-  s.prefix_dev = static_cast<uint8_t*>(s.raw.data_ptr()) + 4 * R;
-  return s;
+// Wait until everything enqueued on `stream` so far has completed and its writes
+// to pinned host memory are visible.  The stream itself writes a sequence number
+// into a pinned word when it gets there (hipStreamWriteValue32) and the host
+// polls that word: a few microseconds sooner than hipStreamSynchronize wakes up,
+// which is most of what a small conversion costs.  Falls back to the blocking
+// wait if the stream operation is not available or takes long.
+void wait_for_stream(hipStream_t stream) {
+  static thread_local Tensor flag_t;
+  static thread_local uint32_t seq = 0;
+  static thread_local bool usable = true;
+  if (usable) {
+    if (!flag_t.defined()) {
+      flag_t = at::zeros({16}, at::TensorOptions().dtype(at::kInt).pinned_memory(true));
+    }
+    volatile uint32_t* flag = reinterpret_cast<volatile uint32_t*>(flag_t.data_ptr());
+    const uint32_t want = ++seq;
+    if (hipStreamWriteValue32(stream, const_cast<uint32_t*>(flag), want, 0) == hipSuccess) {
+      for (int spin = 0; spin < (1 << 22); ++spin) {
+        if (*flag == want) return;
+        __builtin_ia32_pause();
+      }
+    } else {
+      (void)hipGetLastError();
+      usable = false;
+    }
+  }
+  C10_HIP_CHECK(hipStreamSynchronize(stream));
 }
 
 // Scan the per-row keep-counts and move the kept chunks (nt_exclusive_scan_i32,
@@ -305,11 +379,13 @@ Tensor compact(const Tensor& data, const Tensor& bmask, int64_t R, int64_t M, in
 }
 
 // Upload sizes[B, D] and the element offsets computed from them in one copy.
+// The host side of the copy comes from torch's pinned-memory allocator, which
+// keeps the block until the asynchronous copy has left it: no wait here.
 void upload_meta(const Tensor& sizes, const Tensor& like, Tensor* sizes_dev, Tensor* offsets_dev, int64_t* total) {
   const int64_t B = sizes.size(0), D = sizes.size(1);
   const int64_t n = B * D + B + 1;
-  Tensor& stage = pinned_staging(n * 8);
-  int64_t* h = reinterpret_cast<int64_t*>(stage.data_ptr());
+  Tensor host = at::empty({n}, at::TensorOptions().dtype(at::kLong).pinned_memory(true));
+  int64_t* h = host.data_ptr<int64_t>();
   const int64_t* s = sizes.const_data_ptr<int64_t>();
   std::memcpy(h, s, static_cast<size_t>(B * D) * 8);
   int64_t* off = h + B * D;
@@ -323,11 +399,7 @@ void upload_meta(const Tensor& sizes, const Tensor& like, Tensor* sizes_dev, Ten
   off[B] = acc;
   *total = acc;
   Tensor meta = at::empty({n}, like.options().dtype(at::kLong));
-  hipStream_t stream = c10::hip::getCurrentHIPStream(like.device().index()).stream();
-  C10_HIP_CHECK(hipMemcpyAsync(meta.data_ptr(), h, static_cast<size_t>(n) * 8, hipMemcpyHostToDevice, stream));
-  // the staging buffer is reused by the next conversion of this thread: the copy
-  // must have left it
-  C10_HIP_CHECK(hipStreamSynchronize(stream));
+  meta.copy_(host, /*non_blocking=*/true);
   *sizes_dev = meta.narrow(0, 0, B * D).view({B, D});
   *offsets_dev = meta.narrow(0, B * D, B + 1);
 }
@@ -353,53 +425,58 @@ Lowered from_rows(const Tensor& tensor, int64_t mask_dims, CountRows count_rows,
   TORCH_CHECK(R <= (int64_t(1) << 26), "nested_tensor_from_tensor_mask: ", R,
               " mask rows exceed what this conversion stages on the host (67 108 864)");
   c10::hip::HIPGuard guard(tensor.device().index());
-  RowStats st = alloc_row_stats(tensor, R);
-  count_rows(R, M, st.counts_dev, st.prefix_dev);
-  // one device-to-host copy: the row counts and the "row keeps a prefix" flags
+  // The keep-counts (int32) and the "row keeps a prefix" flags (uint8) of the R
+  // rows are the one thing the host needs from the device: the kernel writes
+  // them straight into pinned host memory (which the device addresses), and the
+  // host waits for the stream.
   Tensor& stage = pinned_staging(5 * R + 16);
+  int32_t* counts = reinterpret_cast<int32_t*>(stage.data_ptr());
+  uint8_t* prefix = static_cast<uint8_t*>(stage.data_ptr()) + 4 * R;
   hipStream_t stream = c10::hip::getCurrentHIPStream(tensor.device().index()).stream();
   if (R > 0) {
-    C10_HIP_CHECK(hipMemcpyAsync(stage.data_ptr(), st.raw.const_data_ptr(), static_cast<size_t>(5 * R),
-                                 hipMemcpyDeviceToHost, stream));
-    C10_HIP_CHECK(hipStreamSynchronize(stream));
+    count_rows(R, M, counts, prefix);
+    wait_for_stream(stream);
   }
-  const int32_t* counts = reinterpret_cast<const int32_t*>(stage.data_ptr());
-  const uint8_t* prefix = static_cast<const uint8_t*>(stage.data_ptr()) + 4 * R;
 
   // Nested size from the counts: at every mask level the extent is the number of
   // children that keep anything (masking.cpp:203-222); the selection must be
   // rectangular or at::stack would have thrown.  `leading`: the kept children
   // come first at every level.
   bool leading = true;
-  for (int64_t r = 0; r < R; ++r) leading = leading && prefix[r] != 0;
   std::vector<int64_t> total(B, 0);
   std::vector<std::vector<int64_t>> extents(B, std::vector<int64_t>(levels, 0));   // outermost first
-  std::vector<uint8_t> alive, next;
+  std::vector<uint8_t> alive(rows_per > 0 ? rows_per : 1), next(rows_per > 0 ? rows_per : 1);
   for (int64_t b = 0; b < B; ++b) {
     const int32_t* c = counts + b * rows_per;
-    int64_t sum = 0, mx = 0;
+    const uint8_t* pf = prefix + b * rows_per;
+    int64_t sum = 0;
+    int32_t mx = 0;
+    uint8_t all_prefix = 1;
     for (int64_t r = 0; r < rows_per; ++r) {
-      sum += c[r];
-      if (c[r] > mx) mx = c[r];
+      const int32_t v = c[r];
+      sum += v;
+      mx = v > mx ? v : mx;
+      all_prefix &= pf[r];
+      alive[r] = v > 0;
     }
+    leading = leading && all_prefix != 0;
     total[b] = sum;
     extents[b][levels - 1] = mx;
     // walk the mask levels upwards: alive[i] = child i keeps anything
-    alive.assign(rows_per, 0);
-    for (int64_t r = 0; r < rows_per; ++r) alive[r] = c[r] > 0;
     int64_t n = rows_per;
     for (int64_t lev = levels - 2; lev >= 0; --lev) {
       const int64_t width = shape[lev + 1];      // children per parent at this level
-      const int64_t parents = n / width;
-      next.assign(parents, 0);
+      const int64_t parents = width > 0 ? n / width : 0;
       int64_t mxc = 0;
       for (int64_t p = 0; p < parents; ++p) {
-        int64_t cnt = 0;
-        for (int64_t i = 0; i < width; ++i) {
-          const uint8_t a = alive[p * width + i];
-          if (i > 0 && a > alive[p * width + i - 1]) leading = false;
-          cnt += a;
+        const uint8_t* a = alive.data() + p * width;
+        int64_t cnt = a[0];
+        uint8_t rises = 0;
+        for (int64_t i = 1; i < width; ++i) {
+          rises |= static_cast<uint8_t>(a[i] > a[i - 1]);
+          cnt += a[i];
         }
+        if (rises) leading = false;
         next[p] = cnt > 0;
         if (cnt > mxc) mxc = cnt;
       }
@@ -447,7 +524,12 @@ Lowered from_rows(const Tensor& tensor, int64_t mask_dims, CountRows count_rows,
     Tensor out = remove_padding(tensor, sizes_dev, offsets_dev, numel, n_ragged);
     return {out, sizes, sizes_dev, offsets_dev};
   }
-  Tensor buf = compact(tensor, byte_mask(), R, M, chunk, kept_total, st.counts_dev);
+  // rare: the selection is a box that does not start at the origin of every
+  // constituent.  The compaction scans the counts on the device.
+  Tensor counts_dev = at::empty({R}, tensor.options().dtype(at::kInt));
+  C10_HIP_CHECK(hipMemcpyAsync(counts_dev.data_ptr(), counts, static_cast<size_t>(R) * 4, hipMemcpyHostToDevice, stream));
+  C10_HIP_CHECK(hipStreamSynchronize(stream));   // the staging buffer is reused by the next conversion
+  Tensor buf = compact(tensor, byte_mask(), R, M, chunk, kept_total, counts_dev.const_data_ptr<int32_t>());
   return {buf, sizes, Tensor(), Tensor()};
 }
 
@@ -481,10 +563,10 @@ Lowered from_mask(const Tensor& tensor_in, const Tensor& mask_in, int64_t nested
     const bool* keep = keep_host.const_data_ptr<bool>();
     int64_t kept = 0;
     for (int64_t b = 0; b < B; ++b) kept += keep[b];
-    RowStats st = alloc_row_stats(tensor, 1);
-    check(nt_mask_row_counts(static_cast<const uint8_t*>(bmask.const_data_ptr()), 1, B, st.counts_dev,
-                             st.prefix_dev, stream_of(tensor)));
-    Tensor buf = compact(tensor, bmask, 1, B, row_elems, kept, st.counts_dev);
+    Tensor stats = at::empty({8}, tensor.options().dtype(at::kInt));
+    check(nt_mask_row_counts(static_cast<const uint8_t*>(bmask.const_data_ptr()), 1, B, stats.data_ptr<int32_t>(),
+                             reinterpret_cast<uint8_t*>(stats.data_ptr<int32_t>() + 4), stream_of(tensor)));
+    Tensor buf = compact(tensor, bmask, 1, B, row_elems, kept, stats.const_data_ptr<int32_t>());
     std::vector<int64_t> full(tensor.sizes().begin() + 1, tensor.sizes().end());
     if (mask.dim() == 1) {
       if (kept == 0) return empty_nt();
@@ -689,6 +771,7 @@ TORCH_LIBRARY(nestedtensor, m) {
   m.def("nt_from_padded_tensor(Tensor tensor, float padding, int nested_dim) -> (Tensor, Tensor)");
 
   m.def("offsets_from_sizes(Tensor sizes) -> Tensor");
+  m.def("pack_device(Tensor[] tensors) -> (Tensor, Tensor, Tensor, Tensor)");
   m.def("add_padding(Tensor buffer, Tensor sizes, Tensor offsets, int[] padded_sizes, int n_ragged, "
         "float padding) -> Tensor");
   m.def("add_padding_mask(Tensor buffer, Tensor sizes, Tensor offsets, int[] padded_sizes, int n_ragged, "
@@ -705,6 +788,7 @@ TORCH_LIBRARY(nestedtensor, m) {
 // "CUDA" is the dispatch key of the HIP device on PyTorch-ROCm.
 TORCH_LIBRARY_IMPL(nestedtensor, CUDA, m) {
   m.impl("offsets_from_sizes", offsets_from_sizes);
+  m.impl("pack_device", pack_device);
   m.impl("add_padding", add_padding);
   m.impl("add_padding_mask", add_padding_mask);
   m.impl("remove_padding", remove_padding);

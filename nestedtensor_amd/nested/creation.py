@@ -4,8 +4,11 @@ nested_tensor_impl they call, nestedtensor/csrc/creation.cpp:28-222)."""
 import torch
 
 from .. import ops
-from ..impl import NestedTensorImpl, device_offsets
+from .. import _C
+from ..impl import NestedTensorImpl
 from . import nested
+
+_pack_device = _C.ops.pack_device.default
 
 _HINT = (
     "To form a valid NestedTensor all Tensor / NestedTensor constiuents of the given list must be "
@@ -70,21 +73,19 @@ def nested_tensor_impl(data, dtype, device, requires_grad, pin_memory, channels_
         # Packed.h:77-79: at::ones({0}); EfficientSizeNode.h:10-12: 0-d sizes
         buffer = torch.ones(0).to(device, dtype)
         return NestedTensorImpl(buffer, torch.zeros((), dtype=torch.int64))
-    _verify_variables(tensors)
-    sizes = torch.tensor([list(t.shape) for t in tensors], dtype=torch.int64).reshape(
-        len(tensors), tensors[0].dim())
     src_device = tensors[0].device
     if src_device.type == "cuda":
-        # constituents already in HBM: one gather launch into the packed buffer
-        sizes_dev = sizes.to(src_device)
-        offsets = device_offsets(sizes_dev, sizes.size(0), sizes.size(1))
-        total = int(sizes.prod(1).sum())
-        buffer = ops.pack_device(tensors, offsets, total, tensors[0].dtype, src_device)
+        # constituents already in HBM: checked, sized and gathered into the packed
+        # buffer by one operator of the extension (one launch, one metadata upload)
+        buffer, sizes, sizes_dev, offsets = _pack_device(tensors)
         impl = NestedTensorImpl(buffer, sizes)
         impl._sizes_dev, impl._offsets_dev = sizes_dev, offsets
         if buffer.dtype != dtype or buffer.device != device:
             impl = impl.with_buffer(buffer.to(device, dtype))
         return impl
+    _verify_variables(tensors)
+    sizes = torch.tensor([list(t.shape) for t in tensors], dtype=torch.int64).reshape(
+        len(tensors), tensors[0].dim())
     total = int(sizes.prod(1).sum())
     if (device.type == "cuda" and src_device.type == "cpu"
             and total * tensors[0].element_size() >= len(tensors) * _DIRECT_COPY_BYTES):

@@ -158,9 +158,9 @@ class NestedTensor:
 
     def is_contiguous(self, memory_format=torch.contiguous_format):
         if memory_format == torch.contiguous_format:
-            return torch.ops.nestedtensor.get_is_contiguous(self, 0)
+            return ops.is_contiguous(self._impl, 0)
         if memory_format == torch.channels_last:
-            return torch.ops.nestedtensor.get_is_contiguous(self, 2)
+            return ops.is_contiguous(self._impl, 2)
         raise RuntimeError("Given memory format " + str(memory_format) + " not supported.")
 
     def nested_size(self, dim=None):
@@ -310,11 +310,12 @@ class NestedTensor:
         constituent and a bool mask that is True where an element stores data.
         If mask_dim is not passed the mask has the smallest dimensionality that
         can represent the data; a mask_dim lower than that is an error."""
-        return torch.ops.nestedtensor.to_tensor_mask(self, mask_dim)
+        # the handler torch.ops.nestedtensor.to_tensor_mask(self, mask_dim) is routed to
+        return ops.to_tensor_mask(ops.contiguous(self._impl), mask_dim)
 
     def to_padded_tensor(self, padding=-1):
-        padding = float(padding)
-        return torch.ops.nestedtensor.to_padded_tensor(self, padding)
+        # the handler torch.ops.nestedtensor.to_padded_tensor(self, padding) is routed to
+        return ops.to_padded_tensor(ops.contiguous(self._impl), float(padding))
 
     def to_packed_sequence(self):
         if not self.dim() == 3 and self.nested_dim() == 1:

@@ -228,7 +228,7 @@ def to_mask(impl, mask_dim=None):
     if impl.dim() > 1 and mask_dim is not None and mask_dim > 1:
         # masking.cpp:428-453: the first mask_dim - 1 constituent dims, no merge
         K = mask_dim - 1
-        if bool((impl.sizes[:, :K] == 0).any()):
+        if impl.has_empty_constituent() and bool((impl.sizes[:, :K] == 0).any()):
             raise RuntimeError("Empty tensors are not yet supported.")
         return build_mask(impl, mask_dim)
     if impl.D == 0:
@@ -274,25 +274,6 @@ def from_padded_tensor(padded, target):
         target = target.with_buffer(torch.empty(0, dtype=padded.dtype, device=padded.device))
     out = _remove_padding(padded, target.sizes_dev(), target.offsets_dev(), total, nrag)
     return target.with_buffer(out)
-
-
-# ---------------------------------------------------------------------------
-# list of tensors -> packed
-
-
-def pack_device(tensors, offsets_dev, total, dtype, device):
-    """impl::pack (Packed.h:75-98) for constituents that already live on the
-    device: one gather launch (nt_pack) instead of B copy_ calls."""
-    keep = [t.contiguous() for t in tensors]
-    out = torch.empty(total, dtype=dtype, device=device)
-    ptrs = torch.tensor([t.data_ptr() for t in keep], dtype=torch.int64).to(device)
-    with _C.on_device(device):
-        _C.check(_C.lib.nt_pack(
-            _C.ptr(ptrs), _C.ptr(out), _C.ptr(offsets_dev), len(keep),
-            _elem_bytes(dtype), _C.current_stream(device)))
-    # `keep` must outlive the launch on this stream; torch's caching allocator
-    # only reuses the blocks for later work on the same stream.
-    return out
 
 
 # ---------------------------------------------------------------------------
