@@ -21,9 +21,19 @@ The same JSON line carries
   rows         - the remaining rows of the path (to_tensor_mask, to_mask,
                  nested_tensor_from_tensor_mask / _from_padded_tensor, pack, the
                  offsets scan, C4 attention) on configurations C1, C2 and C4.
+
+Every row is the median over timed batches of calls, with the slowest batch
+and the mean beside it.  All device legs run first; what the CPU oracle times
+runs after the last of them.  Two more modes issue dispatches for profiler runs
+and print only the sizes the counters are to be set against:
+  --pmc-probe  a plain copy of known size, then one pad and one un-pad launch;
+  --mha-probe  the kernels of the C3 and C4 attention layers and the vendor GEMM
+               on C3's projection shapes.
 """
 
 import argparse
+import contextlib
+import gc
 import json
 import os
 import sys
@@ -40,8 +50,26 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, GB/s
 # unit, WRITE_SIZE: 1.0 KiB per unit).
 PAD_TRAFFIC_RATIO = 1.0001
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, TFLOP/s
+MFMA_F32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, TFLOP/s
 
 METRIC = "ragged->padded HBM GB/s + nested BERT MHA tokens/s (B=32, L<=512, d=768)"
+
+
+@contextlib.contextmanager
+def _no_gc():
+    """Timed regions run with Python's cyclic collector off (and collected just
+    before).  A full collection walks every tracked object of the interpreter,
+    about 40 ms with torch imported, and starts whenever the allocation counters
+    say so: inside a loop of 20-microsecond calls it is a stall of two thousand
+    calls' worth that has nothing to do with the call being timed."""
+    was = gc.isenabled()
+    gc.collect()
+    gc.disable()
+    try:
+        yield
+    finally:
+        if was:
+            gc.enable()
 
 
 def parse():
@@ -60,6 +88,10 @@ def parse():
     ap.add_argument("--pmc-probe", action="store_true",
                     help="one plain copy of known size, then one pad and one un-pad launch of the "
                          "first C5 chunk; meant to run under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
+    ap.add_argument("--mha-probe", action="store_true",
+                    help="the kernels of the C3 fp16 and C4 bf16 attention layers, each layer issued twice "
+                         "(the second pass with warm caches), then the vendor GEMM (torch.addmm) on the two "
+                         "C3 projection shapes; meant to run under rocprofv3 --kernel-trace or --pmc")
     return ap.parse_args()
 
 
@@ -136,20 +168,21 @@ def bench_c5(args, torch, dev):
     step_start = torch.cuda.Event(enable_timing=True)
     step_end = torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    step_start.record()
-    i = 0
-    for s in range(args.steps):
-        for m in meta:
-            e = ev[i]
-            e[0].record()
-            pad(m)
-            e[1].record()
-            unpad(m)
-            e[2].record()
-            i += 1
-    step_end.record()
-    torch.cuda.synchronize()
+    with _no_gc():
+        t0 = time.perf_counter()
+        step_start.record()
+        i = 0
+        for s in range(args.steps):
+            for m in meta:
+                e = ev[i]
+                e[0].record()
+                pad(m)
+                e[1].record()
+                unpad(m)
+                e[2].record()
+                i += 1
+        step_end.record()
+        torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     total_ms = step_start.elapsed_time(step_end)
     ms_per_step = total_ms / args.steps
@@ -211,11 +244,48 @@ def pmc_probe(args, torch, dev):
                       "unpad_valid_bytes": m.numel() * eb}))
 
 
-def cpu_baseline_c5(torch, n_sample=96):
+def mha_probe(args, torch, dev):
+    """Dispatches for kernel-trace and hardware-counter runs of the attention
+    layers: min_mha on C3 (fp16) twice, bt_min_mha on C4 (bf16) twice, and
+    torch.addmm (the vendor GEMM) on C3's two projection shapes twice.  Prints
+    the shapes and flop counts the counters are to be set against."""
+    import nestedtensor_amd as nt
+    out = {}
+    for tag, seed, B, E, H, dtype in (("C3", 1010 + 2, 32, 768, 12, torch.float16),
+                                      ("C4", 1010 + 3, 128, 1024, 16, torch.bfloat16)):
+        g = torch.Generator().manual_seed(seed)
+        if tag == "C3":
+            lens = [int(v) for v in torch.randint(32, 513, (B,), generator=g)]
+        else:
+            lens = [int(v) for v in torch.empty(B).exponential_(1.0 / 96.0, generator=g).round().clamp(8, 512)]
+        xs = [torch.randn(L, E, generator=g).to(dtype) for L in lens]
+        W_in = (torch.randn(3 * E, E, generator=g) * 0.02).to(dtype).to(dev)
+        W_out = (torch.randn(E, E, generator=g) * 0.02).to(dtype).to(dev)
+        b_in, b_out = torch.zeros(3 * E, dtype=dtype, device=dev), torch.zeros(E, dtype=dtype, device=dev)
+        a = nt.nested_tensor(xs, device=dev, dtype=dtype)
+        op = torch.ops.nestedtensor.min_mha if tag == "C3" else torch.ops.nestedtensor.bt_min_mha
+        torch.cuda.synchronize()
+        for _ in range(2):
+            op(H, 64, 0.0, False, a, a, a, W_in, b_in, 64 ** -0.5, W_out, b_out)
+        torch.cuda.synchronize()
+        T = sum(lens)
+        out[tag] = dict(tokens=T, embed=E, heads=H, sum_L2=sum(L * L for L in lens),
+                        flops_in_proj=2 * T * E * 3 * E, flops_out_proj=2 * T * E * E,
+                        flops_attention=4 * E * sum(L * L for L in lens))
+        if tag == "C3":
+            x = a._impl.buffer.reshape(T, E)
+            for _ in range(2):
+                torch.addmm(b_in, x, W_in.t())
+                torch.addmm(b_out, x, W_out.t())
+            torch.cuda.synchronize()
+    print(json.dumps(out))
+
+
+def cpu_baseline_c5(torch, n_sample=128):
     """The oracle's to_padded_tensor + from_padded_tensor on the first n_sample
     constituents of C5 (same seeded lengths), timed on the host cores."""
     import oracle
-    torch.set_num_threads(os.cpu_count() or 1)
+    torch.set_num_threads(_host_threads())
     g = torch.Generator().manual_seed(1010 + 4)
     lengths = torch.randint(1, 2049, (4096,), generator=g)[:n_sample]
     E = 4096
@@ -244,7 +314,7 @@ def cpu_baseline_c5(torch, n_sample=96):
                 host_cpus=os.cpu_count())
 
 
-def bench_mha_c3(args, torch, dev):
+def bench_mha_c3(args, torch, dev, later):
     import nestedtensor_amd as nt
     import oracle
     g = torch.Generator().manual_seed(1010 + 2)
@@ -261,17 +331,10 @@ def bench_mha_c3(args, torch, dev):
         return torch.ops.nestedtensor.min_mha(H, hd, 0.0, False, a, a, a, dW_in, db_in, hd ** -0.5,
                                               dW_out, db_out)
 
-    for _ in range(5):
-        out = layer()
-    torch.cuda.synchronize()
+    out = layer()
+    ms = _time_gpu(torch, layer, iters=50, warmup=5)
     iters = 50
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(iters):
-        out = layer()
-    e1.record()
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / iters
     # the same three launches replayed from a HIP graph (no host work between them)
     graph_ms = None
     try:
@@ -286,11 +349,12 @@ def bench_mha_c3(args, torch, dev):
         for _ in range(5):
             graph.replay()
         torch.cuda.synchronize()
-        e0.record()
-        for _ in range(iters):
-            graph.replay()
-        e1.record()
-        torch.cuda.synchronize()
+        with _no_gc():
+            e0.record()
+            for _ in range(iters):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
         graph_ms = e0.elapsed_time(e1) / iters
         assert torch.equal(gout._impl.buffer, out._impl.buffer)
     except Exception as exc:      # report, do not hide
@@ -315,43 +379,74 @@ def bench_mha_c3(args, torch, dev):
     ms_enc = None if args.no_encoder else _time_gpu(torch, encoder_layer, iters=50, warmup=5)
     flops_enc = flops + 16 * T * E * E
     res = dict(workload="C3: nested BERT-base self-attention, fp16, B=32, L~U[32,512], d=768, 12x64",
-               tokens=T, ms_per_layer=ms, ms_per_layer_hip_graph=graph_ms, tokens_per_s=T / (ms * 1e-3), flops=flops,
+               tokens=T, ms_per_layer=float(ms), ms_per_layer_max=ms.max, ms_per_layer_mean=ms.mean,
+               timing=ms.fields()["timing"], ms_per_layer_hip_graph=graph_ms,
+               tokens_per_s=T / (ms * 1e-3), flops=flops,
                roofline=dict(bound="mfma", achieved=flops / (ms * 1e-3) / 1e12, peak=MFMA_F16_PEAK_TFLOPS,
                              unit="TFLOP/s", frac=flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS))
     if ms_enc is not None:
         res["encoder_layer"] = dict(
             workload="the same batch through a whole BERT-base encoder layer (attention, add + layer norm, "
                      "768-3072-768 feed-forward with gelu, add + layer norm), 7 launches",
-            ms_per_layer=ms_enc, tokens_per_s=T / (ms_enc * 1e-3), flops=flops_enc,
-            TFLOPs=flops_enc / (ms_enc * 1e-3) / 1e12,
+            ms_per_layer=float(ms_enc), ms_per_layer_max=ms_enc.max, tokens_per_s=T / (ms_enc * 1e-3),
+            flops=flops_enc, TFLOPs=flops_enc / (ms_enc * 1e-3) / 1e12,
             frac_of_mfma_peak=flops_enc / (ms_enc * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS)
     if not args.no_cpu:
-        torch.set_num_threads(os.cpu_count() or 1)
-        ref = oracle.ref_nested_tensor(xs, dtype=torch.float16)
-        best = None
-        for it in range(2):
-            t0 = time.perf_counter()
-            exp = oracle.min_mha(H, hd, 0.0, False, ref, ref, ref, W_in, b_in, hd ** -0.5, W_out, b_out)
-            dt = time.perf_counter() - t0
-            best = dt if best is None else min(best, dt)
-        err = (out._impl.buffer.float().cpu() - torch.cat([p.reshape(-1) for p in exp]).float()).abs().max()
-        res["max_abs_err_vs_oracle"] = float(err)
-        res["cpu_baseline"] = dict(value=T / best, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
-                                   sample="full C3 layer, oracle min_mha in fp16 on the host, best of 2")
+        got = out._impl.buffer.float().cpu()
+
+        def _cpu_layer():
+            ref = oracle.ref_nested_tensor(xs, dtype=torch.float16)
+            best = None
+            for it in range(2):
+                t0 = time.perf_counter()
+                exp = oracle.min_mha(H, hd, 0.0, False, ref, ref, ref, W_in, b_in, hd ** -0.5, W_out, b_out)
+                dt = time.perf_counter() - t0
+                best = dt if best is None else min(best, dt)
+            err = (got - torch.cat([p.reshape(-1) for p in exp]).float()).abs().max()
+            res["max_abs_err_vs_oracle"] = float(err)
+            res["cpu_baseline"] = dict(value=T / best, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
+                                       sample="full C3 layer, oracle min_mha in fp16 on the host, best of 2")
+        later.append(_cpu_layer)
     return res
 
 
-def _time_gpu(torch, fn, iters=20, warmup=3):
+class Ms(float):
+    """Milliseconds per call: the median over timed batches, with the slowest
+    batch, the mean and the batch shape beside it.  A one-off stall (a host
+    thread descheduled while the device waits for the next launch, an allocator
+    growth, a first-use cost) moves `max` and `mean` and leaves the median."""
+
+    def fields(self):
+        return dict(ms=float(self), ms_max=self.max, ms_mean=self.mean,
+                    timing="median / max / mean over %d batches of %d calls" % (self.batches, self.per))
+
+
+def _time_gpu(torch, fn, iters=20, warmup=3, per=5):
+    """`iters` calls of fn (rounded up to whole batches of `per`), an event
+    between batches.  Events are not put between single calls: an event costs
+    the device a few microseconds, which is the size of the smallest rows."""
     for _ in range(warmup):
         fn()
+    batches = max(3, -(-iters // per))
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(batches + 1)]
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(iters):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / iters
+    with _no_gc():
+        ev[0].record()
+        for b in range(batches):
+            for _ in range(per):
+                fn()
+            ev[b + 1].record()
+        torch.cuda.synchronize()
+    t = sorted(ev[b].elapsed_time(ev[b + 1]) / per for b in range(batches))
+    mid = batches // 2
+    ms = Ms(t[mid] if batches % 2 else 0.5 * (t[mid - 1] + t[mid]))
+    ms.max, ms.mean, ms.batches, ms.per = t[-1], ev[0].elapsed_time(ev[batches]) / (batches * per), batches, per
+    return ms
+
+
+def _host_threads():
+    """Threads for the CPU legs: the visible cores, at most the 16 a one-GPU box grants."""
+    return max(1, min(os.cpu_count() or 1, 16))
 
 
 def _time_cpu(fn, runs=2):
@@ -364,28 +459,42 @@ def _time_cpu(fn, runs=2):
     return best * 1e3
 
 
-def bench_rows(args, torch, dev):
+def bench_rows(args, torch, dev, later):
     """The other rows of the hot path, each on the benchmark configuration that
     exercises it, through the package's Python surface (so allocation of the
     result and, for dense -> nested, the device-to-host copy of the row counts
-    are inside the timed region).  GB/s = algorithmic bytes / time."""
+    are inside the timed region).  GB/s = algorithmic bytes / median time.
+
+    Only device work is timed here.  What the CPU oracle has to time is appended
+    to `later` as closures over host copies of the inputs; main() runs them after
+    every device leg, so that no host thread pool is busy (or still spinning)
+    while a device row is being timed."""
     import nestedtensor_amd as nt
     import oracle
     from nestedtensor_amd import _C
-    from nestedtensor_amd.impl import device_offsets
+    from nestedtensor_amd import ops as _ops
+    from nestedtensor_amd.impl import NestedTensorImpl, device_offsets
     rows = {}
     cpu = not args.no_cpu
-    if cpu:
-        torch.set_num_threads(os.cpu_count() or 1)
 
-    def entry(ms, nbytes, cpu_ms=None, **kw):
-        d = dict(ms=ms, GBps=nbytes / (ms * 1e-3) / 1e9, frac_of_hbm_peak=nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+    def entry(ms, nbytes, **kw):
+        d = ms.fields()
+        d.update(GBps=nbytes / (ms * 1e-3) / 1e9, frac_of_hbm_peak=nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                  algorithmic_bytes=nbytes)
-        if cpu_ms is not None:
-            d["cpu_oracle_ms"] = cpu_ms
-            d["cpu_oracle_GBps"] = nbytes / (cpu_ms * 1e-3) / 1e9
         d.update(kw)
         return d
+
+    def cpu_leg(key, fn, runs, nbytes=None):
+        """Time fn on the host later and file it under rows[key]."""
+        if not cpu:
+            return
+
+        def job():
+            c_ms = _time_cpu(fn, runs)
+            rows[key]["cpu_oracle_ms"] = c_ms
+            nb = rows[key]["algorithmic_bytes"] if nbytes is None else nbytes
+            rows[key]["cpu_oracle_GBps"] = nb / (c_ms * 1e-3) / 1e9
+        later.append(job)
 
     # ---- C1: 64 fp32 [L_i, 256], round trip ---------------------------------
     g = torch.Generator().manual_seed(1010 + 0)
@@ -396,22 +505,21 @@ def bench_rows(args, torch, dev):
     ref = oracle.ref_nested_tensor(parts)
     nvalid, npadded = a.numel(), 64 * 128 * 256
     padded = a.to_padded_tensor(-1e30)
-    ms_pad = _time_gpu(torch, lambda: a.to_padded_tensor(0))
-    ms_back = _time_gpu(torch, lambda: nt.nested_tensor_from_padded_tensor(padded, padding=-1e30))
-    ms_len = _time_gpu(torch, lambda: nt.from_padded_tensor(padded, a))
+    ms_pad = _time_gpu(torch, lambda: a.to_padded_tensor(0), iters=40)
+    ms_back = _time_gpu(torch, lambda: nt.nested_tensor_from_padded_tensor(padded, padding=-1e30), iters=40)
+    ms_len = _time_gpu(torch, lambda: nt.from_padded_tensor(padded, a), iters=40)
     back = nt.nested_tensor_from_padded_tensor(padded, padding=-1e30)
     assert torch.equal(back._impl.buffer.view(torch.int32).cpu(), ref.buffer.view(torch.int32))
-    c_pad = c_back = None
-    if cpu:
-        cp = oracle.to_padded_tensor(ref, -1e30)
-        c_pad = _time_cpu(lambda: oracle.to_padded_tensor(ref, 0), 3)
-        c_back = _time_cpu(lambda: oracle.from_padded_tensor(cp, ref), 3)
-        c_val = _time_cpu(lambda: oracle.nt_from_tensor_mask_vectorised(cp, cp != -1e30), 3)
-    rows["C1_to_padded_tensor"] = entry(ms_pad, 4 * (nvalid + npadded), c_pad)
+    rows["C1_to_padded_tensor"] = entry(ms_pad, 4 * (nvalid + npadded))
     rows["C1_nested_tensor_from_padded_tensor"] = entry(
-        ms_back, 4 * (npadded + 2 * nvalid), c_val if cpu else None,
+        ms_back, 4 * (npadded + 2 * nvalid),
         note="value-based; includes the device-to-host copy of the row counts")
-    rows["C1_from_padded_tensor_length_based"] = entry(ms_len, 4 * 2 * nvalid, c_back)
+    rows["C1_from_padded_tensor_length_based"] = entry(ms_len, 4 * 2 * nvalid)
+    cp = oracle.to_padded_tensor(ref, -1e30)
+    cpu_leg("C1_to_padded_tensor", lambda: oracle.to_padded_tensor(ref, 0), 3)
+    cpu_leg("C1_from_padded_tensor_length_based", lambda: oracle.from_padded_tensor(cp, ref), 3)
+    cpu_leg("C1_nested_tensor_from_padded_tensor",
+            lambda: oracle.nt_from_tensor_mask_vectorised(cp, cp != -1e30), 3)
 
     # ---- C2: 16 fp32 images [3, H_i, W_i] -----------------------------------
     g = torch.Generator().manual_seed(1010 + 1)
@@ -424,40 +532,38 @@ def bench_rows(args, torch, dev):
     data, mask = a2.to_tensor_mask()
     ms_tm = _time_gpu(torch, lambda: a2.to_tensor_mask())
     ms_m = _time_gpu(torch, lambda: torch.ops.nestedtensor.to_mask(a2, 4))
-    ms_fm = _time_gpu(torch, lambda: nt.nested_tensor_from_tensor_mask(data, mask), iters=10)
+    ms_fm = _time_gpu(torch, lambda: nt.nested_tensor_from_tensor_mask(data, mask))
     dev_imgs = [p.to(dev) for p in imgs]
-    ms_pack = _time_gpu(torch, lambda: nt.nested_tensor(dev_imgs, device=dev), iters=10)
+    ms_pack = _time_gpu(torch, lambda: nt.nested_tensor(dev_imgs, device=dev))
     back2 = nt.nested_tensor_from_tensor_mask(data, mask)
     assert torch.equal(back2._impl.buffer, a2._impl.buffer)
-    c_tm = c_fm = c_m = c_pack = None
-    if cpu:
-        ref2 = oracle.ref_nested_tensor(imgs)
-        c_tm = _time_cpu(lambda: oracle.to_tensor_mask(ref2), 1)
-        dcpu, mcpu = data.cpu(), mask.cpu()
-        c_fm = _time_cpu(lambda: oracle.nt_from_tensor_mask_vectorised(dcpu, mcpu), 1)
-        c_m = _time_cpu(lambda: oracle.to_mask(ref2, 4), 1)
-        c_pack = _time_cpu(lambda: oracle.ref_nested_tensor(imgs), 1)
-    rows["C2_to_tensor_mask"] = entry(ms_tm, 4 * (nvalid2 + npadded2) + npadded2, c_tm)
-    rows["C2_to_mask"] = entry(ms_m, npadded2, c_m)
+    rows["C2_to_tensor_mask"] = entry(ms_tm, 4 * (nvalid2 + npadded2) + npadded2)
+    rows["C2_to_mask"] = entry(ms_m, npadded2)
     rows["C2_nested_tensor_from_tensor_mask"] = entry(
-        ms_fm, npadded2 + 2 * 4 * nvalid2, c_fm,
+        ms_fm, npadded2 + 2 * 4 * nvalid2,
         note="includes the device-to-host copy of the row counts; CPU figure is the vectorised "
              "restatement, the reference's literal walk does one host call per mask element")
-    rows["C2_nested_tensor_pack_from_device_tensors"] = entry(ms_pack, 2 * 4 * nvalid2, c_pack)
+    rows["C2_nested_tensor_pack_from_device_tensors"] = entry(ms_pack, 2 * 4 * nvalid2)
+    if cpu:
+        ref2 = oracle.ref_nested_tensor(imgs)
+        dcpu, mcpu = data.cpu(), mask.cpu()
+        cpu_leg("C2_to_tensor_mask", lambda: oracle.to_tensor_mask(ref2), 1)
+        cpu_leg("C2_nested_tensor_from_tensor_mask", lambda: oracle.nt_from_tensor_mask_vectorised(dcpu, mcpu), 1)
+        cpu_leg("C2_to_mask", lambda: oracle.to_mask(ref2, 4), 1)
+        cpu_leg("C2_nested_tensor_pack_from_device_tensors", lambda: oracle.ref_nested_tensor(imgs), 1)
+    del data, mask, back2, dev_imgs, a2
 
     # ---- metadata scan --------------------------------------------------------
     sizes = torch.randint(1, 2049, (4096, 2), dtype=torch.int64).to(dev)
-    ms_scan = _time_gpu(torch, lambda: device_offsets(sizes, 4096, 2))
-    rows["offsets_scan_B4096"] = dict(ms=ms_scan)
+    ms_scan = _time_gpu(torch, lambda: device_offsets(sizes, 4096, 2), iters=40)
+    rows["offsets_scan_B4096"] = ms_scan.fields()
 
     # ---- row-wise ops either side of attention: C3 encoder width and a large buffer
-    from nestedtensor_amd import ops as _ops
     for tag, lens_rw, E_rw in (("C3", [int(v) for v in torch.randint(32, 513, (32,), generator=torch.Generator().manual_seed(1012))], 768),
                                ("large", [2048] * 256, 4096)):
         T_rw = sum(lens_rw)
         buf = torch.randn(T_rw * E_rw, device=dev, dtype=torch.float16)
         sizes_rw = torch.tensor([[L, E_rw] for L in lens_rw], dtype=torch.int64)
-        from nestedtensor_amd.impl import NestedTensorImpl
         x_rw = NestedTensorImpl(buf, sizes_rw)
         r_rw = NestedTensorImpl(torch.randn_like(buf), sizes_rw)
         w_rw, b_rw = torch.randn(E_rw, device=dev).half(), torch.randn(E_rw, device=dev).half()
@@ -465,19 +571,19 @@ def bench_rows(args, torch, dev):
         ms_ln = _time_gpu(torch, lambda: _ops.layer_norm(x_rw, (E_rw,), w_rw, b_rw, 1e-5))
         ms_rln = _time_gpu(torch, lambda: _ops.layer_norm(x_rw, (E_rw,), w_rw, b_rw, 1e-5, residual=r_rw))
         ms_add = _time_gpu(torch, lambda: _ops.add(x_rw, r_rw))
-        c_ln = c_rln = c_add = None
+        rows[tag + "_layer_norm_fp16"] = entry(ms_ln, 2 * nb, rows=T_rw, width=E_rw)
+        rows[tag + "_residual_layer_norm_fp16"] = entry(ms_rln, 3 * nb, rows=T_rw, width=E_rw)
+        rows[tag + "_packed_add_fp16"] = entry(ms_add, 3 * nb, rows=T_rw, width=E_rw)
         if cpu and tag == "C3":
-            def _split(t):
+            def _split(t, lens_rw=lens_rw, E_rw=E_rw):
                 return [p.reshape(L, E_rw) for p, L in zip(t.cpu().split([L * E_rw for L in lens_rw]), lens_rw)]
             ref_rw = oracle.ref_nested_tensor(_split(buf), dtype=torch.float16)
             ref_res = oracle.ref_nested_tensor(_split(r_rw.buffer), dtype=torch.float16)
             w_c, b_c = w_rw.cpu(), b_rw.cpu()
-            c_ln = _time_cpu(lambda: oracle.layer_norm(ref_rw, (E_rw,), w_c, b_c, 1e-5), 2)
-            c_add = _time_cpu(lambda: oracle.add(ref_rw, ref_res), 2)
-            c_rln = _time_cpu(lambda: oracle.layer_norm(oracle.add(ref_rw, ref_res), (E_rw,), w_c, b_c, 1e-5), 2)
-        rows[tag + "_layer_norm_fp16"] = entry(ms_ln, 2 * nb, c_ln, rows=T_rw, width=E_rw)
-        rows[tag + "_residual_layer_norm_fp16"] = entry(ms_rln, 3 * nb, c_rln, rows=T_rw, width=E_rw)
-        rows[tag + "_packed_add_fp16"] = entry(ms_add, 3 * nb, c_add, rows=T_rw, width=E_rw)
+            cpu_leg("C3_layer_norm_fp16", lambda: oracle.layer_norm(ref_rw, (768,), w_c, b_c, 1e-5), 2)
+            cpu_leg("C3_packed_add_fp16", lambda: oracle.add(ref_rw, ref_res), 2)
+            cpu_leg("C3_residual_layer_norm_fp16",
+                    lambda: oracle.layer_norm(oracle.add(ref_rw, ref_res), (768,), w_c, b_c, 1e-5), 2)
         del buf, x_rw, r_rw
 
     # ---- softmax over the ragged last dim: the [H, L_i, L_i] score blocks of C3 -------
@@ -485,16 +591,14 @@ def bench_rows(args, torch, dev):
     lens_sm = [int(v) for v in torch.randint(32, 513, (32,), generator=g)]
     sizes_sm = torch.tensor([[12, L, L] for L in lens_sm], dtype=torch.int64)
     buf_sm = torch.randn(int(sizes_sm.prod(1).sum()), device=dev, dtype=torch.float16)
-    from nestedtensor_amd.impl import NestedTensorImpl as _ImplSm
-    x_sm = _ImplSm(buf_sm, sizes_sm)
+    x_sm = NestedTensorImpl(buf_sm, sizes_sm)
     ms_sm = _time_gpu(torch, lambda: _ops.softmax(x_sm, -1))
-    c_sm = None
+    rows["C3_scores_softmax_fp16"] = entry(ms_sm, 2 * 2 * buf_sm.numel(), rows=int((sizes_sm[:, 0] * sizes_sm[:, 1]).sum()),
+                                           note="what the fused attention kernel never writes: the per-sequence score blocks")
     if cpu:
         parts_sm = [p.reshape(12, L, L) for p, L in zip(buf_sm.cpu().split([12 * L * L for L in lens_sm]), lens_sm)]
         ref_sm = oracle.ref_nested_tensor(parts_sm, dtype=torch.float16)
-        c_sm = _time_cpu(lambda: oracle.softmax(ref_sm, -1), 2)
-    rows["C3_scores_softmax_fp16"] = entry(ms_sm, 2 * 2 * buf_sm.numel(), c_sm, rows=int((sizes_sm[:, 0] * sizes_sm[:, 1]).sum()),
-                                           note="what the fused attention kernel never writes: the per-sequence score blocks")
+        cpu_leg("C3_scores_softmax_fp16", lambda: oracle.softmax(ref_sm, -1), 2)
     del buf_sm, x_sm
 
     # ---- interop formats built from the offsets array ------------------------------
@@ -505,24 +609,25 @@ def bench_rows(args, torch, dev):
     table = torch.randn(V_io, E_io, generator=g).half().to(dev)
     a_ids = nt.nested_tensor(ids_io, device=dev, dtype=torch.int64)
     T_io = sum(lens_io)
-    ms_emb = _time_gpu(torch, lambda: torch.nn.functional.embedding(a_ids, table))
-    ms_bag = _time_gpu(torch, lambda: torch.nn.functional.embedding_bag(a_ids, table, mode="sum"))
+    ms_emb = _time_gpu(torch, lambda: torch.nn.functional.embedding(a_ids, table), iters=40)
+    ms_bag = _time_gpu(torch, lambda: torch.nn.functional.embedding_bag(a_ids, table, mode="sum"), iters=40)
+    nt.check_index_errors()
     x_io = torch.nn.functional.embedding(a_ids, table)
     ms_ps = _time_gpu(torch, lambda: x_io.to_packed_sequence())
-    c_emb = c_ps = c_bag = None
+    rows["C3_embedding_fp16"] = entry(ms_emb, T_io * (8 + 2 * 2 * E_io),
+                                      note="out-of-range indices are counted on the device and reported later "
+                                           "(deferred index check): no device-to-host read in the call")
+    rows["C3_embedding_bag_sum_fp16"] = entry(ms_bag, T_io * (8 + 2 * E_io) + 32 * 2 * E_io,
+                                              note="CPU figure on an fp32 table (torch's CPU embedding_bag has no fp16 path)")
+    rows["C3_to_packed_sequence_fp16"] = entry(ms_ps, T_io * (8 + 2 * 2 * E_io))
     if cpu:
         ref_ids = oracle.ref_nested_tensor(ids_io, dtype=torch.int64)
         tcpu = table.cpu()
-        c_emb = _time_cpu(lambda: oracle.embedding(tcpu, ref_ids), 2)
         tcpu32 = tcpu.float()
-        c_bag = _time_cpu(lambda: oracle.embedding_bag(ref_ids, tcpu32, "sum"), 2)
         ref_x = oracle.ref_nested_tensor([p.cpu() for p in x_io.unbind()], dtype=torch.float16)
-        c_ps = _time_cpu(lambda: oracle.to_packed_sequence(ref_x), 2)
-    rows["C3_embedding_fp16"] = entry(ms_emb, T_io * (8 + 2 * 2 * E_io), c_emb,
-                                      note="includes the device-to-host read of the out-of-range counter")
-    rows["C3_embedding_bag_sum_fp16"] = entry(ms_bag, T_io * (8 + 2 * E_io) + 32 * 2 * E_io, c_bag,
-                                              note="CPU figure on an fp32 table (torch's CPU embedding_bag has no fp16 path)")
-    rows["C3_to_packed_sequence_fp16"] = entry(ms_ps, T_io * (8 + 2 * 2 * E_io), c_ps)
+        cpu_leg("C3_embedding_fp16", lambda: oracle.embedding(tcpu, ref_ids), 2)
+        cpu_leg("C3_embedding_bag_sum_fp16", lambda: oracle.embedding_bag(ref_ids, tcpu32, "sum"), 2)
+        cpu_leg("C3_to_packed_sequence_fp16", lambda: oracle.to_packed_sequence(ref_x), 2)
     big_T, big_E = 1 << 20, 1024
     big_idx = torch.randint(V_io, (big_T,), device=dev)
     big_tab = torch.randn(V_io, big_E, device=dev, dtype=torch.float16)
@@ -530,35 +635,22 @@ def bench_rows(args, torch, dev):
     stream = _C.current_stream(dev)
     ms_big = _time_gpu(torch, lambda: _C.check(_C.lib.nt_gather_rows(
         _C.ptr(big_tab), V_io, big_E * 2, _C.ptr(big_idx), _C.ptr(big_out), big_T, None, stream)))
-    rows["large_gather_rows_fp16"] = entry(ms_big, big_T * (8 + 2 * 2 * big_E), None, rows=big_T, width=big_E,
+    rows["large_gather_rows_fp16"] = entry(ms_big, big_T * (8 + 2 * 2 * big_E), rows=big_T, width=big_E,
                                            note="2 GiB written; the 62 MB table is re-read from cache")
-    del big_idx, big_tab, big_out
+    del big_idx, big_tab, big_out, table, x_io
 
     # ---- channels-last ragged images: per-constituent transpose -----------------------
     g = torch.Generator().manual_seed(1010 + 1)
     hw_t = torch.randint(480, 1025, (16, 2), generator=g)
     sizes_t = torch.tensor([[64, int(h), int(w)] for h, w in hw_t], dtype=torch.int64)
     buf_t = torch.randn(int(sizes_t.prod(1).sum()), device=dev, dtype=torch.float16)
-    from nestedtensor_amd.impl import NestedTensorImpl as _Impl
-    img = _Impl(buf_t, sizes_t)
+    img = NestedTensorImpl(buf_t, sizes_t)
     nhwc = _ops.transpose_nchw_nhwc(img)
     ms_t0 = _time_gpu(torch, lambda: _ops.transpose_nchw_nhwc(img))
     ms_t1 = _time_gpu(torch, lambda: _ops.transpose_nhwc_nchw(nhwc))
     assert torch.equal(_ops.transpose_nhwc_nchw(nhwc).buffer, buf_t)
     rows["C2x64ch_transpose_nchw_nhwc_fp16"] = entry(ms_t0, 2 * 2 * buf_t.numel())
     rows["C2x64ch_transpose_nhwc_nchw_fp16"] = entry(ms_t1, 2 * 2 * buf_t.numel())
-    if cpu:
-        # CPU side on the first two images (GB/s does not depend on the count)
-        n2 = int(sizes_t[:2].prod(1).sum())
-        parts_t = [p.reshape(tuple(int(v) for v in sz)) for p, sz in
-                   zip(buf_t[:n2].cpu().split([int(v) for v in sizes_t[:2].prod(1)]), sizes_t[:2])]
-        ref_t = oracle.ref_nested_tensor(parts_t, dtype=torch.float16)
-        ref_nhwc = oracle.transpose_nchw_nhwc(ref_t)
-        for key, fn in (("C2x64ch_transpose_nchw_nhwc_fp16", lambda: oracle.transpose_nchw_nhwc(ref_t)),
-                        ("C2x64ch_transpose_nhwc_nchw_fp16", lambda: oracle.transpose_nhwc_nchw(ref_nhwc))):
-            c_ms = _time_cpu(fn, 2)
-            rows[key]["cpu_oracle_GBps"] = 2 * 2 * n2 / (c_ms * 1e-3) / 1e9
-            rows[key]["cpu_oracle_sample"] = "first 2 of 16 images, %.1f ms" % c_ms
     # 1x1 convolution 64 -> 256 channels: row-major input (transpose, GEMM, transpose)
     # against the channels-last storage of the same images (the GEMM alone)
     w11 = (torch.randn(256, 64, 1, 1, device=dev) * 0.1).half()
@@ -569,18 +661,39 @@ def bench_rows(args, torch, dev):
     conv_bytes = 2 * pix * (64 + 256)
     for key, ms_c in (("C2x64ch_conv2d_1x1_to_256ch_fp16", ms_c0),
                       ("C2x64ch_conv2d_1x1_to_256ch_channels_last_fp16", ms_c1)):
-        rows[key] = entry(ms_c, conv_bytes, None, pixels=pix)
+        rows[key] = entry(ms_c, conv_bytes, pixels=pix)
         rows[key]["tflops"] = 2.0 * pix * 64 * 256 / (ms_c * 1e-3) / 1e12
     if cpu:
+        # CPU side on the first two images (GB/s does not depend on the count)
+        n2 = int(sizes_t[:2].prod(1).sum())
+        parts_t = [p.reshape(tuple(int(v) for v in sz)) for p, sz in
+                   zip(buf_t[:n2].cpu().split([int(v) for v in sizes_t[:2].prod(1)]), sizes_t[:2])]
+        ref_t = oracle.ref_nested_tensor(parts_t, dtype=torch.float16)
         h0, w0 = int(sizes_t[0, 1]), int(sizes_t[0, 2])
         x0 = buf_t[:64 * h0 * w0].reshape(64, h0, w0).float().cpu()
         ref_c = oracle.ref_nested_tensor([x0], dtype=torch.float32)
-        w_c = w11.float().cpu()
-        c_ms = _time_cpu(lambda: oracle.conv2d(ref_c, w_c), 1)
-        for key in ("C2x64ch_conv2d_1x1_to_256ch_fp16", "C2x64ch_conv2d_1x1_to_256ch_channels_last_fp16"):
-            rows[key]["cpu_oracle_tflops"] = 2.0 * h0 * w0 * 64 * 256 / (c_ms * 1e-3) / 1e12
-            rows[key]["cpu_oracle_sample"] = "first of 16 images in fp32, %.1f ms" % c_ms
+        w_c11 = w11.float().cpu()
+
+        def _cpu_images():
+            ref_nhwc = oracle.transpose_nchw_nhwc(ref_t)
+            for key, fn in (("C2x64ch_transpose_nchw_nhwc_fp16", lambda: oracle.transpose_nchw_nhwc(ref_t)),
+                            ("C2x64ch_transpose_nhwc_nchw_fp16", lambda: oracle.transpose_nhwc_nchw(ref_nhwc))):
+                c_ms = _time_cpu(fn, 2)
+                rows[key]["cpu_oracle_GBps"] = 2 * 2 * n2 / (c_ms * 1e-3) / 1e9
+                rows[key]["cpu_oracle_sample"] = "first 2 of 16 images, %.1f ms" % c_ms
+            c_ms = _time_cpu(lambda: oracle.conv2d(ref_c, w_c11), 1)
+            for key in ("C2x64ch_conv2d_1x1_to_256ch_fp16", "C2x64ch_conv2d_1x1_to_256ch_channels_last_fp16"):
+                rows[key]["cpu_oracle_tflops"] = 2.0 * h0 * w0 * 64 * 256 / (c_ms * 1e-3) / 1e12
+                rows[key]["cpu_oracle_sample"] = "first of 16 images in fp32, %.1f ms" % c_ms
+        later.append(_cpu_images)
     del buf_t, img, nhwc, img_cl, w11
+
+    def mha_row(ms, n_tok, flops, **kw):
+        d = ms.fields()
+        d.update(kw)
+        d.update(tokens_per_s=n_tok / (ms * 1e-3), flops=flops, TFLOPs=flops / (ms * 1e-3) / 1e12,
+                 frac_of_mfma_peak=flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS)
+        return d
 
     # ---- C4: bt_min_mha bf16, high raggedness ---------------------------------
     g = torch.Generator().manual_seed(1010 + 3)
@@ -595,29 +708,39 @@ def bench_rows(args, torch, dev):
     ms4 = _time_gpu(torch, lambda: torch.ops.nestedtensor.bt_min_mha(
         H, 64, 0.0, False, a4, a4, a4, W_in, b_in, 64 ** -0.5, W_out, b_out), iters=50, warmup=5)
     T4 = sum(lens)
-    fl4 = 8 * T4 * E * E + 4 * E * sum(L * L for L in lens)
-    rows["C4_bt_min_mha_bf16"] = dict(ms=ms4, tokens=T4, tokens_per_s=T4 / (ms4 * 1e-3), flops=fl4,
-                                      TFLOPs=fl4 / (ms4 * 1e-3) / 1e12,
-                                      frac_of_mfma_peak=fl4 / (ms4 * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS)
+    rows["C4_bt_min_mha_bf16"] = mha_row(ms4, T4, 8 * T4 * E * E + 4 * E * sum(L * L for L in lens), tokens=T4)
+
+    # ---- C3 in fp32: the reference's own dtype for this test configuration ------------
+    g = torch.Generator().manual_seed(1010 + 2)
+    lens3 = [int(v) for v in torch.randint(32, 513, (32,), generator=g)]
+    E3, H3 = 768, 12
+    a3 = nt.nested_tensor([torch.randn(L, E3, generator=g) for L in lens3], device=dev, dtype=torch.float32)
+    W3_in = (torch.randn(3 * E3, E3, generator=g) * 0.02).to(dev)
+    W3_out = (torch.randn(E3, E3, generator=g) * 0.02).to(dev)
+    b3_in, b3_out = torch.zeros(3 * E3, device=dev), torch.zeros(E3, device=dev)
+    ms3 = _time_gpu(torch, lambda: torch.ops.nestedtensor.min_mha(
+        H3, 64, 0.0, False, a3, a3, a3, W3_in, b3_in, 64 ** -0.5, W3_out, b3_out), iters=20, warmup=3)
+    T3 = sum(lens3)
+    fl3 = 8 * T3 * E3 * E3 + 4 * E3 * sum(L * L for L in lens3)
+    rows["C3_min_mha_fp32"] = mha_row(ms3, T3, fl3, tokens=T3)
+    rows["C3_min_mha_fp32"]["frac_of_mfma_peak"] = fl3 / (ms3 * 1e-3) / 1e12 / MFMA_F32_PEAK_TFLOPS
+    rows["C3_min_mha_fp32"]["peak"] = "fp32 MFMA, %.1f TFLOP/s" % MFMA_F32_PEAK_TFLOPS
+    del a3, W3_in, W3_out
 
     # ---- a larger layer for scale: 16 sequences of 256..2048 tokens, d = 2048, 16 heads of 128 ----
     g = torch.Generator().manual_seed(1010 + 6)
     El, Hl = 2048, 16
     lens_l = [int(v) for v in torch.randint(256, 2049, (16,), generator=g)]
     bufl = torch.randn(sum(lens_l) * El, device=dev, dtype=torch.float16)
-    from nestedtensor_amd.impl import NestedTensorImpl as _ImplL
-    al = nt.NestedTensor(_ImplL(bufl, torch.tensor([[L, El] for L in lens_l], dtype=torch.int64)))
+    al = nt.NestedTensor(NestedTensorImpl(bufl, torch.tensor([[L, El] for L in lens_l], dtype=torch.int64)))
     Wl_in = (torch.randn(3 * El, El, device=dev) * 0.02).half()
     Wl_out = (torch.randn(El, El, device=dev) * 0.02).half()
     bl_in, bl_out = torch.zeros(3 * El, device=dev).half(), torch.zeros(El, device=dev).half()
     msl = _time_gpu(torch, lambda: torch.ops.nestedtensor.min_mha(
         Hl, 128, 0.0, False, al, al, al, Wl_in, bl_in, 128 ** -0.5, Wl_out, bl_out), iters=20, warmup=3)
     Tl = sum(lens_l)
-    fll = 8 * Tl * El * El + 4 * El * sum(L * L for L in lens_l)
-    rows["large_min_mha_fp16"] = dict(
-        ms=msl, workload="B=16, L~U[256,2048], d=2048, 16x128", tokens=Tl, tokens_per_s=Tl / (msl * 1e-3),
-        flops=fll, TFLOPs=fll / (msl * 1e-3) / 1e12,
-        frac_of_mfma_peak=fll / (msl * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS)
+    rows["large_min_mha_fp16"] = mha_row(msl, Tl, 8 * Tl * El * El + 4 * El * sum(L * L for L in lens_l),
+                                         workload="B=16, L~U[256,2048], d=2048, 16x128", tokens=Tl)
     del bufl, al, Wl_in, Wl_out
 
     # ---- cross-attention: 100 queries per sequence over ragged memories (decoder-style) ----
@@ -634,23 +757,21 @@ def bench_rows(args, torch, dev):
     msx = _time_gpu(torch, lambda: torch.ops.nestedtensor.min_mha(Hx, 64, 0.0, False, aq, am, am, *xargs),
                     iters=50, warmup=5)
     Tq, Tk = 100 * len(kv_lens), sum(kv_lens)
-    flx = 2 * Ex * Ex * (2 * Tq + 2 * Tk) + 4 * Ex * 100 * Tk
-    rows["cross_attention_fp16"] = dict(
-        ms=msx, workload="B=32, 100 queries per sequence, memory L~U[256,1024], d=512, 8x64",
-        query_tokens=Tq, memory_tokens=Tk, flops=flx, TFLOPs=flx / (msx * 1e-3) / 1e12,
-        frac_of_mfma_peak=flx / (msx * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS)
+    rows["cross_attention_fp16"] = mha_row(
+        msx, Tq, 2 * Ex * Ex * (2 * Tq + 2 * Tk) + 4 * Ex * 100 * Tk,
+        workload="B=32, 100 queries per sequence, memory L~U[256,1024], d=512, 8x64",
+        query_tokens=Tq, memory_tokens=Tk)
     if cpu:
-        rq, rm = oracle.ref_nested_tensor(qs, dtype=torch.float16), oracle.ref_nested_tensor(mems, dtype=torch.float16)
-        ref_out = None
+        got = torch.ops.nestedtensor.min_mha(Hx, 64, 0.0, False, aq, am, am, *xargs)._impl.buffer.float().cpu()
 
         def _cpu_cross():
-            nonlocal ref_out
+            rq, rm = oracle.ref_nested_tensor(qs, dtype=torch.float16), oracle.ref_nested_tensor(mems, dtype=torch.float16)
+            t0 = time.perf_counter()
             ref_out = oracle.min_mha(Hx, 64, 0.0, False, rq, rm, rm, Wx_in, bx_in, 64 ** -0.5, Wx_out, bx_out)
-        rows["cross_attention_fp16"]["cpu_oracle_ms"] = _time_cpu(_cpu_cross, 1)
-        got = torch.ops.nestedtensor.min_mha(Hx, 64, 0.0, False, aq, am, am, *xargs)
-        exp = torch.cat([p.reshape(-1) for p in ref_out]).float()
-        rows["cross_attention_fp16"]["max_abs_err_vs_oracle"] = float(
-            (got._impl.buffer.float().cpu() - exp).abs().max())
+            rows["cross_attention_fp16"]["cpu_oracle_ms"] = (time.perf_counter() - t0) * 1e3
+            exp = torch.cat([p.reshape(-1) for p in ref_out]).float()
+            rows["cross_attention_fp16"]["max_abs_err_vs_oracle"] = float((got - exp).abs().max())
+        later.append(_cpu_cross)
     return rows
 
 
@@ -669,6 +790,9 @@ def main():
 
     if args.pmc_probe:
         pmc_probe(args, torch, dev)
+        return
+    if args.mha_probe:
+        mha_probe(args, torch, dev)
         return
     c5 = bench_c5(args, torch, dev)
     line = {
@@ -691,11 +815,16 @@ def main():
         "roofline": c5["roofline"],
         "unpad": c5["unpad"],
     }
+    # every device leg first, then everything the CPU oracle has to time
+    later = []
     if not args.no_mha:
-        line["mha"] = bench_mha_c3(args, torch, dev)
+        line["mha"] = bench_mha_c3(args, torch, dev, later)
     if not args.no_rows:
-        line["rows"] = bench_rows(args, torch, dev)
+        line["rows"] = bench_rows(args, torch, dev, later)
     if not args.no_cpu:
+        torch.set_num_threads(_host_threads())
+        for job in later:
+            job()
         line["cpu_baseline"] = cpu_baseline_c5(torch)
     print(json.dumps(line))
 

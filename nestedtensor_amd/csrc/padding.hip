@@ -16,7 +16,6 @@
 //
 // All index math is int64: the largest configuration holds 1.7e10 elements.
 #include "nt_common.h"
-#include <stdlib.h>
 
 // Tuning knobs of the row kernels (compile-time).
 #ifndef NT_ROW_UNROLL
@@ -671,9 +670,7 @@ static int launch_rows_t(int eb, const RowParams& p, int64_t max_row_bytes, hipS
 // Short rows: see row_batch_kernel (nrag == 1) and row_group_kernel.
 template <int MODE, int kT>
 static int launch_batch(int eb, const RowParams& p, hipStream_t stream) {
-  static int rpg_env = -1;
-  if (rpg_env < 0) { const char* e = getenv("NT_ROW_GROUP_RT"); rpg_env = e ? atoi(e) : 0; }
-  const int rpg = p.nrag == 1 ? 2 : (rpg_env > 0 ? rpg_env : NT_ROW_GROUP);
+  const int rpg = p.nrag == 1 ? 2 : NT_ROW_GROUP;
   const int64_t groups = (p.nrows + rpg - 1) / rpg;
   const int64_t wgs = (groups + (256 / kT) - 1) / (256 / kT);
   const int64_t gx = wgs < 65535 ? wgs : 65535;
@@ -704,9 +701,7 @@ static int launch_rows(int eb, const RowParams& p, int64_t max_row_bytes, hipStr
   if (p.nrows > 0x7fffffffLL) {
     return fail(NT_ERR_UNSUPPORTED, "row count %lld exceeds the grid limit", (long long)p.nrows);
   }
-  static int use_batch = -1;
-  if (use_batch < 0) { const char* e = getenv("NT_ROW_BATCH_RT"); use_batch = (e && atoi(e) == 1) ? 0 : 1; }
-  if (MODE != kPack && p.nrows >= 4096 && use_batch) {
+  if (MODE != kPack && p.nrows >= 4096) {
     // many short rows: several rows per lane group, all of their chunks in flight
     if (max_row_bytes <= 1024) return launch_batch<MODE, 64>(eb, p, stream);
     if (max_row_bytes <= 4096) return launch_batch<MODE, 256>(eb, p, stream);

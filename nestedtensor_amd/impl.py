@@ -162,6 +162,9 @@ class NestedTensorImpl:
         if cached is not None and cached[0] is kv.sizes:
             return cached[1]
         q_lens, k_lens = self.sizes[:, 0], kv.sizes[:, 0]
+        if int(q_lens.sum()) > 0x7fffffff or int(k_lens.sum()) > 0x7fffffff:
+            raise RuntimeError("attention: %d query and %d key tokens; the work list holds token indices "
+                               "as int32" % (int(q_lens.sum()), int(k_lens.sum())))
         q_starts = torch.cumsum(q_lens, 0) - q_lens
         k_starts = torch.cumsum(k_lens, 0) - k_lens
         order = torch.argsort(k_lens, descending=True, stable=True)

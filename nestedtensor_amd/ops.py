@@ -699,10 +699,81 @@ def conv2d(impl, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
 
 # ---- consumers of the offsets array: interop formats ----------------------------
 
-def _raise_if_oob(oob, what):
-    n = int(oob.item())
-    if n:
+# Out-of-range indices.  torch's own device embedding traps asynchronously; here
+# the kernels write zero rows for such indices and count them in a counter that
+# lives on the device for the life of the process (it only ever grows).  How the
+# count reaches the host is a setting:
+#   "deferred"  (default) after each call the counter is copied, asynchronously,
+#               into pinned host memory; the next embedding / embedding_bag call
+#               and check_index_errors() look at that copy and raise IndexError
+#               for whatever has arrived.  No call waits for the device, and the
+#               ops can be captured in a HIP graph.
+#   "immediate" every call waits for its own count and raises before returning.
+#   "off"       indices are trusted; nothing is copied.
+_INDEX_CHECK_MODES = ("deferred", "immediate", "off")
+_index_check_mode = "deferred"
+_index_counters = {}      # device index -> [device int32[1], pinned int32[1], count already reported]
+
+
+def set_index_check(mode):
+    """Select how out-of-range indices of embedding / embedding_bag are reported
+    ("deferred", "immediate" or "off"); returns the previous setting."""
+    global _index_check_mode
+    if mode not in _INDEX_CHECK_MODES:
+        raise ValueError("index check mode must be one of %s, got %r" % (", ".join(_INDEX_CHECK_MODES), mode))
+    previous, _index_check_mode = _index_check_mode, mode
+    return previous
+
+
+def _index_counter(device):
+    slot = _index_counters.get(device.index)
+    if slot is None:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("embedding / embedding_bag: the index counter of this device cannot be created "
+                               "during stream capture; run the op once before capturing (or set_index_check('off')).")
+        slot = [torch.zeros(1, dtype=torch.int32, device=device),
+                torch.zeros(1, dtype=torch.int32).pin_memory(), 0]
+        _index_counters[device.index] = slot
+    return slot
+
+
+def _report_index_errors(slot, what):
+    seen = int(slot[1][0])            # a read of pinned host memory, no device call
+    if seen != slot[2]:
+        n, slot[2] = seen - slot[2], seen
         raise IndexError("%s: %d index value(s) out of range" % (what, n))
+
+
+def check_index_errors(synchronize=True):
+    """Raise IndexError if an embedding / embedding_bag call issued so far met
+    out-of-range indices that have not been reported yet.  With synchronize (the
+    default) the devices that ran such calls are waited for first, so every call
+    issued before this one is covered; without it only the counts that have
+    already arrived on the host are looked at."""
+    for index, slot in _index_counters.items():
+        if synchronize:
+            torch.cuda.synchronize(index)
+        _report_index_errors(slot, "embedding / embedding_bag (an earlier call)")
+
+
+def _oob_begin(device, what):
+    """Counter pointer for a launch (None when checks are off); in deferred mode
+    reports what earlier calls have left."""
+    if _index_check_mode == "off":
+        return None, None
+    slot = _index_counter(device)
+    if _index_check_mode == "deferred" and not torch.cuda.is_current_stream_capturing():
+        _report_index_errors(slot, what + " (an earlier call)")
+    return slot, _C.ptr(slot[0])
+
+
+def _oob_end(slot, what):
+    if slot is None:
+        return
+    slot[1].copy_(slot[0], non_blocking=True)
+    if _index_check_mode == "immediate":
+        torch.cuda.current_stream(slot[0].device).synchronize()
+        _report_index_errors(slot, what)
 
 
 def embedding(weight, indices, padding_idx=None, max_norm=None, norm_type=2.0,
@@ -729,12 +800,12 @@ def embedding(weight, indices, padding_idx=None, max_norm=None, norm_type=2.0,
     idx64 = idx.to(torch.int64)
     V, E = weight.shape
     out = torch.empty(idx.numel() * E, dtype=weight.dtype, device=weight.device)
-    oob = torch.zeros(1, dtype=torch.int32, device=weight.device)
+    slot, oob = _oob_begin(weight.device, "embedding")
     with _C.on_device(weight.device):
         _C.check(_C.lib.nt_gather_rows(_C.ptr(weight), V, E * weight.element_size(), _C.ptr(idx64),
-                                       _C.ptr(out), idx.numel(), _C.ptr(oob),
+                                       _C.ptr(out), idx.numel(), oob,
                                        _C.current_stream(weight.device)))
-    _raise_if_oob(oob, "embedding")
+        _oob_end(slot, "embedding")
     if indices.sizes.dim() == 0:
         sizes = indices.sizes
     else:
@@ -781,13 +852,13 @@ def embedding_bag(input, weight, offsets=None, max_norm=None, norm_type=2, scale
     V, E = weight.shape
     B = input.B
     out = torch.empty((B, E), dtype=weight.dtype, device=weight.device)
-    oob = torch.zeros(1, dtype=torch.int32, device=weight.device)
+    slot, oob = _oob_begin(weight.device, "embedding_bag")
     with _C.on_device(weight.device):
         _C.check(_C.lib.nt_embedding_bag(_C.ptr(weight), E, V, _C.ptr(idx64), idx64.numel(),
                                          _C.ptr(input.offsets_dev()),
                                          _C.ptr(out), B, E, modes[mode], _C.dtype_code(weight.dtype),
-                                         _C.ptr(oob), _C.current_stream(weight.device)))
-    _raise_if_oob(oob, "embedding_bag")
+                                         oob, _C.current_stream(weight.device)))
+        _oob_end(slot, "embedding_bag")
     return out
 
 

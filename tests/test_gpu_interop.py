@@ -35,10 +35,102 @@ def test_embedding(E, dtype):
     assert torch.equal(got2._impl.buffer.cpu(), exp.buffer)
 
 
-def test_embedding_out_of_range_raises():
-    a = nt.nested_tensor([torch.tensor([1, 2, 50]), torch.tensor([3])], device=DEV, dtype=torch.int64)
-    with pytest.raises(IndexError):
-        torch.nn.functional.embedding(a, torch.randn(10, 4, device=DEV))
+def _bad_and_good():
+    bad = nt.nested_tensor([torch.tensor([1, 2, 50]), torch.tensor([3, -1])], device=DEV, dtype=torch.int64)
+    good = nt.nested_tensor([torch.tensor([1, 2, 5]), torch.tensor([3])], device=DEV, dtype=torch.int64)
+    return bad, good, torch.randn(10, 4, device=DEV)
+
+
+@pytest.mark.parametrize("op", ["embedding", "embedding_bag"])
+def test_out_of_range_indices_immediate(op):
+    fn = getattr(torch.nn.functional, op)
+    bad, good, w = _bad_and_good()
+    previous = nt.set_index_check("immediate")
+    try:
+        with pytest.raises(IndexError, match="2 index value"):
+            fn(bad, w)
+        fn(good, w)                       # nothing is left over for the next call
+        nt.check_index_errors()
+    finally:
+        nt.set_index_check(previous)
+
+
+@pytest.mark.parametrize("op", ["embedding", "embedding_bag"])
+def test_out_of_range_indices_deferred(op):
+    # the default: the call itself returns (zero rows for the bad indices, no wait
+    # for the device); the count is raised by check_index_errors() or by the next call
+    fn = getattr(torch.nn.functional, op)
+    bad, good, w = _bad_and_good()
+    assert nt.set_index_check("deferred") == "deferred"
+    nt.check_index_errors()
+    out = fn(bad, w)
+    dense = out.to_padded_tensor(0) if op == "embedding" else out
+    if op == "embedding":
+        assert torch.equal(dense[0, 2], torch.zeros(4, device=DEV))       # index 50: a zero row
+        assert torch.equal(dense[0, 1], w[2])
+    with pytest.raises(IndexError, match="2 index value"):
+        nt.check_index_errors()
+    nt.check_index_errors()               # reported once
+    fn(bad, w)
+    torch.cuda.synchronize()
+    with pytest.raises(IndexError, match="earlier call"):
+        fn(good, w)
+    fn(good, w)
+    nt.check_index_errors()
+
+
+def test_out_of_range_indices_off():
+    bad, good, w = _bad_and_good()
+    previous = nt.set_index_check("off")
+    try:
+        torch.nn.functional.embedding(bad, w)
+        torch.cuda.synchronize()
+        nt.check_index_errors()
+    finally:
+        nt.set_index_check(previous)
+    with pytest.raises(ValueError):
+        nt.set_index_check("sometimes")
+
+
+@pytest.mark.parametrize("op", ["embedding", "embedding_bag"])
+def test_embedding_ops_under_hip_graph_replays(op):
+    # neither op reads anything back from the device, so both can be captured; every
+    # replay, with new indices and eager work in between, must equal the eager result
+    V, E = 500, 72
+    fn = getattr(torch.nn.functional, op)
+    kw = dict(mode="sum") if op == "embedding_bag" else {}
+    g = torch.Generator().manual_seed(31)
+    lens = [17, 1, 300, 64, 5]
+    a = nt.nested_tensor([torch.randint(V, (L,), generator=g) for L in lens], device=DEV, dtype=torch.int64)
+    w = torch.randn(V, E, generator=g).half().to(DEV)
+
+    def buf(t):
+        return t._impl.buffer if op == "embedding" else t
+
+    for _ in range(3):
+        fn(a, w, **kw)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn(a, w, **kw)
+        with torch.cuda.graph(graph, stream=side):
+            out = fn(a, w, **kw)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(4):
+        a._impl.buffer.copy_(torch.randint(V, (sum(lens),), generator=g).to(DEV))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = buf(out).clone()
+        exp = buf(fn(a, w, **kw))
+        torch.cuda.synchronize()
+        assert torch.equal(got, exp), "replay %d differs from the eager call" % rep
+    # an out-of-range index met during a replay is reported like any other
+    a._impl.buffer[3] = V + 7
+    graph.replay()
+    with pytest.raises(IndexError, match="1 index value"):
+        nt.check_index_errors()
 
 
 @pytest.mark.parametrize("mode", ["sum", "mean", "max"])
