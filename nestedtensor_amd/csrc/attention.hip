@@ -16,9 +16,10 @@
 // the softmax row reductions are in-lane plus one cross-half shuffle, and the
 // score accumulators are, as they stand, the B-operand of the second product.
 //
-// Any head_dim / fp32 takes the generic kernel further down (one wavefront per
-// query row, fp32 FMA); it is the parity path for shapes the MFMA kernel does
-// not cover, not a performance path.
+// fp32 with head_dim 32 / 64 / 128 has a kernel of its own on the fp32 matrix
+// instruction (further down).  Any other head_dim takes the generic kernel (one
+// wavefront per query row, fp32 FMA); it is the parity path for shapes the MFMA
+// kernels do not cover, not a performance path.
 #include "nt_common.h"
 
 namespace nt {
@@ -723,6 +724,181 @@ __global__ __launch_bounds__(64) void attention_rows_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// fp32 attention on the matrix pipe (v_mfma_f32_32x32x2_f32), head_dim 32 / 64 /
+// 128.  Same transposed formulation as above: per wavefront 32 query rows, one
+// per lane pair (q = lane % 32; the two lane halves hold different keys),
+//   S^T[key, q] = K[key, :] . Q[q, :]      A = K rows (LDS), B = Q (registers)
+//   O^T[d,  q] += V^T[d, key] P^T[key, q]  A = V as it lies row-major in LDS, B = P^T
+// so the score accumulators are the B operand of the second product as they
+// stand and V needs no transpose.  The k index of an MFMA step only has to mean
+// the same thing in both operands: in the first product lane half g takes head
+// dims 8t + 4g .. 8t + 4g + 3 over four consecutive steps (one 16-byte LDS read
+// of the K row); in the second, step i contracts the key that accumulator i of
+// that lane half holds, 8 (i / 4) + 4 g + i % 4.  Everything stays fp32
+// (exp2 on scores prescaled by log2 e).  A workgroup owns 128 query rows of
+// (sequence, head) and walks the sequence's keys in tiles of 32, the next tile's
+// global loads in flight while the current one is multiplied, two LDS buffers.
+template <int HD>
+__global__ __launch_bounds__(256) void varlen_attention_f32_kernel(
+    const float* __restrict__ Q, int64_t ldq, const float* __restrict__ Kp, int64_t ldk,
+    const float* __restrict__ Vp, int64_t ldv, float* __restrict__ O, int64_t ldo,
+    const int64_t* __restrict__ q_offsets, const int64_t* __restrict__ kv_offsets,
+    float scale_log2e) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  constexpr int kKT = 32;                      // keys per tile
+  constexpr int kKs = HD + 4;                  // K row stride in floats: 16-byte reads of 16 rows hit 16 bank groups
+  constexpr int kVs = HD + 8;                  // V row stride: the two lane halves (keys 4 apart) use different banks
+  constexpr int kBuf = kKT * (kKs + kVs);
+  constexpr int kC4 = HD / 4;                  // 16-byte pieces per row
+  constexpr int kPieces = kKT * kC4 / 256;     // pieces per thread and operand: 1, 2, 4
+  __shared__ __align__(16) float lds[2 * kBuf];
+
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int64_t q_begin = q_offsets[b];
+  const int64_t Lq = q_offsets[b + 1] - q_begin;
+  const int64_t q0 = (int64_t)blockIdx.x * 128;
+  if (q0 >= Lq) return;                        // uniform
+  const int64_t kv_begin = kv_offsets[b];
+  const int64_t Lk = kv_offsets[b + 1] - kv_begin;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 31, half = lane >> 5;
+
+  // this lane's query row, prescaled: dims 8t + 4 half + u  ->  qf[4t + u]
+  const int64_t qrow = q0 + wave * 32 + col;
+  const bool q_ok = qrow < Lq;
+  float qf[HD / 2];
+  {
+    const float* qp = Q + (q_begin + (q_ok ? qrow : q0)) * ldq + (int64_t)h * HD + 4 * half;
+#pragma unroll
+    for (int t = 0; t < HD / 8; ++t) {
+      f32x4 v = *reinterpret_cast<const f32x4*>(qp + 8 * t);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) qf[4 * t + u] = q_ok ? v[u] * scale_log2e : 0.0f;
+    }
+  }
+
+  f32x4 kreg[kPieces], vreg[kPieces];
+  const float* kbase = Kp + kv_begin * ldk + (int64_t)h * HD;
+  const float* vbase = Vp + kv_begin * ldv + (int64_t)h * HD;
+  auto gload = [&](int64_t k0) {
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i) {
+      const int p = tid + 256 * i;
+      const int row = p / kC4, c4 = p % kC4;
+      const int64_t key = k0 + row;
+      const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+      // rows past the last key are zero: 0 * V must not meet a NaN
+      kreg[i] = key < Lk ? *reinterpret_cast<const f32x4*>(kbase + key * ldk + 4 * c4) : zero;
+      vreg[i] = key < Lk ? *reinterpret_cast<const f32x4*>(vbase + key * ldv + 4 * c4) : zero;
+    }
+  };
+  auto lstore = [&](float* buf) {
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i) {
+      const int p = tid + 256 * i;
+      const int row = p / kC4, c4 = p % kC4;
+      *reinterpret_cast<f32x4*>(buf + row * kKs + 4 * c4) = kreg[i];
+      *reinterpret_cast<f32x4*>(buf + kKT * kKs + row * kVs + 4 * c4) = vreg[i];
+    }
+  };
+
+  acc16 o[HD / 32];
+#pragma unroll
+  for (int j = 0; j < HD / 32; ++j)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[j][i] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;       // l_run: this lane half's keys only
+
+  const int64_t n_tiles = (Lk + kKT - 1) / kKT;
+  if (n_tiles > 0) {
+    gload(0);
+    lstore(lds);
+  }
+  __syncthreads();
+  for (int64_t t = 0; t < n_tiles; ++t) {
+    float* cur = lds + (t & 1) * kBuf;
+    const bool more = t + 1 < n_tiles;
+    if (more) gload((t + 1) * kKT);
+    const float* Ks = cur + col * kKs + 4 * half;
+    const float* Vs = cur + kKT * kKs + 4 * half * kVs + col;
+
+    acc16 s;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.0f;
+#pragma unroll
+    for (int tt = 0; tt < HD / 8; ++tt) {
+      const f32x4 kf = *reinterpret_cast<const f32x4*>(Ks + 8 * tt);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[u], qf[4 * tt + u], s, 0, 0, 0);
+    }
+    // accumulator i: key 8 (i / 4) + 4 half + i % 4 of the tile, query col
+    const int64_t left = Lk - t * kKT;
+    if (left < kKT) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        if (8 * (i / 4) + 4 * half + (i % 4) >= left) s[i] = -INFINITY;
+      }
+    }
+    float m_tile = s[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) m_tile = fmaxf(m_tile, s[i]);
+    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));      // finite: the tile holds a valid key
+    const float m_new = fmaxf(m_run, m_tile);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    m_run = m_new;
+    float l_tile = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      s[i] = __builtin_amdgcn_exp2f(s[i] - m_new);
+      l_tile += s[i];
+    }
+    l_run = l_run * alpha + l_tile;
+#pragma unroll
+    for (int j = 0; j < HD / 32; ++j) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[j][i] *= alpha;
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float* vrow = Vs + (8 * (i / 4) + (i % 4)) * kVs;
+#pragma unroll
+      for (int j = 0; j < HD / 32; ++j) {
+        o[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[32 * j], s[i], o[j], 0, 0, 0);
+      }
+    }
+    if (more) lstore(lds + ((t + 1) & 1) * kBuf);
+    __syncthreads();
+  }
+
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;     // no keys: zeros
+  if (q_ok) {
+    // accumulator i of block j: head dim 32 j + 8 (i / 4) + 4 half + i % 4
+    float* op = O + (q_begin + qrow) * ldo + (int64_t)h * HD + 4 * half;
+#pragma unroll
+    for (int j = 0; j < HD / 32; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4 v = {o[j][4 * g] * inv, o[j][4 * g + 1] * inv, o[j][4 * g + 2] * inv, o[j][4 * g + 3] * inv};
+        *reinterpret_cast<f32x4*>(op + 32 * j + 8 * g) = v;
+      }
+    }
+  }
+}
+
+template <int HD>
+static int launch_f32(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
+                      int64_t ldv, void* out, int64_t ldo, const int64_t* qo, const int64_t* kvo,
+                      int64_t B, int64_t H, int64_t max_q, float scale, hipStream_t s) {
+  dim3 grid((unsigned)((max_q + 127) / 128), (unsigned)H, (unsigned)B);
+  hipLaunchKernelGGL((varlen_attention_f32_kernel<HD>), grid, dim3(256), 0, s,
+                     static_cast<const float*>(q), ldq, static_cast<const float*>(k), ldk,
+                     static_cast<const float*>(v), ldv, static_cast<float*>(out), ldo, qo, kvo,
+                     scale * 1.4426950408889634f);
+  return check_launch("varlen_attention_f32_kernel");
+}
+
 template <typename T>
 static int launch_generic(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
                           int64_t ldv, void* out, int64_t ldo, const int64_t* qo,
@@ -783,6 +959,21 @@ extern "C" int nt_varlen_attention(const void* q, int64_t ldq, const void* k, in
   if (head_dim == kHd && dtype == NT_BF16) {
     return launch_mfma<__bf16>(q, ldq, k, ldk, v, ldv, out, ldo, q_offsets, kv_offsets, B,
                                num_heads, max_q_len, scale, s);
+  }
+  if (dtype == NT_F32 && (head_dim == 32 || head_dim == 64 || head_dim == 128) &&
+      ((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) % 16 == 0 &&
+      (ldq | ldk | ldv | ldo) % 4 == 0) {
+    // 16-byte row pieces: every row start must be 16-byte aligned
+    if (head_dim == 32) {
+      return launch_f32<32>(q, ldq, k, ldk, v, ldv, out, ldo, q_offsets, kv_offsets, B, num_heads,
+                            max_q_len, scale, s);
+    }
+    if (head_dim == 64) {
+      return launch_f32<64>(q, ldq, k, ldk, v, ldv, out, ldo, q_offsets, kv_offsets, B, num_heads,
+                            max_q_len, scale, s);
+    }
+    return launch_f32<128>(q, ldq, k, ldk, v, ldv, out, ldo, q_offsets, kv_offsets, B, num_heads,
+                           max_q_len, scale, s);
   }
   switch (dtype) {
     case NT_F32:

@@ -78,12 +78,13 @@ def test_min_mha_reference_shapes(dtype, H, B, Lmax, hd):
     assert got.nested_size() == nt.nested_tensor(xs).nested_size()
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("H,hd,lens", [(8, 32, (1, 64, 65, 300, 129)), (4, 128, (130, 7, 257, 64)),
                                        (2, 32, (513,)), (3, 128, (1, 2, 3)),
                                        (3, 32, (70, 200))])     # E = 96: not a multiple of the fused tile
 def test_mfma_attention_head_dims_32_and_128(dtype, H, hd, lens):
-    """head_dim 32 and 128 take the same MFMA kernel as 64 (self- and cross-attention)."""
+    """head_dim 32 and 128 take the same MFMA kernels as 64 (self- and cross-attention);
+    fp32 runs on the fp32 matrix instruction."""
     E = H * hd
     amp = 0.5 if dtype == torch.bfloat16 else 1.0
     xs, W_in, b_in, W_out, b_out = make_case(E, list(lens), 23, dtype, w_std=E ** -0.5, bias_std=0.1, x_std=amp)
@@ -103,11 +104,11 @@ def test_mfma_attention_head_dims_32_and_128(dtype, H, hd, lens):
     check(got, exp, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("hd", [32, 64, 128])
-def test_mfma_attention_boundary_lengths(hd):
-    """Every length around the 32-row wavefront blocks, the 64-key tiles and the
-    128-row query tiles, in one batch, as queries and (rotated) as keys."""
-    dtype = torch.float16
+def test_mfma_attention_boundary_lengths(hd, dtype):
+    """Every length around the 32-row wavefront blocks, the 32- and 64-key tiles and
+    the 128-row query tiles, in one batch, as queries and (rotated) as keys."""
     H = 2
     E = H * hd
     lens = [1, 2, 31, 32, 33, 63, 64, 65, 95, 96, 97, 127, 128, 129, 191, 192, 193, 255, 256, 257]
