@@ -165,6 +165,17 @@ def dtype_code(dtype):
     raise RuntimeError("nestedtensor_amd: dtype %s is not supported by this op" % dtype)
 
 
+def staging_device(what):
+    """The device that host (CPU) nested tensors are staged through: the current
+    HIP device.  There is no host implementation of the path; without a GPU the
+    conversion fails here."""
+    if not torch.cuda.is_available():
+        raise RuntimeError(
+            "nestedtensor_amd: %s of a host tensor is staged through the HIP device, "
+            "and no device is visible." % what)
+    return torch.device("cuda", torch.cuda.current_device())
+
+
 def require_device(t, what):
     if not t.is_cuda:
         raise RuntimeError(

@@ -113,20 +113,20 @@ def nested_tensor_impl(data, dtype, device, requires_grad, pin_memory, channels_
 
 def nested_tensor(data, dtype=None, device=None, requires_grad=False, pin_memory=False,
                   channels_last=False):
-    """
-    Arguments match torch.tensor
-    """
-    if dtype is None:
-        dtype = torch.get_default_dtype()
-    if device is None:
-        device = torch.device('cpu')
-    if channels_last is None:
-        channels_last = False
-    return nested.NestedTensor(
-        nested_tensor_impl(data, dtype, device, requires_grad, pin_memory, channels_last))
+    """A NestedTensor that owns a packed copy of the tensors in ``data``.  Keyword
+    arguments are those of torch.tensor (nested/creation.py:9-19): dtype defaults
+    to torch's default dtype, device to the host; channels_last=None means False."""
+    impl = nested_tensor_impl(
+        data,
+        torch.get_default_dtype() if dtype is None else dtype,
+        torch.device("cpu") if device is None else device,
+        requires_grad, pin_memory, bool(channels_last))
+    return nested.NestedTensor(impl)
 
 
 def as_nested_tensor(data, dtype=None, device=None, requires_grad=False, pin_memory=False):
-    if not isinstance(data, nested.NestedTensor):
-        return nested_tensor(data, dtype, device, requires_grad, pin_memory)
-    return data
+    """``data`` itself when it already is a NestedTensor (the other arguments are
+    then ignored, nested/creation.py:22-26); otherwise nested_tensor(...)."""
+    if isinstance(data, nested.NestedTensor):
+        return data
+    return nested_tensor(data, dtype, device, requires_grad, pin_memory)

@@ -27,51 +27,54 @@ _from_tensor_mask_lowered = _C.ops.from_tensor_mask_lowered.default
 _from_padded_value_lowered = _C.ops.from_padded_value_lowered.default
 
 
+def _check_dense_arguments(tensor, nested_dim, mask=None, with_mask=False):
+    """The argument errors of the reference's entry point (nested/masking.py:18-41),
+    in its order and wording; one table, walked until the first that applies."""
+    checks = [(tensor is None, "Tensor can't be undefined (None).")]
+    if with_mask:
+        checks.append((mask is None, "Mask can't be undefined (None)."))
+    for failed, message in checks:
+        if failed:
+            raise RuntimeError(message)
+    rank = tensor.dim()
+    checks = [
+        (rank == 0, "Can't construct nested tensor from a scalar."),
+        (nested_dim == 0, "Nested dimension can't be 0."),
+        (nested_dim is not None and nested_dim != 0 and nested_dim > rank,
+         "Nested dimension ({0}) can't be bigger than data tensor dimension ({1}).".format(nested_dim, rank)),
+    ]
+    if with_mask:
+        n_data, n_mask = tensor.numel(), mask.numel()
+        checks.append((n_data == 0 and n_mask != 0, "Data tensor can't be emtpy if a mask has values."))
+        checks.append((n_data != 0 and n_mask == 0, "Mask tensor can't be emtpy if a data tensor has values."))
+    for failed, message in checks:
+        if failed:
+            raise RuntimeError(message)
+
+
+def _on_host(nested_result):
+    impl = nested_result._impl
+    return nested.NestedTensor(impl.with_buffer(impl.buffer.cpu()))
+
+
 def nested_tensor_from_padded_tensor(tensor, nested_dim=1, padding=-1):
     """``nested_tensor_from_tensor_mask(tensor, tensor != padding, nested_dim)``
     (nested/masking.py:12-14).  On the device the mask is never materialised: the
-    keep-counts are taken straight from the data (nt_value_row_counts)."""
-    if tensor is None:
-        raise RuntimeError("Tensor can't be undefined (None).")
-    if tensor.dim() == 0:
-        raise RuntimeError("Can't construct nested tensor from a scalar.")
-    if nested_dim == 0:
-        raise RuntimeError("Nested dimension can't be 0.")
-    if nested_dim is not None and nested_dim > tensor.dim():
-        raise RuntimeError("Nested dimension ({0}) can't be bigger than data tensor dimension ({1}).".format(
-            nested_dim, tensor.dim()))
-    if not tensor.is_cuda or tensor.dim() < 2 or tensor.numel() < 2 or tensor.dtype not in _C.ELEM_TYPE:
-        mask = (tensor != padding)
-        return nested_tensor_from_tensor_mask(tensor, mask, nested_dim)
+    keep-counts are taken straight from the data (nt_value_row_counts).  A host
+    tensor is staged through the device and the result returned to the host."""
+    _check_dense_arguments(tensor, nested_dim)
+    if not tensor.is_cuda:
+        staged = tensor.to(_C.staging_device("nested_tensor_from_padded_tensor"))
+        return _on_host(nested_tensor_from_padded_tensor(staged, nested_dim, padding))
+    if tensor.dim() < 2 or tensor.numel() < 2 or tensor.dtype not in _C.ELEM_TYPE:
+        return nt_from_tensor_mask(tensor, tensor != padding, nested_dim)
     return _wrap_lowered(*_from_padded_value_lowered(tensor, float(padding), nested_dim))
 
 
-# Constructs nested tensor from passed tensor and mask.
 def nested_tensor_from_tensor_mask(tensor, mask, nested_dim=1):
-    if tensor is None:
-        raise RuntimeError("Tensor can't be undefined (None).")
-
-    if mask is None:
-        raise RuntimeError("Mask can't be undefined (None).")
-
-    # Scalar was passed
-    if tensor.dim() == 0:
-        raise RuntimeError("Can't construct nested tensor from a scalar.")
-
-    if nested_dim == 0:
-        raise RuntimeError("Nested dimension can't be 0.")
-
-    if nested_dim is not None and nested_dim > tensor.dim():
-        raise RuntimeError("Nested dimension ({0}) can't be bigger than data tensor dimension ({1}).".format(
-            nested_dim, tensor.dim()))
-
-    if tensor.numel() == 0 and mask.numel() != 0:
-        raise RuntimeError("Data tensor can't be emtpy if a mask has values.")
-
-    if tensor.numel() != 0 and mask.numel() == 0:
-        raise RuntimeError(
-            "Mask tensor can't be emtpy if a data tensor has values.")
-
+    """The nested tensor of the entries of ``tensor`` that ``mask`` keeps
+    (nested/masking.py:17-43)."""
+    _check_dense_arguments(tensor, nested_dim, mask, with_mask=True)
     return nt_from_tensor_mask(tensor, mask, nested_dim)
 
 
@@ -85,6 +88,9 @@ def _wrap_lowered(buffer, sizes, sizes_dev, offsets_dev):
 
 
 def nt_from_tensor_mask(tensor, mask, nested_dim):
+    if not tensor.is_cuda and mask.numel() > 1:      # smaller masks are answered on the host
+        dev = _C.staging_device("nested_tensor_from_tensor_mask")
+        return _on_host(nt_from_tensor_mask(tensor.to(dev), mask.to(dev), nested_dim))
     return _wrap_lowered(*_from_tensor_mask_lowered(tensor, mask, nested_dim))
 
 

@@ -61,6 +61,30 @@ def _check_no_empty(impl):
 
 
 # ---------------------------------------------------------------------------
+# host nested tensors
+#
+# The reference serves nested tensors in host memory with CPU loops
+# (masking.cpp:297-319, 511-532, 627-649).  Here the conversions exist on the
+# device only; a nested tensor whose buffer lies in host memory is staged: the
+# packed buffer goes to the current device, the device path runs, and the dense
+# results come back to the host.  Same results, two extra copies.
+
+
+def _to_host(result):
+    if isinstance(result, tuple):
+        return tuple(_to_host(r) for r in result)
+    return result.cpu() if torch.is_tensor(result) else result
+
+
+def _stage(impl, what, with_data=True):
+    """Device twin of a host nested tensor: the packed buffer copied to the
+    current device (or, when only the nested size is needed, an empty buffer)."""
+    dev = _C.staging_device(what)
+    buf = impl.buffer.to(dev) if with_data else torch.empty(0, dtype=impl.buffer.dtype, device=dev)
+    return impl.with_buffer(buf)
+
+
+# ---------------------------------------------------------------------------
 # packed -> padded
 
 
@@ -69,7 +93,8 @@ def add_padding(impl, padding, with_mask=False, shape=None):
     [B] + shape for a caller-given shape that holds every constituent).  With
     with_mask, nt_add_padding_mask writes the bool mask of the same shape in the
     same launch and (padded, mask) is returned."""
-    _C.require_device(impl.buffer, "to_padded_tensor")
+    if not impl.buffer.is_cuda:
+        return _to_host(add_padding(_stage(impl, "to_padded_tensor"), padding, with_mask, shape))
     B, D = impl.B, impl.D
     max_size = impl.max_sizes()
     nrag = _n_ragged(impl)
@@ -171,7 +196,8 @@ def build_mask(impl, kept_dims):
         return torch.tensor(True, device=dev)
     if kept_dims == 1:
         return torch.ones(impl.B, dtype=torch.bool, device=dev)
-    _C.require_device(impl.buffer, "to_tensor_mask")
+    if not impl.buffer.is_cuda:
+        return _to_host(build_mask(_stage(impl, "to_mask", with_data=False), kept_dims))
     K = kept_dims - 1
     if K > 3:
         raise RuntimeError("masks over more than 3 constituent dimensions are not supported.")
@@ -247,7 +273,10 @@ def from_padded_tensor(padded, target):
     whose nested size the result takes."""
     if padded.dim() != target.dim():
         raise RuntimeError("Target size has different dimension as input padded Tensor.")
-    _C.require_device(padded, "from_padded_tensor")
+    if not padded.is_cuda:
+        # a host tensor: staged through the device, the packed result comes back
+        res = from_padded_tensor(padded.to(_C.staging_device("from_padded_tensor")), target)
+        return res.with_buffer(res.buffer.cpu())
     padded = padded.contiguous()
     B, D = target.B, target.D
     if padded.size(0) != B:

@@ -572,3 +572,33 @@ def test_from_padded_tensor_compares_in_the_tensors_own_type(dtype, padding):
     got = nt.nested_tensor_from_padded_tensor(padded.to(DEV), padding=padding)
     exp = oracle.nested_tensor_from_tensor_mask(padded, mask)
     nt_matches(got, exp.unbind(), dtype)
+
+
+# ---- nested tensors in host memory: staged through the device -----------------
+
+def test_host_nested_tensors_are_staged_through_the_device():
+    # the reference's default device is the host (nested/creation.py:15-16); its
+    # conversions there are CPU loops (masking.cpp:297-319, 511-532, 627-649)
+    g = torch.Generator().manual_seed(77)
+    parts = [torch.randn(int(l), 5, generator=g) for l in (3, 1, 7, 4)]
+    a = nt.nested_tensor(parts)
+    assert a.device.type == "cpu"
+    ref = oracle.ref_nested_tensor(parts)
+    padded = a.to_padded_tensor(-2.0)
+    assert padded.device.type == "cpu" and torch.equal(padded, oracle.to_padded_tensor(ref, -2.0))
+    t, m = a.to_tensor_mask()
+    exp_t, exp_m = oracle.to_tensor_mask(ref)
+    assert t.device.type == "cpu" and m.device.type == "cpu"
+    assert torch.equal(t, exp_t) and torch.equal(m, exp_m.to(torch.bool))
+    for md in (2, 3):
+        got = torch.ops.nestedtensor.to_mask(a, md)
+        assert got.device.type == "cpu" and torch.equal(got, oracle.to_mask(ref, md).to(torch.bool))
+    back = nt.nested_tensor_from_tensor_mask(t, m)
+    assert back.device.type == "cpu" and torch.equal(back._impl.buffer, ref.buffer)
+    assert back.nested_size() == a.nested_size()
+    back = nt.nested_tensor_from_padded_tensor(padded, padding=-2.0)
+    assert back.device.type == "cpu" and torch.equal(back._impl.buffer, ref.buffer)
+    back = nt.from_padded_tensor(padded, a)
+    assert back.device.type == "cpu" and torch.equal(back._impl.buffer, ref.buffer)
+    back = nt.from_padded_tensor(padded, a.nested_size())
+    assert torch.equal(back._impl.buffer, ref.buffer)

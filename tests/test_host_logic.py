@@ -173,14 +173,25 @@ def test_from_tensor_mask_host_only_cases():
     assert len(r) == 0
 
 
-def test_compute_ops_refuse_host_tensors():
+def test_host_tensors_need_the_device():
+    # conversions of host nested tensors are staged through the device; compute ops
+    # want the nested tensor moved first.  Nothing falls back to host arithmetic:
+    # without a visible device every one of them raises.
+    if torch.cuda.is_available():
+        pytest.skip("a device is visible: staging is covered by the device tests")
     a = nt.nested_tensor([torch.randn(2, 3), torch.randn(4, 3)])
-    with pytest.raises(RuntimeError, match="HIP device only"):
+    with pytest.raises(RuntimeError, match="staged through the HIP device"):
         a.to_padded_tensor(0)
-    with pytest.raises(RuntimeError, match="HIP device only"):
+    with pytest.raises(RuntimeError, match="staged through the HIP device"):
         a.to_tensor_mask()
-    with pytest.raises(RuntimeError, match="HIP device only"):
+    with pytest.raises(RuntimeError, match="staged through the HIP device"):
+        torch.ops.nestedtensor.to_mask(a, 2)
+    with pytest.raises(RuntimeError, match="staged through the HIP device"):
         nt.nested_tensor_from_tensor_mask(torch.randn(2, 3), torch.ones(2, 3, dtype=torch.bool))
+    with pytest.raises(RuntimeError, match="staged through the HIP device"):
+        nt.nested_tensor_from_padded_tensor(torch.randn(2, 3), padding=0)
+    with pytest.raises(RuntimeError, match="staged through the HIP device"):
+        nt.from_padded_tensor(torch.randn(2, 4, 3), a)
     mha = torch.nn.MultiheadAttention(3, 1).eval()
     with pytest.raises(RuntimeError, match="HIP device only"):
         mha(a, a, a)
