@@ -246,15 +246,17 @@ def pmc_probe(args, torch, dev):
 
 def mha_probe(args, torch, dev):
     """Dispatches for kernel-trace and hardware-counter runs of the attention
-    layers: min_mha on C3 (fp16) twice, bt_min_mha on C4 (bf16) twice, and
-    torch.addmm (the vendor GEMM) on C3's two projection shapes twice.  Prints
-    the shapes and flop counts the counters are to be set against."""
+    layers: min_mha on C3 (fp16) twice, torch.addmm (the vendor GEMM) on C3's two
+    projection shapes twice, bt_min_mha on C4 (bf16) twice and min_mha on C3 in
+    fp32 twice.  Prints the shapes and flop counts the counters are to be set
+    against."""
     import nestedtensor_amd as nt
     out = {}
     for tag, seed, B, E, H, dtype in (("C3", 1010 + 2, 32, 768, 12, torch.float16),
-                                      ("C4", 1010 + 3, 128, 1024, 16, torch.bfloat16)):
+                                      ("C4", 1010 + 3, 128, 1024, 16, torch.bfloat16),
+                                      ("C3_fp32", 1010 + 2, 32, 768, 12, torch.float32)):
         g = torch.Generator().manual_seed(seed)
-        if tag == "C3":
+        if tag != "C4":
             lens = [int(v) for v in torch.randint(32, 513, (B,), generator=g)]
         else:
             lens = [int(v) for v in torch.empty(B).exponential_(1.0 / 96.0, generator=g).round().clamp(8, 512)]
@@ -263,7 +265,7 @@ def mha_probe(args, torch, dev):
         W_out = (torch.randn(E, E, generator=g) * 0.02).to(dtype).to(dev)
         b_in, b_out = torch.zeros(3 * E, dtype=dtype, device=dev), torch.zeros(E, dtype=dtype, device=dev)
         a = nt.nested_tensor(xs, device=dev, dtype=dtype)
-        op = torch.ops.nestedtensor.min_mha if tag == "C3" else torch.ops.nestedtensor.bt_min_mha
+        op = torch.ops.nestedtensor.bt_min_mha if tag == "C4" else torch.ops.nestedtensor.min_mha
         torch.cuda.synchronize()
         for _ in range(2):
             op(H, 64, 0.0, False, a, a, a, W_in, b_in, 64 ** -0.5, W_out, b_out)
@@ -544,6 +546,14 @@ def bench_rows(args, torch, dev, later):
         note="includes the device-to-host copy of the row counts; CPU figure is the vectorised "
              "restatement, the reference's literal walk does one host call per mask element")
     rows["C2_nested_tensor_pack_from_device_tensors"] = entry(ms_pack, 2 * 4 * nvalid2)
+    # for scale: torch's own device copy of the padded tensor and fill of the mask
+    # (a plain copy / fill of the same bytes, no ragged structure)
+    data2 = torch.empty_like(data)
+    ms_cp = _time_gpu(torch, lambda: data2.copy_(data))
+    ms_fill = _time_gpu(torch, lambda: mask.fill_(True))
+    rows["C2_plain_copy_of_padded_bytes_torch"] = entry(ms_cp, 2 * 4 * npadded2)
+    rows["C2_plain_fill_of_mask_bytes_torch"] = entry(ms_fill, npadded2)
+    del data2
     if cpu:
         ref2 = oracle.ref_nested_tensor(imgs)
         dcpu, mcpu = data.cpu(), mask.cpu()
