@@ -22,6 +22,7 @@
 #include <c10/hip/HIPStream.h>
 #include <torch/library.h>
 
+#include <algorithm>
 #include <cstring>
 #include <tuple>
 #include <vector>
@@ -731,6 +732,137 @@ Tensor mha_self_packed(const Tensor& x, const Tensor& schedule, int64_t num_head
   return out;
 }
 
+// ---- consumers of the offsets array ---------------------------------------------
+
+// After a kernel that may have counted out-of-range indices: the running count
+// goes to its pinned host mirror with an asynchronous copy on the same stream (a
+// copy node when the stream is being captured).  Nothing waits for it here.
+void mirror_counter(const c10::optional<Tensor>& counter, const c10::optional<Tensor>& mirror, void* stream) {
+  if (!counter.has_value() || !counter->defined() || !mirror.has_value() || !mirror->defined()) return;
+  TORCH_CHECK(mirror->is_pinned() && mirror->numel() >= 1 && mirror->scalar_type() == at::kInt,
+              "index counter mirror must be a pinned int32 tensor");
+  C10_HIP_CHECK(hipMemcpyAsync(mirror->data_ptr(), counter->const_data_ptr(), 4, hipMemcpyDeviceToHost,
+                               static_cast<hipStream_t>(stream)));
+}
+
+int32_t* counter_ptr(const c10::optional<Tensor>& counter, const Tensor& like) {
+  if (!counter.has_value() || !counter->defined()) return nullptr;
+  TORCH_CHECK(counter->scalar_type() == at::kInt && counter->numel() >= 1 && counter->device() == like.device(),
+              "index counter must be an int32 tensor on the device of the table");
+  return counter->data_ptr<int32_t>();
+}
+
+// NestedTensor_embedding (functions.cpp:14-63) on the packed index buffer: one
+// gather (nt_gather_rows), result [T, E].  Out-of-range indices give zero rows
+// and are added to `counter` (device int32[1]) when one is passed.
+Tensor embedding_packed(const Tensor& weight_in, const Tensor& indices, const c10::optional<Tensor>& counter,
+                        const c10::optional<Tensor>& mirror) {
+  require_device(indices, "embedding");
+  TORCH_CHECK(weight_in.dim() == 2, "'weight' must be 2-D");
+  TORCH_CHECK(indices.scalar_type() == at::kLong || indices.scalar_type() == at::kInt,
+              "Expected tensor for argument #1 'indices' to have one of the following scalar types: Long, Int; "
+              "but got ", indices.scalar_type(), " instead");
+  TORCH_CHECK(weight_in.device() == indices.device(), "embedding: weight and indices must be on the same device");
+  const Tensor weight = weight_in.contiguous();
+  const Tensor idx = indices.scalar_type() == at::kLong ? indices.contiguous() : indices.to(at::kLong);
+  const int64_t V = weight.size(0), E = weight.size(1), T = idx.numel();
+  c10::hip::HIPGuard guard(weight.device().index());
+  void* stream = stream_of(weight);
+  Tensor out = at::empty({T, E}, weight.options());
+  check(nt_gather_rows(weight.const_data_ptr(), V, E * static_cast<int64_t>(weight.element_size()),
+                       idx.const_data_ptr<int64_t>(), out.data_ptr(), T, counter_ptr(counter, weight), stream));
+  mirror_counter(counter, mirror, stream);
+  return out;
+}
+
+// _nn_functional_embedding_bag (nested/nested.py:43-118): the bags are the
+// constituents, `offsets` the nested tensor's device offsets.  mode: 0 sum, 1 mean, 2 max.
+Tensor embedding_bag_packed(const Tensor& weight_in, const Tensor& indices, const Tensor& offsets, int64_t mode,
+                            const c10::optional<Tensor>& counter, const c10::optional<Tensor>& mirror) {
+  require_device(indices, "embedding_bag");
+  TORCH_CHECK(weight_in.dim() == 2 && weight_in.device() == indices.device(),
+              "embedding_bag: weight must be 2-D on the device of the indices");
+  TORCH_CHECK(offsets.scalar_type() == at::kLong && offsets.numel() >= 1 && offsets.device() == indices.device() &&
+                  offsets.is_contiguous(),
+              "embedding_bag: offsets must be a contiguous int64 tensor on the device of the indices");
+  const Tensor weight = weight_in.contiguous();
+  const Tensor idx = indices.scalar_type() == at::kLong ? indices.contiguous() : indices.to(at::kLong);
+  const int64_t V = weight.size(0), E = weight.size(1), B = offsets.numel() - 1;
+  c10::hip::HIPGuard guard(weight.device().index());
+  void* stream = stream_of(weight);
+  Tensor out = at::empty({B, E}, weight.options());
+  check(nt_embedding_bag(weight.const_data_ptr(), E, V, idx.const_data_ptr<int64_t>(), idx.numel(),
+                         offsets.const_data_ptr<int64_t>(), out.data_ptr(), B, E, static_cast<int>(mode),
+                         dtype_code(weight.scalar_type()), counter_ptr(counter, weight), stream));
+  mirror_counter(counter, mirror, stream);
+  return out;
+}
+
+// NestedTensor.to_packed_sequence (nested/nested.py:484-488) without the unbind:
+// the order of torch.nn.utils.rnn.pack_sequence(..., enforce_sorted=False).
+// lengths: host int64 [B] (all > 0); row_offsets: device token offsets [B + 1];
+// buffer viewed as [T, row_elems].  The three small index arrays are derived here
+// from the lengths (a sort of B numbers) and reach the device in one copy
+// from pinned memory; the row order is then built on the device
+// (nt_packed_sequence_index) and the rows moved by one gather.  Returns (data
+// [T, row_elems], batch_sizes (host), sorted_indices, unsorted_indices (device)).
+std::tuple<Tensor, Tensor, Tensor, Tensor> packed_sequence_lowered(const Tensor& buffer, const Tensor& lengths,
+                                                                   const Tensor& row_offsets, int64_t row_elems) {
+  require_device(buffer, "to_packed_sequence");
+  TORCH_CHECK(lengths.device().is_cpu() && lengths.scalar_type() == at::kLong && lengths.dim() == 1 &&
+                  lengths.is_contiguous(),
+              "to_packed_sequence: lengths must be a contiguous host int64 vector");
+  const int64_t B = lengths.numel();
+  TORCH_CHECK(B > 0 && row_offsets.numel() == B + 1 && row_offsets.scalar_type() == at::kLong &&
+                  row_offsets.device() == buffer.device() && row_offsets.is_contiguous(),
+              "to_packed_sequence: row offsets must be a contiguous int64 [B + 1] tensor on the buffer's device");
+  const int64_t* len = lengths.const_data_ptr<int64_t>();
+  int64_t T = 0, Lmax = 0;
+  for (int64_t b = 0; b < B; ++b) {
+    TORCH_CHECK(len[b] > 0, "Length of all samples has to be greater than 0, but found an element in "
+                            "'lengths' that is <= 0");
+    T += len[b];
+    Lmax = std::max(Lmax, len[b]);
+  }
+  TORCH_CHECK(buffer.numel() == T * row_elems, "to_packed_sequence: buffer does not hold ", T, " rows of ", row_elems);
+  // decreasing length, ties as torch.sort leaves them: the same call that
+  // torch.nn.utils.rnn.pack_padded_sequence(enforce_sorted=False) makes, so the
+  // permutation is the reference's also where lengths repeat
+  const Tensor order_t = std::get<1>(lengths.sort(/*dim=*/-1, /*descending=*/true)).contiguous();
+  const int64_t* order = order_t.const_data_ptr<int64_t>();
+  Tensor batch_sizes = at::empty({Lmax}, at::kLong);
+  int64_t* bs = batch_sizes.data_ptr<int64_t>();
+  const int64_t n = 2 * B + Lmax;
+  Tensor host = at::empty({n}, at::TensorOptions().dtype(at::kLong).pinned_memory(true));
+  int64_t* rank = host.data_ptr<int64_t>();
+  int64_t* sorted = rank + B;
+  int64_t* starts = sorted + B;
+  for (int64_t r = 0; r < B; ++r) {
+    sorted[r] = order[r];
+    rank[order[r]] = r;
+  }
+  // batch_sizes[t] = number of sequences longer than t: walk the sorted lengths from the short end
+  int64_t alive = B, acc = 0;
+  for (int64_t t = 0; t < Lmax; ++t) {
+    while (alive > 0 && len[order[alive - 1]] <= t) --alive;
+    bs[t] = alive;
+    starts[t] = acc;
+    acc += alive;
+  }
+  c10::hip::HIPGuard guard(buffer.device().index());
+  void* stream = stream_of(buffer);
+  Tensor meta = at::empty({n}, buffer.options().dtype(at::kLong));
+  meta.copy_(host, /*non_blocking=*/true);
+  Tensor rank_dev = meta.narrow(0, 0, B), sorted_dev = meta.narrow(0, B, B), starts_dev = meta.narrow(0, 2 * B, Lmax);
+  Tensor index = at::empty({T}, buffer.options().dtype(at::kLong));
+  Tensor data = at::empty({T, row_elems}, buffer.options());
+  check(nt_packed_sequence_index(row_offsets.const_data_ptr<int64_t>(), rank_dev.const_data_ptr<int64_t>(),
+                                 starts_dev.const_data_ptr<int64_t>(), B, T, index.data_ptr<int64_t>(), stream));
+  check(nt_gather_rows(buffer.const_data_ptr(), T, row_elems * static_cast<int64_t>(buffer.element_size()),
+                       index.const_data_ptr<int64_t>(), data.data_ptr(), T, nullptr, stream));
+  return std::make_tuple(data, batch_sizes, sorted_dev, rank_dev);
+}
+
 }  // namespace
 
 // Schemas.  The first block are the reference's operators, names and argument
@@ -780,6 +912,11 @@ TORCH_LIBRARY(nestedtensor, m) {
   m.def("build_mask(Tensor sizes, int[] extents) -> Tensor");
   m.def("from_tensor_mask_lowered(Tensor tensor, Tensor mask, int nested_dim) -> (Tensor, Tensor, Tensor, Tensor)");
   m.def("from_padded_value_lowered(Tensor tensor, float padding, int nested_dim) -> (Tensor, Tensor, Tensor, Tensor)");
+  m.def("embedding_packed(Tensor weight, Tensor indices, Tensor? counter, Tensor? mirror) -> Tensor");
+  m.def("embedding_bag_packed(Tensor weight, Tensor indices, Tensor offsets, int mode, Tensor? counter, "
+        "Tensor? mirror) -> Tensor");
+  m.def("packed_sequence_lowered(Tensor buffer, Tensor lengths, Tensor row_offsets, int row_elems) -> "
+        "(Tensor, Tensor, Tensor, Tensor)");
   m.def("linear_packed(Tensor x, Tensor weight, Tensor? bias, int act) -> Tensor");
   m.def("mha_self_packed(Tensor x, Tensor schedule, int num_heads, int head_dim, Tensor in_proj_weight, "
         "Tensor? in_proj_bias, float scaling, Tensor out_proj_weight, Tensor? out_proj_bias) -> Tensor");
@@ -797,6 +934,9 @@ TORCH_LIBRARY_IMPL(nestedtensor, CUDA, m) {
   m.impl("nt_from_padded_tensor", nt_from_padded_tensor_op);
   m.impl("linear_packed", linear_packed);
   m.impl("mha_self_packed", mha_self_packed);
+  m.impl("embedding_packed", embedding_packed);
+  m.impl("embedding_bag_packed", embedding_bag_packed);
+  m.impl("packed_sequence_lowered", packed_sequence_lowered);
 }
 
 // Operators on plain tensors of any device: merge_tensor_mask is host logic over

@@ -27,6 +27,9 @@ _remove_padding = _C.ops.remove_padding.default
 _build_mask = _C.ops.build_mask.default
 _linear_packed = _C.ops.linear_packed.default
 _mha_self_packed = _C.ops.mha_self_packed.default
+_embedding_packed = _C.ops.embedding_packed.default
+_embedding_bag_packed = _C.ops.embedding_bag_packed.default
+_packed_sequence_lowered = _C.ops.packed_sequence_lowered.default
 
 
 _ELEM_BYTES = {}
@@ -786,20 +789,18 @@ def check_index_errors(synchronize=True):
 
 
 def _oob_begin(device, what):
-    """Counter pointer for a launch (None when checks are off); in deferred mode
-    reports what earlier calls have left."""
+    """The device's counter slot for a launch (None when checks are off); in
+    deferred mode reports what earlier calls have left.  The operator adds to the
+    counter and copies it to the pinned mirror on its stream."""
     if _index_check_mode == "off":
-        return None, None
+        return None
     slot = _index_counter(device)
     if _index_check_mode == "deferred" and not torch.cuda.is_current_stream_capturing():
         _report_index_errors(slot, what + " (an earlier call)")
-    return slot, _C.ptr(slot[0])
+    return slot
 
 
 def _oob_end(slot, what):
-    if slot is None:
-        return
-    slot[1].copy_(slot[0], non_blocking=True)
     if _index_check_mode == "immediate":
         torch.cuda.current_stream(slot[0].device).synchronize()
         _report_index_errors(slot, what)
@@ -825,16 +826,14 @@ def embedding(weight, indices, padding_idx=None, max_norm=None, norm_type=2.0,
                            "types: Long, Int; but got %s instead" % idx.dtype)
     if weight.device != idx.device:
         raise RuntimeError("embedding: weight and indices must be on the same device")
-    weight = weight.contiguous()
-    idx64 = idx.to(torch.int64)
-    V, E = weight.shape
-    out = torch.empty(idx.numel() * E, dtype=weight.dtype, device=weight.device)
-    slot, oob = _oob_begin(weight.device, "embedding")
-    with _C.on_device(weight.device):
-        _C.check(_C.lib.nt_gather_rows(_C.ptr(weight), V, E * weight.element_size(), _C.ptr(idx64),
-                                       _C.ptr(out), idx.numel(), oob,
-                                       _C.current_stream(weight.device)))
+    E = weight.size(1)
+    slot = _oob_begin(weight.device, "embedding")
+    if slot is None:
+        out = _embedding_packed(weight, idx, None, None)
+    else:
+        out = _embedding_packed(weight, idx, slot[0], slot[1])
         _oob_end(slot, "embedding")
+    out = out.reshape(-1)
     if indices.sizes.dim() == 0:
         sizes = indices.sizes
     else:
@@ -876,18 +875,11 @@ def embedding_bag(input, weight, offsets=None, max_norm=None, norm_type=2, scale
     _C.require_device(idx, "embedding_bag")
     if weight.dim() != 2 or weight.device != idx.device:
         raise RuntimeError("embedding_bag: weight must be 2-D on the device of the indices")
-    weight = weight.contiguous()
-    idx64 = idx.to(torch.int64)
-    V, E = weight.shape
-    B = input.B
-    out = torch.empty((B, E), dtype=weight.dtype, device=weight.device)
-    slot, oob = _oob_begin(weight.device, "embedding_bag")
-    with _C.on_device(weight.device):
-        _C.check(_C.lib.nt_embedding_bag(_C.ptr(weight), E, V, _C.ptr(idx64), idx64.numel(),
-                                         _C.ptr(input.offsets_dev()),
-                                         _C.ptr(out), B, E, modes[mode], _C.dtype_code(weight.dtype),
-                                         oob, _C.current_stream(weight.device)))
-        _oob_end(slot, "embedding_bag")
+    slot = _oob_begin(weight.device, "embedding_bag")
+    if slot is None:
+        return _embedding_bag_packed(weight, idx, input.offsets_dev(), modes[mode], None, None)
+    out = _embedding_bag_packed(weight, idx, input.offsets_dev(), modes[mode], slot[0], slot[1])
+    _oob_end(slot, "embedding_bag")
     return out
 
 
@@ -923,33 +915,14 @@ def to_packed_sequence(impl):
     if impl.has_empty_constituent():
         raise RuntimeError("Length of all samples has to be greater than 0, but found an element in "
                            "'lengths' that is <= 0")
-    lengths = impl.sizes[:, 0].contiguous()
-    # as torch.nn.utils.rnn.pack_padded_sequence(enforce_sorted=False) orders them
-    sorted_lengths, sorted_indices = torch.sort(lengths, descending=True)
-    B, Lmax = impl.B, int(sorted_lengths[0])
-    unsorted_indices = torch.empty_like(sorted_indices)
-    unsorted_indices[sorted_indices] = torch.arange(B)
-    # batch_sizes[t] = number of sequences longer than t
-    batch_sizes = (lengths.unsqueeze(0) > torch.arange(Lmax).unsqueeze(1)).sum(1)
-    step_starts = torch.cumsum(batch_sizes, 0) - batch_sizes
-    dev = buf.device
     trailing = [int(v) for v in opt[2:]]
     row_elems = 1
     for v in trailing:
         row_elems *= v
-    T = int(lengths.sum())
-    index = torch.empty(T, dtype=torch.int64, device=dev)
-    data = torch.empty([T] + trailing, dtype=buf.dtype, device=dev)
-    # one upload for the three small index arrays
-    meta = torch.cat([unsorted_indices, sorted_indices, step_starts]).to(dev)
-    rank_dev, sorted_dev, starts_dev = meta[:B], meta[B:2 * B], meta[2 * B:]
-    with _C.on_device(dev):
-        stream = _C.current_stream(dev)
-        _C.check(_C.lib.nt_packed_sequence_index(_C.ptr(impl.row_offsets_dev()), _C.ptr(rank_dev),
-                                                 _C.ptr(starts_dev), B, T, _C.ptr(index), stream))
-        _C.check(_C.lib.nt_gather_rows(_C.ptr(buf), T, row_elems * buf.element_size(), _C.ptr(index),
-                                       _C.ptr(data), T, None, stream))
-    return torch.nn.utils.rnn.PackedSequence(data, batch_sizes, sorted_dev, rank_dev)
+    data, batch_sizes, sorted_dev, rank_dev = _packed_sequence_lowered(
+        buf, impl.sizes[:, 0].contiguous(), impl.row_offsets_dev(), row_elems)
+    return torch.nn.utils.rnn.PackedSequence(data.reshape([data.size(0)] + trailing), batch_sizes, sorted_dev,
+                                             rank_dev)
 
 
 # ---- channels-last ragged images: per-constituent transposes ------------------------
