@@ -658,10 +658,13 @@ def _pair(v):
     return (v[0], v[0]) if len(v) == 1 else v
 
 
-def _dense_via_padding(impl, pad_value, dense_op, out_channels, k, stride, padding, dilation):
+def _dense_via_padding(impl, pad_value, dense_op, out_channels, k, stride, padding, dilation, ceil_mode=False):
     """to_padded_tensor -> one dense call over the whole batch -> from_padded_tensor
     with the per-constituent output sizes
-    ``(s + 2 p - d (k - 1) - 1) // stride + 1`` (pooling.cpp:50-53, conv2d.cpp:80-84)."""
+    ``(s + 2 p - d (k - 1) - 1) // stride + 1`` (pooling.cpp:50-53, conv2d.cpp:80-84).
+    With ceil_mode the division rounds up and a last window that would start past
+    the input and its left padding is dropped, as ATen's pooling_output_shape does
+    for each constituent on the reference's per-constituent route (pooling.cpp:60-72)."""
     if impl.dim() != 4:
         raise RuntimeError("Input must be 4 dimensional.")
     _C.require_device(impl.buffer, "dense op on a NestedTensor")
@@ -673,7 +676,14 @@ def _dense_via_padding(impl, pad_value, dense_op, out_channels, k, stride, paddi
     if out_channels is not None:
         sizes[:, 0] = out_channels
     for j in (0, 1):
-        sizes[:, 1 + j] = (sizes[:, 1 + j] + 2 * padding[j] - dilation[j] * (k[j] - 1) - 1) // stride[j] + 1
+        extent = sizes[:, 1 + j]
+        span = extent + 2 * padding[j] - dilation[j] * (k[j] - 1) - 1
+        if ceil_mode:
+            out = torch.div(span + stride[j] - 1, stride[j], rounding_mode="floor") + 1
+            out = out - ((out - 1) * stride[j] >= extent + padding[j]).to(out.dtype)
+        else:
+            out = torch.div(span, stride[j], rounding_mode="floor") + 1
+        sizes[:, 1 + j] = out
     if bool((sizes <= 0).any()):
         raise RuntimeError("Output size is too small")
     target = NestedTensorImpl(torch.empty(0, dtype=result.dtype, device=result.device), sizes)
@@ -689,14 +699,18 @@ def max_pool2d(impl, kernel_size, stride=None, padding=0, dilation=1, ceil_mode=
     pad value is -inf, which makes the result equal to pooling each constituent on
     its own (what the reference's tests assert) also for windows that reach past a
     constituent's edge."""
-    if ceil_mode or return_indices:
-        raise NotImplementedError("max_pool2d on a NestedTensor: ceil_mode / return_indices are not supported.")
+    if return_indices:
+        # not part of the reference's operator either (pooling.cpp:34-40)
+        raise NotImplementedError("max_pool2d on a NestedTensor: return_indices is not supported.")
     k = _pair(kernel_size)
     s = _pair(stride) if stride not in (None, [], ()) else k
     p, d = _pair(padding), _pair(dilation)
+    # ceil_mode: a window that reaches past a constituent's edge sees -inf there, in
+    # the padded batch as in the constituent pooled on its own
     return _dense_via_padding(
         impl, float("-inf"),
-        lambda x: torch.nn.functional.max_pool2d(x, k, s, p, d, False), None, k, s, p, d)
+        lambda x: torch.nn.functional.max_pool2d(x, k, s, p, d, bool(ceil_mode)), None, k, s, p, d,
+        ceil_mode=bool(ceil_mode))
 
 
 def conv2d(impl, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):

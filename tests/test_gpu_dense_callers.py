@@ -34,6 +34,22 @@ def test_max_pool2d_equals_per_constituent(shapes, dtype):
     assert torch.equal(pool(a)._impl.buffer.cpu(), exp.buffer)
 
 
+@pytest.mark.parametrize("k,s,p,d", [((3, 3), (2, 2), (1, 1), (1, 1)), ((2, 2), (2, 2), (0, 0), (1, 1)),
+                                     ((3, 2), (3, 2), (1, 0), (1, 1)), ((3, 3), (2, 3), (1, 1), (2, 1))])
+def test_max_pool2d_ceil_mode_equals_per_constituent(k, s, p, d):
+    # pooling.cpp:60-72: the per-constituent route passes ceil_mode on; odd and even
+    # extents so that some last windows reach past the edge and some are dropped
+    shapes = [(2, 7, 5), (2, 3, 9), (2, 8, 8), (2, 6, 10), (2, 13, 4), (2, 5, 5)]
+    ts = [t - 3.0 for t in _rand(shapes, torch.float32, 5)]
+    a = nt.nested_tensor(ts, device=DEV)
+    got = torch.nn.functional.max_pool2d(a, kernel_size=k, stride=s, padding=p, dilation=d, ceil_mode=True)
+    exp = oracle.max_pool2d(oracle.ref_nested_tensor(ts), k, s, p, d, ceil_mode=True)
+    assert got.nested_size() == nt.nested_tensor(list(exp.unbind())).nested_size()
+    assert torch.equal(got._impl.buffer.cpu(), exp.buffer)
+    with pytest.raises(NotImplementedError):
+        torch.nn.functional.max_pool2d(a, 2, return_indices=True)
+
+
 CONV_CASES = [
     # shapes, weight shape, stride, padding, dilation, groups
     ([(2, 2, 3), (2, 4, 2), (2, 2, 2)], (3, 2, 1, 1), 1, 0, 1, 1),
