@@ -58,11 +58,21 @@ template <> struct Mma<__bf16> {
   }
 };
 
+// fp32: v_mfma_f32_32x32x2_f32 contracts two k values per instruction, one per
+// lane half.  Which two is free as long as both operands agree, so a fragment is
+// the same 16-byte piece of a row as for the 16-bit types (lane half g holds
+// k = 8 s + 4 g .. + 3 of step s) and is spent over four instructions: the LDS
+// reads are the conflict-free 128-bit ones of the swizzled layout instead of
+// 4-byte column reads (which collide four to eight ways in it).
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 template <> struct Mma<float> {
-  typedef float Frag;
-  static constexpr int kK = 2;
+  typedef f32x4 Frag;
+  static constexpr int kK = 8;
   static __device__ __forceinline__ acc16 run(Frag a, Frag b, acc16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[0], b[0], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[1], b[1], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2], b[2], c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a[3], b[3], c, 0, 0, 0);
   }
 };
 
