@@ -602,3 +602,72 @@ def test_host_nested_tensors_are_staged_through_the_device():
     assert back.device.type == "cpu" and torch.equal(back._impl.buffer, ref.buffer)
     back = nt.from_padded_tensor(padded, a.nested_size())
     assert torch.equal(back._impl.buffer, ref.buffer)
+
+
+# ---- many short rows: the kernels that share the row decode ----------------------
+
+def _short_row_case(kind, g):
+    """Shapes with at least 4096 output rows of at most 4 KiB."""
+    if kind == "one ragged dim, rows up to 600 bytes":
+        return [(int(l),) for l in torch.randint(1, 301, (6000,), generator=g)]
+    if kind == "one ragged dim, rows up to 3840 bytes":
+        return [(int(l), 24) for l in torch.randint(1, 41, (5000,), generator=g)]
+    if kind == "two ragged dims":
+        hw = torch.randint(1, 201, (40, 2), generator=g)
+        hw[0] = torch.tensor([150, 200])
+        return [(min(int(h), 150), int(w)) for h, w in hw]
+    if kind == "three ragged dims":
+        chw = torch.randint(1, 7, (8, 1), generator=g), torch.randint(1, 201, (8, 1), generator=g), \
+            torch.randint(1, 151, (8, 1), generator=g)
+        shapes = [(int(c), int(h), int(w)) for c, h, w in zip(*chw)]
+        shapes[0] = (6, 200, 150)
+        return shapes
+    if kind == "two ragged dims and a regular tail":
+        hw = torch.randint(1, 121, (50, 2), generator=g)
+        hw[0] = torch.tensor([120, 120])
+        return [(int(h), int(w), 3) for h, w in hw]
+    raise AssertionError(kind)
+
+
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.float16, torch.float32, torch.float64])
+@pytest.mark.parametrize("kind", ["one ragged dim, rows up to 600 bytes", "one ragged dim, rows up to 3840 bytes",
+                                  "two ragged dims", "three ragged dims", "two ragged dims and a regular tail"])
+def test_many_short_rows(kind, dtype):
+    # from 4096 rows of at most 4 KiB on, pad / un-pad take the row-batch / row-group
+    # kernels and masks of 1 MiB or more the flat plane kernel: every element size,
+    # one to three ragged dims, rows at every alignment
+    g = torch.Generator().manual_seed(len(kind))
+    shapes = _short_row_case(kind, g)
+    if dtype == torch.float64 and kind == "one ragged dim, rows up to 3840 bytes":
+        shapes = [(l, 12) for l, _ in shapes]
+    if dtype.is_floating_point:
+        parts = [torch.randn(*s, generator=g).to(dtype) for s in shapes]
+    else:
+        parts = [torch.randint(1, 200, s, generator=g).to(dtype) for s in shapes]
+    a = nt.nested_tensor(parts, device=DEV, dtype=dtype)
+    ref = oracle.ref_nested_tensor(parts, dtype=dtype)
+    pad_value = 7 if dtype == torch.uint8 else -10000.0      # no N(0, 1) sample rounds to it
+    padded = a.to_padded_tensor(pad_value)
+    bits_equal(padded, oracle.to_padded_tensor(ref, pad_value))
+    bits_equal(nt.from_padded_tensor(padded, a)._impl.buffer, ref.buffer)
+    data, mask = a.to_tensor_mask()
+    exp_d, exp_m = oracle.to_tensor_mask(ref)
+    bits_equal(data, exp_d)
+    assert mask.shape == exp_m.shape and torch.equal(mask.cpu(), exp_m.to(torch.bool))
+    full = torch.ops.nestedtensor.to_mask(a, a.dim())
+    assert torch.equal(full.cpu(), oracle.to_mask(ref, a.dim()).to(torch.bool))
+    # a goal shape larger than the batch maximum in every dim: regular dims are
+    # walked as ragged, the extra region is padding in the data and zeros in the mask
+    goal = [m + 3 for m in a._impl.max_sizes()]
+    big_d, big_m = torch.ops.nestedtensor.pad_nt(a, goal)
+    exp_bd, exp_bm = oracle.pad_nt(ref, goal)
+    bits_equal(big_d, exp_bd)
+    assert torch.equal(big_m.cpu(), exp_bm.to(torch.bool))
+    bits_equal(nt.from_padded_tensor(big_d, a)._impl.buffer, ref.buffer)
+    # dense -> nested from the full mask and from the padding value
+    again = nt.nested_tensor_from_tensor_mask(data, full)
+    bits_equal(again._impl.buffer, ref.buffer)
+    assert again.nested_size() == a.nested_size()
+    if dtype != torch.uint8:
+        again = nt.nested_tensor_from_padded_tensor(padded, padding=pad_value)
+        bits_equal(again._impl.buffer, ref.buffer)
