@@ -280,6 +280,20 @@ def mha_probe(args, torch, dev):
                 torch.addmm(b_in, x, W_in.t())
                 torch.addmm(b_out, x, W_out.t())
             torch.cuda.synchronize()
+            # the in-projection shape at 1x, 2x and 4x the depth, on the whole batch (two
+            # rounds of output tiles) and on 4096 rows (192 tiles, 24 per XCD: one round): the
+            # differences between depths are the steady-state cost of a K tile, what is
+            # left at depth 0 is a tile's fill and drain
+            from nestedtensor_amd import ops as _ops
+            for rows in (T, 4096):
+                for depth in (E, 2 * E, 4 * E):
+                    xk = torch.randn(rows, depth, device=dev, dtype=dtype)
+                    wk = torch.randn(3 * E, depth, device=dev, dtype=dtype) * 0.02
+                    for _ in range(2):
+                        _ops.linear(xk, wk, b_in)
+                    torch.cuda.synchronize()
+            out["gemm_depth_sweep"] = dict(N=3 * E, rows=[T, 4096], depths=[E, 2 * E, 4 * E],
+                                           order="rows-major, two dispatches per (rows, depth)")
     print(json.dumps(out))
 
 
