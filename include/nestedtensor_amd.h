@@ -131,6 +131,18 @@ int nt_build_mask(uint8_t* mask, const int64_t* sizes, int64_t B, int64_t D, int
 int nt_pack(const void* const* srcs, void* packed, const int64_t* offsets, int64_t B,
             int elem_bytes, void* stream);
 
+/* nt_pack for a handful of constituents, without anything on the device before
+ * the launch: table_host (host memory) holds sizes[B * D], then offsets[B + 1]
+ * (element offsets), then the B source pointers, B * D + 2 B + 1 int64 entries in
+ * all, at most nt_pack_table_max_entries().  The table travels in the kernel
+ * arguments; if table_dev is not NULL the kernel also leaves a copy of it there
+ * (device int64, same layout), which is the device metadata the pad / mask
+ * operators take.  Same reference code as nt_pack (impl::pack,
+ * nestedtensor/csrc/storage/Packed.h:75-98). */
+int64_t nt_pack_table_max_entries(void);
+int nt_pack_table(const int64_t* table_host, int64_t B, int64_t D, void* packed, int64_t* table_dev,
+                  int elem_bytes, void* stream);
+
 /* ---- mask -> nested size, compaction ----------------------------------- */
 
 /* Row statistics of a byte mask viewed as [R, M] (nonzero = true):

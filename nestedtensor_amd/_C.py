@@ -43,6 +43,8 @@ SIGNATURES = {
                                  ctypes.POINTER(_i64), _int, _c_void_p]),
     "nt_build_mask": (_int, [_c_void_p, _c_void_p, _i64, _i64, _i64, ctypes.POINTER(_i64), _c_void_p]),
     "nt_pack": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _int, _c_void_p]),
+    "nt_pack_table_max_entries": (_i64, []),
+    "nt_pack_table": (_int, [_c_void_p, _i64, _i64, _c_void_p, _c_void_p, _int, _c_void_p]),
     "nt_mask_row_counts": (_int, [_c_void_p, _i64, _i64, _c_void_p, _c_void_p, _c_void_p]),
     "nt_value_row_counts": (_int, [_c_void_p, _int, ctypes.c_double, _i64, _i64, _c_void_p, _c_void_p,
                                    _c_void_p]),

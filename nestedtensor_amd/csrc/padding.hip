@@ -838,3 +838,78 @@ extern "C" int nt_pack(const void* const* srcs, void* packed, const int64_t* off
   // rows finish early.
   return launch_rows<kPack>(elem_bytes, p, (int64_t)1 << 22, (hipStream_t)stream);
 }
+
+// nt_pack for a handful of constituents: the table (sizes, offsets, source
+// pointers) travels in the kernel arguments, so nothing has to reach the device
+// before the launch, and the kernel leaves a copy of the table in device memory
+// for the operators that follow.
+namespace nt {
+constexpr int kPackTableMax = 384;     // int64 entries; with the other arguments well inside the 4 KiB of kernel arguments
+struct PackTable {
+  int64_t v[kPackTableMax];            // sizes[B * D], offsets[B + 1], source pointers[B]
+};
+
+template <int EB>
+__global__ __launch_bounds__(256) void pack_table_kernel(PackTable t, char* dst, int64_t B, int64_t D,
+                                                         int64_t* table_out) {
+  const int64_t row = row_index();
+  if (row >= B) return;
+  if (row == 0 && tile_index() == 0 && table_out != nullptr) {
+    const int64_t n = B * D + 2 * B + 1;
+    for (int64_t i = threadIdx.x; i < n; i += 256) table_out[i] = t.v[i];
+  }
+  const int64_t off = t.v[B * D + row];
+  const int64_t n = (t.v[B * D + row + 1] - off) * EB;
+  if (n <= 0) return;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  move_row<EB, kUnpad, 256>(dst + off * EB, reinterpret_cast<const char*>(t.v[B * D + B + 1 + row]), n, n, zero);
+}
+}  // namespace nt
+
+extern "C" int64_t nt_pack_table_max_entries(void) { return nt::kPackTableMax; }
+
+extern "C" int nt_pack_table(const int64_t* table_host, int64_t B, int64_t D, void* packed,
+                             int64_t* table_dev, int elem_bytes, void* stream) {
+  if (B == 0) return NT_OK;
+  const int64_t n = B * D + 2 * B + 1;
+  if (B < 0 || D < 0 || !table_host) return fail(NT_ERR_INVALID_ARGUMENT, "bad pack args");
+  if (n > nt::kPackTableMax) {
+    return fail(NT_ERR_UNSUPPORTED, "pack table of %lld entries exceeds the %d that fit in kernel arguments",
+                (long long)n, nt::kPackTableMax);
+  }
+  nt::PackTable t;
+  int64_t longest = 0;
+  for (int64_t i = 0; i < n; ++i) t.v[i] = table_host[i];
+  for (int64_t i = n; i < nt::kPackTableMax; ++i) t.v[i] = 0;
+  for (int64_t b = 0; b < B; ++b) {
+    const int64_t len = t.v[B * D + b + 1] - t.v[B * D + b];
+    if (len < 0) return fail(NT_ERR_INVALID_ARGUMENT, "pack offsets must not decrease");
+    longest = len > longest ? len : longest;
+  }
+  if (longest == 0 && table_dev == nullptr) return NT_OK;
+  if (longest > 0 && !packed) return fail(NT_ERR_INVALID_ARGUMENT, "bad pack args");
+  // the grid of the row kernels for un-pad / pack: a bounded number of looping
+  // workgroups per row, sized for the longest constituent
+  const int64_t tile_bytes = 256 * NT_ROW_UNROLL * 16;
+  int64_t tiles = (longest * elem_bytes + tile_bytes - 1) / tile_bytes;
+  int64_t y_cap = (int64_t)NT_ROW_TARGET_WGS / B;
+  if (y_cap < 1) y_cap = 1;
+  if (y_cap > NT_ROW_MAX_TILES_UNPAD) y_cap = NT_ROW_MAX_TILES_UNPAD;
+  int64_t gy = tiles < y_cap ? tiles : y_cap;
+  if (gy < 1) gy = 1;
+#if NT_ROW_TILE_FAST
+  dim3 grid((unsigned)gy, (unsigned)B, 1);
+#else
+  dim3 grid((unsigned)B, (unsigned)gy, 1);
+#endif
+  hipStream_t s = (hipStream_t)stream;
+  char* dst = static_cast<char*>(packed);
+  switch (elem_bytes) {
+    case 1: hipLaunchKernelGGL((nt::pack_table_kernel<1>), grid, dim3(256), 0, s, t, dst, B, D, table_dev); break;
+    case 2: hipLaunchKernelGGL((nt::pack_table_kernel<2>), grid, dim3(256), 0, s, t, dst, B, D, table_dev); break;
+    case 4: hipLaunchKernelGGL((nt::pack_table_kernel<4>), grid, dim3(256), 0, s, t, dst, B, D, table_dev); break;
+    case 8: hipLaunchKernelGGL((nt::pack_table_kernel<8>), grid, dim3(256), 0, s, t, dst, B, D, table_dev); break;
+    default: return fail(NT_ERR_INVALID_ARGUMENT, "elem_bytes must be 1, 2, 4 or 8, got %d", elem_bytes);
+  }
+  return check_launch("pack_table_kernel");
+}

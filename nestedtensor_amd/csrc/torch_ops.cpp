@@ -214,9 +214,10 @@ Tensor build_mask(const Tensor& sizes_dev, at::IntArrayRef ext) {
 
 // impl::pack (Packed.h:75-98) with the checks of _verify_variables
 // (creation.cpp:28-171) for constituents that already live on the device: one
-// gather launch (nt_pack) instead of B copy_ calls.  The nested size, the element
-// offsets computed from it and the table of source pointers reach the device in
-// one copy from pinned memory.  Returns (buffer, sizes, sizes_dev, offsets_dev).
+// gather launch (nt_pack / nt_pack_table) instead of B copy_ calls.  The nested
+// size, the element offsets computed from it and the table of source pointers
+// reach the device in the launch's own arguments when they fit there, else in one
+// copy from pinned memory.  Returns (buffer, sizes, sizes_dev, offsets_dev).
 std::tuple<Tensor, Tensor, Tensor, Tensor> pack_device(at::TensorList tensors) {
   static const char* hint =
       "To form a valid NestedTensor all Tensor / NestedTensor constiuents of the given list must be "
@@ -245,7 +246,12 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> pack_device(at::TensorList tensors) {
   Tensor sizes = at::empty({B, D}, at::kLong);
   int64_t* sp = sizes.data_ptr<int64_t>();
   const int64_t n = B * D + (B + 1) + B;
-  Tensor host = at::empty({n}, at::TensorOptions().dtype(at::kLong).pinned_memory(true));
+  // a small table goes to the device inside the kernel arguments of the pack
+  // launch, which also writes the device copy; a large one is uploaded from pinned
+  // memory first
+  const bool in_args = n <= nt_pack_table_max_entries();
+  Tensor host = in_args ? at::empty({n}, at::kLong)
+                        : at::empty({n}, at::TensorOptions().dtype(at::kLong).pinned_memory(true));
   int64_t* h = host.data_ptr<int64_t>();
   int64_t* off = h + B * D;
   int64_t* ptrs = off + B + 1;
@@ -259,13 +265,17 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> pack_device(at::TensorList tensors) {
   }
   off[B] = acc;
   Tensor meta = at::empty({n}, first.options().dtype(at::kLong));
-  meta.copy_(host, /*non_blocking=*/true);
   Tensor sizes_dev = meta.narrow(0, 0, B * D).view({B, D});
   Tensor offsets_dev = meta.narrow(0, B * D, B + 1);
   Tensor buffer = at::empty({acc}, first.options());
-  if (acc > 0) {
-    check(nt_pack(reinterpret_cast<const void* const*>(meta.const_data_ptr<int64_t>() + B * D + B + 1),
-                  buffer.data_ptr(), offsets_dev.const_data_ptr<int64_t>(), B, eb, stream_of(first)));
+  if (in_args) {
+    check(nt_pack_table(h, B, D, buffer.data_ptr(), meta.data_ptr<int64_t>(), eb, stream_of(first)));
+  } else {
+    meta.copy_(host, /*non_blocking=*/true);
+    if (acc > 0) {
+      check(nt_pack(reinterpret_cast<const void* const*>(meta.const_data_ptr<int64_t>() + B * D + B + 1),
+                    buffer.data_ptr(), offsets_dev.const_data_ptr<int64_t>(), B, eb, stream_of(first)));
+    }
   }
   // `keep` may hold temporaries; torch's caching allocator reuses their blocks
   // only for later work on this same stream

@@ -671,3 +671,26 @@ def test_many_short_rows(kind, dtype):
     if dtype != torch.uint8:
         again = nt.nested_tensor_from_padded_tensor(padded, padding=pad_value)
         bits_equal(again._impl.buffer, ref.buffer)
+
+
+def test_pack_table_in_kernel_arguments_and_uploaded():
+    # up to nt_pack_table_max_entries() int64 of metadata ride in the kernel arguments of
+    # the pack launch, which also writes their device copy; larger batches upload the
+    # table first.  Both sides of the limit, empty constituents, and the adopted metadata.
+    from nestedtensor_amd import _C
+    limit = int(_C.lib.nt_pack_table_max_entries())
+    g = torch.Generator().manual_seed(91)
+    for B, D in ((1, 1), (16, 3), (limit // 4, 2), (limit // 4 + 5, 2), (3, 2)):
+        shapes = [[int(v) for v in torch.randint(0 if B == 3 else 1, 9, (D,), generator=g)] for _ in range(B)]
+        parts = [torch.randn(*s, generator=g) for s in shapes]
+        dev_parts = [p.to(DEV) for p in parts]
+        a = nt.nested_tensor(dev_parts, device=DEV)
+        ref = oracle.ref_nested_tensor(parts)
+        bits_equal(a._impl.buffer, ref.buffer)
+        assert a.nested_size().unbind() == [torch.Size(p.shape) for p in parts]
+        assert torch.equal(a._impl.sizes_dev().cpu(), a._impl.sizes)
+        exp_off = torch.zeros(B + 1, dtype=torch.int64)
+        exp_off[1:] = torch.cumsum(a._impl.sizes.prod(1), 0)
+        assert torch.equal(a._impl.offsets_dev().cpu(), exp_off)
+        if not a._impl.has_empty_constituent():
+            bits_equal(a.to_padded_tensor(0), oracle.to_padded_tensor(ref, 0))
