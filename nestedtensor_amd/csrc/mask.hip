@@ -60,6 +60,14 @@ __global__ __launch_bounds__(kWave * kRowsPerBlock) void row_counts_kernel(
   }
   for (int64_t base = 0; base < M; base += (int64_t)kWave * VEC) {
     const int64_t i0 = base + (int64_t)lane * VEC;
+    // entries of this lane that exist (the last lanes of the last step hold fewer)
+    const int64_t here = M - i0;
+    const int exist = here >= VEC ? VEC : (here > 0 ? (int)here : 0);
+    // A lane whose VEC entries run past the end of the row reads the LAST VEC
+    // entries of the row instead (one whole 16-byte load like everyone else, no
+    // element-wise tail) and drops the low VEC - exist flags: what is left are the
+    // flags of entries i0 .. M - 1.  The vector path is only taken for M >= VEC.
+    const int64_t ld = (VEC == 1 || here >= VEC) ? i0 : M - VEC;
     T v[NR][VEC];
 #pragma unroll
     for (int r = 0; r < NR; ++r) {
@@ -67,28 +75,25 @@ __global__ __launch_bounds__(kWave * kRowsPerBlock) void row_counts_kernel(
       const T* m = data + (row0 + r) * M;
       if (VEC == 1) {
         if (i0 < M) v[r][0] = m[i0];
-      } else if (i0 + VEC <= M) {
-        // any alignment: the part runs in unaligned-access mode
-        u32x4 raw = load16_unaligned(reinterpret_cast<const char*>(m + i0));
-        __builtin_memcpy(v[r], &raw, 16);
       } else {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          if (i0 + j < M) v[r][j] = m[i0 + j];
-        }
+        // any alignment: the part runs in unaligned-access mode
+        u32x4 raw = load16_unaligned(reinterpret_cast<const char*>(m + ld));
+        __builtin_memcpy(v[r], &raw, 16);
       }
     }
-    // entries of this lane that exist (the last lanes of the last step hold fewer)
-    const int64_t here = M - i0;
-    const int exist = here >= VEC ? VEC : (here > 0 ? (int)here : 0);
     const uint64_t present = __ballot(exist > 0);
 #pragma unroll
     for (int r = 0; r < NR; ++r) {
       if (row0 + r >= R) continue;
       uint32_t flags = 0;
+      if (VEC == 1) {
+        if (exist > 0 && pred(v[r][0])) flags = 1u;
+      } else {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        if (j < exist && pred(v[r][j])) flags |= 1u << j;
+        for (int j = 0; j < VEC; ++j) {
+          if (pred(v[r][j])) flags |= 1u << j;
+        }
+        flags = exist == VEC ? flags : (exist > 0 ? flags >> (VEC - exist) : 0u);
       }
       const int cnt = __popc(flags);
       count[r] += cnt;

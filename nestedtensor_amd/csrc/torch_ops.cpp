@@ -415,6 +415,41 @@ void upload_meta(const Tensor& sizes, const Tensor& like, Tensor* sizes_dev, Ten
   *offsets_dev = meta.narrow(0, B * D, B + 1);
 }
 
+// All n entries of p equal v (one block compare of the array against itself, shifted).
+template <typename T>
+bool all_equal(const T* p, int64_t n, T v) {
+  if (n <= 0) return true;
+  return p[0] == v && (n == 1 || std::memcmp(p, p + 1, static_cast<size_t>(n - 1) * sizeof(T)) == 0);
+}
+
+// Keep-counts c of one constituent, one per mask row, rows indexed by dims[0 .. nd)
+// (row-major).  True iff they describe a leading box: c = w where every row index
+// i_k < ext[k], 0 elsewhere, w > 0 (or everything 0).  Fills ext[0 .. nd] = (row
+// extents, w).  Level by level from the innermost row dim: the children of the
+// first parent are copies of the first child up to some extent and zero after it;
+// the first parent then is the pattern for the level above.
+bool leading_box(const int32_t* c, const int64_t* dims, int64_t nd, int64_t* ext) {
+  int64_t n = 1;
+  for (int64_t k = 0; k < nd; ++k) n *= dims[k];
+  if (n == 0) return false;
+  const int32_t w = c[0];
+  if (w == 0) {
+    for (int64_t k = 0; k <= nd; ++k) ext[k] = 0;
+    return all_equal(c, n, int32_t(0));
+  }
+  int64_t block = 1;                       // entries of one child at the current level
+  for (int64_t k = nd - 1; k >= 0; --k) {
+    const int64_t d = dims[k];
+    int64_t e = 1;
+    while (e < d && std::memcmp(c, c + e * block, static_cast<size_t>(block) * 4) == 0) ++e;
+    if (!all_equal(c + e * block, (d - e) * block, int32_t(0))) return false;
+    ext[k] = e;
+    block *= d;
+  }
+  ext[nd] = w;
+  return true;
+}
+
 // General case of nt_from_tensor_mask (masking.cpp:203-222) for a mask over the
 // first `mask_dims` dims of `tensor`.  Rows = everything but the last mask dim.
 // `count_rows` fills device (counts, prefix flags); `byte_mask` materialises the
@@ -456,10 +491,23 @@ Lowered from_rows(const Tensor& tensor, int64_t mask_dims, CountRows count_rows,
   bool leading = true;
   std::vector<int64_t> total(B, 0);
   std::vector<std::vector<int64_t>> extents(B, std::vector<int64_t>(levels, 0));   // outermost first
-  std::vector<uint8_t> alive(rows_per > 0 ? rows_per : 1), next(rows_per > 0 ? rows_per : 1);
+  std::vector<uint8_t> alive, next;
   for (int64_t b = 0; b < B; ++b) {
     const int32_t* c = counts + b * rows_per;
     const uint8_t* pf = prefix + b * rows_per;
+    // What a padded tensor's mask looks like: every row keeps the same leading w
+    // entries or nothing, and the rows that keep something are a leading box of the
+    // row dims.  Checked with block compares (each count is looked at about twice).
+    if (rows_per > 0 && all_equal(pf, rows_per, uint8_t(1)) &&
+        leading_box(c, shape.data() + 1, levels - 1, extents[b].data())) {
+      int64_t prod = 1;
+      for (int64_t v : extents[b]) prod *= v;
+      total[b] = prod;
+      continue;
+    }
+    // anything else: the walk over every row
+    alive.resize(rows_per > 0 ? rows_per : 1);
+    next.resize(rows_per > 0 ? rows_per : 1);
     int64_t sum = 0;
     int32_t mx = 0;
     uint8_t all_prefix = 1;
