@@ -200,9 +200,10 @@ int nt_linear_act(const void* A, int64_t lda, const void* W, const void* bias, v
  * over that sequence's own keys only:
  *   out[q_off[b] + i, h*hd + d] = sum_j softmax_j(scale * q_i . k_j) v_j[d]
  * q rows are q[(q_off[b] + i) * ldq + h*hd ...], k/v likewise with kv_off.
- * f16 / bf16 with head_dim 64 run on the matrix pipe; any other head_dim, and
- * f32, take a scalar kernel (one wavefront per query row and head), which is a
- * parity path, not a fast one.  Replaces the padded chain of bt_min_mha
+ * f16 / bf16 with head_dim 64 and f32 with head_dim 32, 64 or 128 (rows 16-byte
+ * aligned) run on the matrix pipe; anything else takes a scalar kernel (one
+ * wavefront per query row and head), which is a parity path, not a fast one.
+ * Replaces the padded chain of bt_min_mha
  * (nestedtensor/csrc/cuda/mha.cpp:59-105: to_padded_tensor, batched QK^T,
  * softmax_kernel_kernelLauncher of cuda/attention.h:25-33, PV,
  * from_padded_tensor) and the unwired add_QKV_bias_padding /
@@ -255,6 +256,17 @@ int nt_varlen_attention_vt(const void* q, int64_t ldq, const void* k, int64_t ld
                            int64_t ldvt, void* out, int64_t ldo, const int32_t* schedule,
                            int64_t n_work, int64_t num_heads, int64_t head_dim,
                            int64_t total_kv_tokens, float scale, int dtype, void* stream);
+
+/* nt_varlen_attention (V row-major) driven by the work list of
+ * nt_varlen_attention_vt instead of a padded grid: one workgroup per (item,
+ * head), so only query tiles that exist are launched and the long sequences
+ * start first.  f32 with head_dim 32, 64 or 128; every row 16-byte aligned
+ * (pointers and row strides).  The reference runs f32 bt_min_mha through the same
+ * padded chain as the other types (nestedtensor/csrc/cuda/mha.cpp:59-105). */
+int nt_varlen_attention_scheduled(const void* q, int64_t ldq, const void* k, int64_t ldk,
+                                  const void* v, int64_t ldv, void* out, int64_t ldo,
+                                  const int32_t* schedule, int64_t n_work, int64_t num_heads,
+                                  int64_t head_dim, float scale, int dtype, void* stream);
 
 /* ---- row-wise ops on the packed buffer (the steps either side of attention
  *      in an encoder layer) ------------------------------------------------ */

@@ -740,11 +740,11 @@ __global__ __launch_bounds__(64) void attention_rows_kernel(
 // (sequence, head) and walks the sequence's keys in tiles of 32, the next tile's
 // global loads in flight while the current one is multiplied, two LDS buffers.
 template <int HD>
-__global__ __launch_bounds__(256) void varlen_attention_f32_kernel(
+__device__ __forceinline__ void attention_f32_tile(
     const float* __restrict__ Q, int64_t ldq, const float* __restrict__ Kp, int64_t ldk,
     const float* __restrict__ Vp, int64_t ldv, float* __restrict__ O, int64_t ldo,
-    const int64_t* __restrict__ q_offsets, const int64_t* __restrict__ kv_offsets,
-    float scale_log2e) {
+    const int64_t q_begin, const int64_t Lq, const int64_t q0, const int64_t kv_begin, const int64_t Lk,
+    const int h, float scale_log2e, float* lds) {
   typedef float f32x4 __attribute__((ext_vector_type(4)));
   constexpr int kKT = 32;                      // keys per tile
   constexpr int kKs = HD + 4;                  // K row stride in floats: 16-byte reads of 16 rows hit 16 bank groups
@@ -752,15 +752,6 @@ __global__ __launch_bounds__(256) void varlen_attention_f32_kernel(
   constexpr int kBuf = kKT * (kKs + kVs);
   constexpr int kC4 = HD / 4;                  // 16-byte pieces per row
   constexpr int kPieces = kKT * kC4 / 256;     // pieces per thread and operand: 1, 2, 4
-  __shared__ __align__(16) float lds[2 * kBuf];
-
-  const int b = blockIdx.z, h = blockIdx.y;
-  const int64_t q_begin = q_offsets[b];
-  const int64_t Lq = q_offsets[b + 1] - q_begin;
-  const int64_t q0 = (int64_t)blockIdx.x * 128;
-  if (q0 >= Lq) return;                        // uniform
-  const int64_t kv_begin = kv_offsets[b];
-  const int64_t Lk = kv_offsets[b + 1] - kv_begin;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 31, half = lane >> 5;
 
@@ -887,6 +878,41 @@ __global__ __launch_bounds__(256) void varlen_attention_f32_kernel(
   }
 }
 
+// Workgroup = (128 query rows, head, sequence) on a padded grid: tiles past a
+// sequence's last query row leave at once.
+template <int HD>
+__global__ __launch_bounds__(256) void varlen_attention_f32_kernel(
+    const float* __restrict__ Q, int64_t ldq, const float* __restrict__ Kp, int64_t ldk,
+    const float* __restrict__ Vp, int64_t ldv, float* __restrict__ O, int64_t ldo,
+    const int64_t* __restrict__ q_offsets, const int64_t* __restrict__ kv_offsets,
+    float scale_log2e) {
+  __shared__ __align__(16) float lds[2 * 32 * (2 * HD + 12)];
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int64_t q_begin = q_offsets[b];
+  const int64_t Lq = q_offsets[b + 1] - q_begin;
+  const int64_t q0 = (int64_t)blockIdx.x * 128;
+  if (q0 >= Lq) return;                        // uniform
+  const int64_t kv_begin = kv_offsets[b];
+  attention_f32_tile<HD>(Q, ldq, Kp, ldk, Vp, ldv, O, ldo, q_begin, Lq, q0, kv_begin,
+                         kv_offsets[b + 1] - kv_begin, h, scale_log2e, lds);
+}
+
+// The same tiles from a work list (the items of nt_varlen_attention_vt): only
+// tiles that exist are launched, longest key sequences first, head fastest.
+template <int HD>
+__global__ __launch_bounds__(256) void varlen_attention_f32_sched_kernel(
+    const float* __restrict__ Q, int64_t ldq, const float* __restrict__ Kp, int64_t ldk,
+    const float* __restrict__ Vp, int64_t ldv, float* __restrict__ O, int64_t ldo,
+    const int4* __restrict__ schedule, unsigned num_heads, float scale_log2e) {
+  __shared__ __align__(16) float lds[2 * 32 * (2 * HD + 12)];
+  const int h = (int)(blockIdx.x % num_heads);
+  const int4 item = schedule[2 * (blockIdx.x / num_heads)];
+  const int4 item_kv = schedule[2 * (blockIdx.x / num_heads) + 1];
+  if (item.y <= 0 || item.z >= item.y) return;   // uniform: no query rows in this tile
+  attention_f32_tile<HD>(Q, ldq, Kp, ldk, Vp, ldv, O, ldo, item.x, item.y, item.z, item_kv.x,
+                         item_kv.y > 0 ? item_kv.y : 0, h, scale_log2e, lds);
+}
+
 template <int HD>
 static int launch_f32(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
                       int64_t ldv, void* out, int64_t ldo, const int64_t* qo, const int64_t* kvo,
@@ -997,6 +1023,50 @@ static void launch_vt(dim3 grid, hipStream_t s, const void* q, int64_t ldq, cons
   hipLaunchKernelGGL((varlen_attention_vt_kernel<T, HD>), grid, dim3(256), 0, s, static_cast<const T*>(q),
                      ldq, static_cast<const T*>(k), ldk, static_cast<const T*>(vt), ldvt,
                      static_cast<T*>(out), ldo, sched, num_heads, scale_log2e);
+}
+
+template <int HD>
+static void launch_f32_sched(dim3 grid, hipStream_t s, const void* q, int64_t ldq, const void* k, int64_t ldk,
+                             const void* v, int64_t ldv, void* out, int64_t ldo, const int4* sched,
+                             unsigned num_heads, float scale_log2e) {
+  hipLaunchKernelGGL((varlen_attention_f32_sched_kernel<HD>), grid, dim3(256), 0, s,
+                     static_cast<const float*>(q), ldq, static_cast<const float*>(k), ldk,
+                     static_cast<const float*>(v), ldv, static_cast<float*>(out), ldo, sched, num_heads,
+                     scale_log2e);
+}
+
+extern "C" int nt_varlen_attention_scheduled(const void* q, int64_t ldq, const void* k, int64_t ldk,
+                                             const void* v, int64_t ldv, void* out, int64_t ldo,
+                                             const int32_t* schedule, int64_t n_work, int64_t num_heads,
+                                             int64_t head_dim, float scale, int dtype, void* stream) {
+  if (n_work < 0 || num_heads < 1) return fail(NT_ERR_INVALID_ARGUMENT, "attention_scheduled: bad shape");
+  if (dtype != NT_F32 || (head_dim != 32 && head_dim != 64 && head_dim != 128)) {
+    return fail(NT_ERR_UNSUPPORTED, "attention_scheduled: f32 with head_dim 32, 64 or 128 only (got dtype %d, "
+                "head_dim %lld)", dtype, (long long)head_dim);
+  }
+  if (n_work == 0) return NT_OK;
+  if (!q || !k || !v || !out || !schedule) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "attention_scheduled: NULL pointer");
+  }
+  const int64_t E = num_heads * head_dim;
+  if (ldq < E || ldk < E || ldv < E || ldo < E) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "attention_scheduled: row stride smaller than num_heads*head_dim");
+  }
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) % 16 != 0 || (ldq | ldk | ldv | ldo) % 4 != 0) {
+    return fail(NT_ERR_UNSUPPORTED, "attention_scheduled: rows must be 16-byte aligned");
+  }
+  if (num_heads > 65535 || n_work * num_heads > 0x7fffffffLL) {
+    return fail(NT_ERR_UNSUPPORTED, "attention_scheduled: too many workgroups");
+  }
+  dim3 grid((unsigned)(n_work * num_heads), 1, 1);
+  const float scale_log2e = scale * 1.4426950408889634f;
+  hipStream_t s = (hipStream_t)stream;
+  const int4* sched = reinterpret_cast<const int4*>(schedule);
+  const unsigned nh = (unsigned)num_heads;
+  if (head_dim == 32) launch_f32_sched<32>(grid, s, q, ldq, k, ldk, v, ldv, out, ldo, sched, nh, scale_log2e);
+  else if (head_dim == 64) launch_f32_sched<64>(grid, s, q, ldq, k, ldk, v, ldv, out, ldo, sched, nh, scale_log2e);
+  else launch_f32_sched<128>(grid, s, q, ldq, k, ldk, v, ldv, out, ldo, sched, nh, scale_log2e);
+  return check_launch("varlen_attention_f32_sched_kernel");
 }
 
 extern "C" int nt_varlen_attention_vt(const void* q, int64_t ldq, const void* k, int64_t ldk,

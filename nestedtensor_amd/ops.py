@@ -456,11 +456,20 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
             qc = kc = vc = 0
             ldq = ldk = ldv = E
         with _C.on_device(dev):
-            _C.check(_C.lib.nt_varlen_attention(
-                _offset_ptr(q_t, qc), ldq, _offset_ptr(k_t, kc), ldk, _offset_ptr(v_t, vc), ldv,
-                _C.ptr(attn), E, _C.ptr(query.row_offsets_dev()), _C.ptr(key.row_offsets_dev()),
-                query.B, num_heads, head_dim, max_q, float(scaling), _C.dtype_code(dtype),
-                _C.current_stream(dev)))
+            if dtype == torch.float32 and head_dim in (32, 64, 128):
+                # fp32 on the fp32 matrix instruction, from the work list: only tiles
+                # that exist, longest key sequences first
+                sched = query.attention_schedule(kv=None if same else key)
+                _C.check(_C.lib.nt_varlen_attention_scheduled(
+                    _offset_ptr(q_t, qc), ldq, _offset_ptr(k_t, kc), ldk, _offset_ptr(v_t, vc), ldv,
+                    _C.ptr(attn), E, _C.ptr(sched), sched.size(0), num_heads, head_dim, float(scaling),
+                    _C.dtype_code(dtype), _C.current_stream(dev)))
+            else:
+                _C.check(_C.lib.nt_varlen_attention(
+                    _offset_ptr(q_t, qc), ldq, _offset_ptr(k_t, kc), ldk, _offset_ptr(v_t, vc), ldv,
+                    _C.ptr(attn), E, _C.ptr(query.row_offsets_dev()), _C.ptr(key.row_offsets_dev()),
+                    query.B, num_heads, head_dim, max_q, float(scaling), _C.dtype_code(dtype),
+                    _C.current_stream(dev)))
     out = linear(attn, out_proj_weight, out_proj_bias)
     return query.with_buffer(out.reshape(-1))
 

@@ -510,3 +510,53 @@ def test_min_mha_reference_shapes_large(dtype, H, B, Lmax, hd):
     ref = oracle.ref_nested_tensor(xs, dtype=dtype)
     exp = oracle.min_mha(H, hd, 0.0, False, ref, ref, ref, W_in, b_in, hd ** -0.5, W_out, b_out)
     check(got, exp, dtype)
+
+
+@pytest.mark.parametrize("hd", [32, 64, 128])
+def test_fp32_attention_padded_grid_and_work_list(hd):
+    # the two C entry points of the fp32 matrix-pipe kernel: nt_varlen_attention (grid
+    # padded to the longest sequence, device offsets) and nt_varlen_attention_scheduled
+    # (work list); same tiles, same arithmetic, so the same bits, and both against
+    # a float64 softmax(q k^T) v per sequence and head
+    from nestedtensor_amd import _C
+    from nestedtensor_amd.impl import NestedTensorImpl
+    H = 3
+    E = H * hd
+    q_lens, k_lens = [5, 130, 64, 1, 257], [77, 33, 200, 1, 64]
+    g = torch.Generator().manual_seed(hd)
+    Tq, Tk = sum(q_lens), sum(k_lens)
+    q = torch.randn(Tq, E, generator=g)
+    k = torch.randn(Tk, E, generator=g)
+    v = torch.randn(Tk, E, generator=g)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    qi = NestedTensorImpl(qd.reshape(-1), torch.tensor([[L, E] for L in q_lens], dtype=torch.int64))
+    ki = NestedTensorImpl(kd.reshape(-1), torch.tensor([[L, E] for L in k_lens], dtype=torch.int64))
+    scale = hd ** -0.5
+    out_a = torch.full((Tq, E), float("nan"), device=DEV)
+    out_b = torch.full((Tq, E), float("nan"), device=DEV)
+    stream = _C.current_stream(DEV)
+    _C.check(_C.lib.nt_varlen_attention(
+        _C.ptr(qd), E, _C.ptr(kd), E, _C.ptr(vd), E, _C.ptr(out_a), E, _C.ptr(qi.row_offsets_dev()),
+        _C.ptr(ki.row_offsets_dev()), len(q_lens), H, hd, max(q_lens), scale, _C.dtype_code(torch.float32), stream))
+    sched = qi.attention_schedule(kv=ki)
+    _C.check(_C.lib.nt_varlen_attention_scheduled(
+        _C.ptr(qd), E, _C.ptr(kd), E, _C.ptr(vd), E, _C.ptr(out_b), E, _C.ptr(sched), sched.size(0), H, hd,
+        scale, _C.dtype_code(torch.float32), stream))
+    torch.cuda.synchronize()
+    assert torch.equal(out_a, out_b)
+    exp = torch.empty(Tq, E, dtype=torch.float64)
+    qo = ko = 0
+    for Lq, Lk in zip(q_lens, k_lens):
+        for h in range(H):
+            c = slice(h * hd, (h + 1) * hd)
+            s = (q[qo:qo + Lq, c].double() @ k[ko:ko + Lk, c].double().t()) * scale
+            exp[qo:qo + Lq, c] = torch.softmax(s, -1) @ v[ko:ko + Lk, c].double()
+        qo, ko = qo + Lq, ko + Lk
+    err = (out_a.cpu().double() - exp).abs().max().item()
+    assert err <= FP32_REL * exp.abs().max().item(), err
+    # rows that are not 16-byte aligned are refused by the work-list entry point and
+    # take the scalar kernel in the other
+    rc = _C.lib.nt_varlen_attention_scheduled(
+        _C.ptr(qd), E + 1, _C.ptr(kd), E, _C.ptr(vd), E, _C.ptr(out_b), E, _C.ptr(sched), sched.size(0), H, hd,
+        scale, _C.dtype_code(torch.float32), stream)
+    assert rc != 0
