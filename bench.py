@@ -294,6 +294,33 @@ def mha_probe(args, torch, dev):
                     torch.cuda.synchronize()
             out["gemm_depth_sweep"] = dict(N=3 * E, rows=[T, 4096], depths=[E, 2 * E, 4 * E],
                                            order="rows-major, two dispatches per (rows, depth)")
+            # the attention kernel alone on batches of equal-length sequences (random
+            # operands in the layout the projection writes): what a key tile costs when
+            # sequences are long, and what a workgroup costs when they are short
+            import ctypes
+            from nestedtensor_amd import _C
+            from nestedtensor_amd.impl import NestedTensorImpl
+            sweep = []
+            for count, length in ((8, 2048), (64, 512), (16, 512), (64, 256), (128, 128), (256, 64)):
+                Tn = count * length
+                ldvt = (Tn + 72 + 7) // 8 * 8
+                qk = torch.randn(Tn, 2 * E, device=dev, dtype=dtype)
+                vt = torch.randn(E, ldvt, device=dev, dtype=dtype)
+                o = torch.empty(Tn, E, device=dev, dtype=dtype)
+                impl = NestedTensorImpl(torch.empty(Tn * E, device=dev, dtype=dtype),
+                                        torch.tensor([[length, E]] * count, dtype=torch.int64))
+                sched = impl.attention_schedule()
+                kptr = ctypes.c_void_p(qk.data_ptr() + E * qk.element_size())
+                for _ in range(2):
+                    _C.check(_C.lib.nt_varlen_attention_vt(
+                        _C.ptr(qk), 2 * E, kptr, 2 * E, _C.ptr(vt), ldvt, _C.ptr(o), E, _C.ptr(sched),
+                        sched.size(0), H, 64, Tn, 0.125, _C.dtype_code(dtype), _C.current_stream(dev)))
+                torch.cuda.synchronize()
+                q_tiles, k_tiles = (length + 127) // 128, (length + 63) // 64
+                sweep.append(dict(sequences=count, length=length, workgroups=count * q_tiles * H,
+                                  wavefront_key_tiles=count * q_tiles * 4 * k_tiles * H,
+                                  flops=4 * E * count * length * length))
+            out["attention_length_sweep"] = sweep
     print(json.dumps(out))
 
 
