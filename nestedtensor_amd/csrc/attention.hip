@@ -619,12 +619,17 @@ __global__ __launch_bounds__(256, (HD > 64 ? 2 : NT_ATTN_WAVES_PER_EU)) void var
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
     const int buf = t & 1;
-    gload(st, t + 1);   // past the end: re-reads the last tile
+    const bool more = t + 1 < ntiles;   // uniform
+    if (more) gload(st, t + 1);
     // keep the loads above the MFMA / softmax work (the scheduler would sink them)
     __builtin_amdgcn_sched_barrier(0);
     if (wave_active) tile(buf, t == 0, t == ntiles - 1 && n_last < kKTile);
-    lstore(st, buf ^ 1, t + 1);   // past the end: harmless, the buffer is not read again
-    __syncthreads();
+    // the last tile loads nothing and waits for nothing: a workgroup of a short
+    // sequence is mostly its first loads and its last stores
+    if (more) {
+      lstore(st, buf ^ 1, t + 1);
+      __syncthreads();
+    }
   }
 
   if (!wave_active) return;
