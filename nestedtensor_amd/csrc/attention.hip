@@ -376,14 +376,19 @@ __global__ __launch_bounds__(256, (HD > 64 ? 2 : NT_ATTN_WAVES_PER_EU)) void var
   __shared__ __align__(16) char lds_k[2][kKTile * kKR];
   __shared__ __align__(16) char lds_v[2][HD * kVRow];
 
+  // Every kernel argument is wanted in registers now, together with the work item,
+  // not fetched piecemeal after the first branch: a workgroup of a short sequence is
+  // a chain of dependent memory round trips, and each scalar fetch is one of them.
+  asm volatile("" ::"s"(Q), "s"(K), "s"(Vt), "s"(O), "s"(ldq), "s"(ldk), "s"(ldvt), "s"(ldo));
   const int h = (int)(blockIdx.x % num_heads);
-  const int4 item = schedule[2 * (blockIdx.x / num_heads)];
-  const int4 item_kv = schedule[2 * (blockIdx.x / num_heads) + 1];
-  const int64_t q_begin = item.x;
-  const int Lq = item.y;
-  const int q0 = item.z;
-  const int64_t begin = item_kv.x;
-  const int L = item_kv.y;
+  // the whole work item in one 32-byte scalar load: everything below waits for it
+  typedef int int8v __attribute__((ext_vector_type(8)));
+  const int8v item = *reinterpret_cast<const int8v*>(schedule + 2 * (blockIdx.x / num_heads));
+  const int64_t q_begin = item[0];
+  const int Lq = item[1];
+  const int q0 = item[2];
+  const int64_t begin = item[4];
+  const int L = item[5];
   if (L <= 0 || Lq <= 0) {   // uniform.  No keys: zeros, as in varlen_attention_kernel
     for (int i = threadIdx.x; i < kQTile * (HD / 8); i += 256) {
       const int row = q0 + i / (HD / 8);
