@@ -601,6 +601,18 @@ def bench_rows(args, torch, dev, later):
         cpu_leg("C2_to_tensor_mask", lambda: oracle.to_tensor_mask(ref2), 1)
         cpu_leg("C2_nested_tensor_from_tensor_mask", lambda: oracle.nt_from_tensor_mask_vectorised(dcpu, mcpu), 1)
         cpu_leg("C2_to_mask", lambda: oracle.to_mask(ref2, 4), 1)
+
+        def _literal_walk():
+            # the reference's own algorithm (one host call per mask element) on every
+            # eighth row and column: 1/64 of the elements, the same kind of mask
+            d8, m8 = dcpu[:, :, ::8, ::8].contiguous(), mcpu[:, :, ::8, ::8].contiguous()
+            t0 = time.perf_counter()
+            oracle.nt_from_tensor_mask(d8, m8, 1)
+            dt = time.perf_counter() - t0
+            rows["C2_nested_tensor_from_tensor_mask"]["cpu_literal_walk"] = dict(
+                sample="every eighth row and column of the C2 tensor and mask (1/64 of the elements)",
+                mask_elements=int(m8.numel()), ms=dt * 1e3, ns_per_mask_element=dt * 1e9 / m8.numel())
+        later.append(_literal_walk)
         cpu_leg("C2_nested_tensor_pack_from_device_tensors", lambda: oracle.ref_nested_tensor(imgs), 1)
     del data, mask, back2, dev_imgs, a2
 
