@@ -560,3 +560,47 @@ def test_fp32_attention_padded_grid_and_work_list(hd):
         _C.ptr(qd), E + 1, _C.ptr(kd), E, _C.ptr(vd), E, _C.ptr(out_b), E, _C.ptr(sched), sched.size(0), H, hd,
         scale, _C.dtype_code(torch.float32), stream)
     assert rc != 0
+
+
+def test_encoder_layer_under_hip_graph_replays():
+    # a whole encoder layer on the packed layout (attention, add + layer norm, feed-forward
+    # with gelu in the GEMM epilogue, add + layer norm: seven launches) captured once and
+    # replayed with new token values; every replay must equal the eager layer
+    from nestedtensor_amd import ops
+    E, H = 256, 4
+    xs, W_in, b_in, W_out, b_out = make_case(E, [37, 200, 64, 129, 5], 41, torch.float16, bias_std=0.1)
+    a = nt.nested_tensor(xs, device=DEV, dtype=torch.float16)
+    g = torch.Generator().manual_seed(43)
+    W1 = (torch.randn(4 * E, E, generator=g) * E ** -0.5).half().to(DEV)
+    W2 = (torch.randn(E, 4 * E, generator=g) * (4 * E) ** -0.5).half().to(DEV)
+    b1, b2 = (torch.randn(4 * E, generator=g) * 0.1).half().to(DEV), (torch.randn(E, generator=g) * 0.1).half().to(DEV)
+    ln_w, ln_b = torch.ones(E, device=DEV).half(), torch.zeros(E, device=DEV).half()
+    dW_in, db_in, dW_out, db_out = (t.to(DEV) for t in (W_in, b_in, W_out, b_out))
+
+    def layer():
+        y = torch.ops.nestedtensor.min_mha(H, 64, 0.0, False, a, a, a, dW_in, db_in, 0.125, dW_out, db_out)
+        h = ops.layer_norm(y._impl, (E,), ln_w, ln_b, 1e-5, residual=a._impl)
+        f = ops.linear_nt(h, W1, b1, "gelu")
+        o = ops.linear_nt(f, W2, b2)
+        return ops.layer_norm(o, (E,), ln_w, ln_b, 1e-5, residual=h).buffer
+
+    for _ in range(3):
+        layer()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layer()
+        with torch.cuda.graph(graph, stream=side):
+            out = layer()
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        a._impl.buffer.copy_(torch.randn(a._impl.buffer.shape, generator=g).half().to(DEV))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        exp = layer()
+        torch.cuda.synchronize()
+        assert torch.isfinite(got).all()
+        assert torch.equal(got, exp), "replay %d differs from the eager layer" % rep

@@ -694,3 +694,43 @@ def test_pack_table_in_kernel_arguments_and_uploaded():
         assert torch.equal(a._impl.offsets_dev().cpu(), exp_off)
         if not a._impl.has_empty_constituent():
             bits_equal(a.to_padded_tensor(0), oracle.to_padded_tensor(ref, 0))
+
+
+def test_pad_unpad_mask_under_hip_graph_replays():
+    # pad, length-based un-pad and masks enqueue on the current stream, allocate through
+    # torch and never wait for the device, so they can be captured; every replay, with new
+    # contents in the packed buffer, must equal the eager result.  (The dense -> nested
+    # conversions size their output from device data and cannot be captured.)
+    g = torch.Generator().manual_seed(123)
+    parts = [torch.randn(int(l), 40, generator=g) for l in (5, 17, 1, 33, 12)]
+    a = nt.nested_tensor(parts, device=DEV)
+
+    def work():
+        padded = a.to_padded_tensor(-3.0)
+        data, mask = a.to_tensor_mask()
+        back = nt.from_padded_tensor(padded, a)
+        return padded, data, mask, back._impl.buffer
+
+    for _ in range(3):
+        work()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work()
+        with torch.cuda.graph(graph, stream=side):
+            outs = work()
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        a._impl.buffer.copy_(torch.randn(a._impl.buffer.shape, generator=g).to(DEV))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        exp = work()
+        torch.cuda.synchronize()
+        for x, y in zip(got, exp):
+            assert torch.equal(x, y), "replay %d differs from the eager call" % rep
+        ref = oracle.ref_nested_tensor([p.cpu() for p in a.unbind()])
+        bits_equal(got[0], oracle.to_padded_tensor(ref, -3.0))
+        bits_equal(got[3], ref.buffer)
