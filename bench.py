@@ -420,6 +420,21 @@ def bench_mha_c3(args, torch, dev, later):
         return _ops.layer_norm(o, (E,), ln_w, ln_b, 1e-5, residual=h)
 
     ms_enc = None if args.no_encoder else _time_gpu(torch, encoder_layer, iters=50, warmup=5)
+    enc_graph_ms = None
+    if ms_enc is not None:
+        # the seven launches replayed from a HIP graph
+        try:
+            egraph = torch.cuda.CUDAGraph()
+            eside = torch.cuda.Stream()
+            eside.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(eside):
+                encoder_layer()
+                with torch.cuda.graph(egraph, stream=eside):
+                    encoder_layer()
+            torch.cuda.current_stream().wait_stream(eside)
+            enc_graph_ms = float(_time_gpu(torch, egraph.replay, iters=50, warmup=5))
+        except Exception as exc:      # report, do not hide
+            enc_graph_ms = "graph capture failed: %r" % (exc,)
     flops_enc = flops + 16 * T * E * E
     res = dict(workload="C3: nested BERT-base self-attention, fp16, B=32, L~U[32,512], d=768, 12x64",
                tokens=T, ms_per_layer=float(ms), ms_per_layer_max=ms.max, ms_per_layer_mean=ms.mean,
@@ -431,7 +446,8 @@ def bench_mha_c3(args, torch, dev, later):
         res["encoder_layer"] = dict(
             workload="the same batch through a whole BERT-base encoder layer (attention, add + layer norm, "
                      "768-3072-768 feed-forward with gelu, add + layer norm), 7 launches",
-            ms_per_layer=float(ms_enc), ms_per_layer_max=ms_enc.max, tokens_per_s=T / (ms_enc * 1e-3),
+            ms_per_layer=float(ms_enc), ms_per_layer_max=ms_enc.max, ms_per_layer_hip_graph=enc_graph_ms,
+            tokens_per_s=T / (ms_enc * 1e-3),
             flops=flops_enc, TFLOPs=flops_enc / (ms_enc * 1e-3) / 1e12,
             frac_of_mfma_peak=flops_enc / (ms_enc * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS)
     if not args.no_cpu:
