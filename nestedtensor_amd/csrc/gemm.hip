@@ -30,6 +30,13 @@
 #include "nt_common.h"
 
 // Compile-time tuning knobs.
+// Measurement aid, never set in a product build: bits that take one ingredient
+// out of the K loop of the global -> LDS path so that its cost can be read off a
+// depth sweep (results are then wrong).  1: no MFMA, 2: no global -> LDS loads,
+// 4: fragments read once instead of every step, 8: no barrier.
+#ifndef NT_GEMM_ABLATE
+#define NT_GEMM_ABLATE 0
+#endif
 #ifndef NT_GEMM_FORCE_CFG
 #define NT_GEMM_FORCE_CFG (-1)           // 0, 1, 2: always that tile shape (experiments)
 #endif
@@ -246,6 +253,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
     static_assert(kNB >= 2 && (kNB - 2) * kN <= 63, "vmcnt is a 6-bit counter");
     auto dma_tile = [&](int buf, int64_t kt_in) {
       const int64_t kt = kt_in >= nk ? nk - 1 : kt_in;    // past the end: re-read, never used
+      if (NT_GEMM_ABLATE & 2) return;
 #pragma unroll
       for (int i = 0; i < kN; ++i) {
         const unsigned dst = __builtin_amdgcn_readfirstlane(
@@ -276,28 +284,40 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"((kNB - 2) * kN) : "memory");
     __syncthreads();
     int buf = 0;
+    Frag fa[2][WM], fb[2][WN];
+    if (NT_GEMM_ABLATE & 4) {
+      read_frags(fa[0], fb[0], 0, 0);
+      read_frags(fa[1], fb[1], 0, 1);
+    }
     for (int64_t kt = 0; kt < nk; ++kt) {
       const int buf_new = buf == 0 ? kNB - 1 : buf - 1;    // == (kt + kNB - 1) % kNB, free since the last barrier
       dma_tile(buf_new, kt + kNB - 1);
-      Frag fa[2][WM], fb[2][WN];
-      read_frags(fa[0], fb[0], buf, 0);
+      if (NT_GEMM_ABLATE & 4) {
+        asm volatile("" : "+v"(fa[0][0]), "+v"(fb[0][0]), "+v"(fa[1][0]), "+v"(fb[1][0]));
+      } else {
+        read_frags(fa[0], fb[0], buf, 0);
+      }
 #pragma unroll
       for (int s = 0; s < kSteps; ++s) {
-        if (s + 1 < kSteps) read_frags(fa[(s + 1) & 1], fb[(s + 1) & 1], buf, s + 1);
+        if (s + 1 < kSteps && !(NT_GEMM_ABLATE & 4)) read_frags(fa[(s + 1) & 1], fb[(s + 1) & 1], buf, s + 1);
+        if (NT_GEMM_ABLATE & 1) {
+          asm volatile("" ::"v"(fa[s & 1][0]), "v"(fb[s & 1][0]), "v"(fa[s & 1][WM - 1]), "v"(fb[s & 1][WN - 1]));
+        } else {
 #pragma unroll
-        for (int i = 0; i < WM; ++i)
+          for (int i = 0; i < WM; ++i)
 #pragma unroll
-          for (int jj = 0; jj < WN; ++jj) {
-            if (VT_OUT) {
-              acc[i][jj] = MM::run(fa[s & 1][i], fb[s & 1][jj], acc[i][jj]);
-            } else {
-              acc[i][jj] = MM::run(fb[s & 1][jj], fa[s & 1][i], acc[i][jj]);
+            for (int jj = 0; jj < WN; ++jj) {
+              if (VT_OUT) {
+                acc[i][jj] = MM::run(fa[s & 1][i], fb[s & 1][jj], acc[i][jj]);
+              } else {
+                acc[i][jj] = MM::run(fb[s & 1][jj], fa[s & 1][i], acc[i][jj]);
+              }
             }
-          }
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
       asm volatile("s_waitcnt vmcnt(%0)" :: "n"((kNB - 2) * kN) : "memory");
-      __syncthreads();
+      if (!(NT_GEMM_ABLATE & 8)) __syncthreads();
       buf = buf + 1 == kNB ? 0 : buf + 1;
     }
     // The last kNB - 1 iterations issued clamped re-reads of the last K tile; up to
