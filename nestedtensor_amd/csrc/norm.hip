@@ -197,7 +197,9 @@ static int launch_layer_norm(const void* x, const void* residual, const void* ga
   if (n % kPer == 0 && align % 16 == 0 && pieces <= kWave * 4 * 4) {
     if (pieces <= 64) return launch_layer_norm_vec<T, 1, 1>(x, residual, gamma, beta, out, rows, n, eps, stream);
     if (pieces <= 128) return launch_layer_norm_vec<T, 2, 1>(x, residual, gamma, beta, out, rows, n, eps, stream);
-    if (pieces <= 256) return launch_layer_norm_vec<T, 1, 4>(x, residual, gamma, beta, out, rows, n, eps, stream);
+    // up to 4 KiB a wavefront keeps the whole row (no barrier, no LDS): measured 4.7 against
+    // 3.9 TB/s for 4 KiB rows shared by four wavefronts; at 8 KiB the shared row wins (4.8 : 3.6)
+    if (pieces <= 256) return launch_layer_norm_vec<T, 4, 1>(x, residual, gamma, beta, out, rows, n, eps, stream);
     if (pieces <= 512) return launch_layer_norm_vec<T, 2, 4>(x, residual, gamma, beta, out, rows, n, eps, stream);
     return launch_layer_norm_vec<T, 4, 4>(x, residual, gamma, beta, out, rows, n, eps, stream);
   }
