@@ -673,7 +673,8 @@ def test_many_short_rows(kind, dtype):
         bits_equal(again._impl.buffer, ref.buffer)
 
 
-def test_pack_table_in_kernel_arguments_and_uploaded():
+@pytest.mark.parametrize("dtype", [torch.float32, torch.uint8, torch.float16, torch.float64])
+def test_pack_table_in_kernel_arguments_and_uploaded(dtype):
     # up to nt_pack_table_max_entries() int64 of metadata ride in the kernel arguments of
     # the pack launch, which also writes their device copy; larger batches upload the
     # table first.  Both sides of the limit, empty constituents, and the adopted metadata.
@@ -682,10 +683,10 @@ def test_pack_table_in_kernel_arguments_and_uploaded():
     g = torch.Generator().manual_seed(91)
     for B, D in ((1, 1), (16, 3), (limit // 4, 2), (limit // 4 + 5, 2), (3, 2)):
         shapes = [[int(v) for v in torch.randint(0 if B == 3 else 1, 9, (D,), generator=g)] for _ in range(B)]
-        parts = [torch.randn(*s, generator=g) for s in shapes]
+        parts = [(torch.randn(*s, generator=g) * 40).to(dtype) for s in shapes]
         dev_parts = [p.to(DEV) for p in parts]
-        a = nt.nested_tensor(dev_parts, device=DEV)
-        ref = oracle.ref_nested_tensor(parts)
+        a = nt.nested_tensor(dev_parts, device=DEV, dtype=dtype)
+        ref = oracle.ref_nested_tensor(parts, dtype=dtype)
         bits_equal(a._impl.buffer, ref.buffer)
         assert a.nested_size().unbind() == [torch.Size(p.shape) for p in parts]
         assert torch.equal(a._impl.sizes_dev().cpu(), a._impl.sizes)
