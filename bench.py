@@ -216,9 +216,10 @@ def bench_c5(args, torch, dev):
 
 
 def pmc_probe(args, torch, dev):
-    """Three dispatches for hardware-counter runs: a plain device copy of 4 GiB
-    (reads 4 GiB, writes 4 GiB: the calibration for the counters' unit), one
-    nt_add_padding and one nt_remove_padding launch on the first C5 chunk."""
+    """Dispatches for hardware-counter runs: a plain device copy of 4 GiB (reads
+    4 GiB, writes 4 GiB: the calibration for the counters' unit), one
+    nt_add_padding and one nt_remove_padding launch on the first C5 chunk, then
+    one launch each of the short-row kernels on C2."""
     from nestedtensor_amd import _C
     from nestedtensor_amd.impl import NestedTensorImpl
     _, packed, chunks = build_c5(torch, NestedTensorImpl, dev, args.chunk, args.chunk)
@@ -239,9 +240,27 @@ def pmc_probe(args, torch, dev):
                                       m.B, 2, 1, _C.i64_array(ext), eb, stream))
     torch.cuda.synchronize()
     assert torch.equal(back.view(torch.int16), m.buffer.view(torch.int16))
-    print(json.dumps({"copy_bytes_read": src.numel() * 2, "copy_bytes_written": src.numel() * 2,
-                      "pad_valid_bytes": m.numel() * eb, "pad_padded_bytes": padded.numel() * eb,
-                      "unpad_valid_bytes": m.numel() * eb}))
+    info = {"copy_bytes_read": src.numel() * 2, "copy_bytes_written": src.numel() * 2,
+            "pad_valid_bytes": m.numel() * eb, "pad_padded_bytes": padded.numel() * eb,
+            "unpad_valid_bytes": m.numel() * eb}
+    del src, dst, padded, back, packed, chunks
+    # then the short-row kernels on C2 (16 fp32 images [3, H, W]), one launch each through
+    # the package: pad, mask, length-based un-pad, pack of device tensors, row counts + un-pad
+    import nestedtensor_amd as nt
+    g = torch.Generator().manual_seed(1010 + 1)
+    hw = torch.randint(480, 1025, (16, 2), generator=g)
+    imgs = [torch.rand(3, int(h), int(w), generator=g).to(dev) for h, w in hw]
+    a2 = nt.nested_tensor(imgs, device=dev)           # pack
+    padded2 = a2.to_padded_tensor(0)                  # pad
+    mask2 = torch.ops.nestedtensor.to_mask(a2, 4)     # mask
+    back2 = nt.from_padded_tensor(padded2, a2)        # un-pad
+    again = nt.nested_tensor_from_tensor_mask(padded2, mask2)   # row counts, un-pad
+    torch.cuda.synchronize()
+    assert torch.equal(back2._impl.buffer, a2._impl.buffer) and torch.equal(again._impl.buffer, a2._impl.buffer)
+    info.update(c2_valid_bytes=a2.numel() * 4, c2_padded_bytes=padded2.numel() * 4, c2_mask_bytes=mask2.numel(),
+                c2_launch_order="pack_table_kernel, row_group_kernel<4,0> (pad), mask_plane_kernel, "
+                                "row_group_kernel<4,1> (un-pad), row_counts_kernel, row_group_kernel<4,1>")
+    print(json.dumps(info))
 
 
 def mha_probe(args, torch, dev):
