@@ -790,6 +790,81 @@ Tensor mha_self_packed(const Tensor& x, const Tensor& schedule, int64_t num_head
   return out;
 }
 
+// ---- row-wise operators on the packed buffer ------------------------------------
+
+const void* opt_ptr(const c10::optional<Tensor>& t) {
+  return (t.has_value() && t->defined()) ? t->const_data_ptr() : nullptr;
+}
+
+// nt_layer_norm over the packed [rows, n] view of x; residual (same shape) is added
+// first.  The caller has checked the nested sizes.
+Tensor layer_norm_packed(const Tensor& x, const c10::optional<Tensor>& residual, const c10::optional<Tensor>& weight,
+                         const c10::optional<Tensor>& bias, int64_t n, double eps) {
+  require_device(x, "layer_norm");
+  TORCH_CHECK(x.is_contiguous() && n > 0 && x.numel() % n == 0, "layer_norm: the buffer must hold whole rows of ", n);
+  for (const auto* t : {&residual, &weight, &bias}) {
+    TORCH_CHECK(!t->has_value() || !(*t)->defined() ||
+                    ((*t)->scalar_type() == x.scalar_type() && (*t)->device() == x.device() && (*t)->is_contiguous()),
+                "layer_norm: operands must be contiguous tensors of the input's dtype on the input's device");
+  }
+  TORCH_CHECK(!residual.has_value() || !residual->defined() || residual->numel() == x.numel(),
+              "layer_norm: the residual must have the size of the input");
+  c10::hip::HIPGuard guard(x.device().index());
+  Tensor out = at::empty_like(x);
+  check(nt_layer_norm(x.const_data_ptr(), opt_ptr(residual), opt_ptr(weight), opt_ptr(bias), out.data_ptr(),
+                      x.numel() / n, n, eps, dtype_code(x.scalar_type()), stream_of(x)));
+  return out;
+}
+
+// mul == false: out[i] = a[i] + scale * b[i % period]; mul == true: out[i] = scale * a[i] * b[i % period]
+// (b absent: scale * a[i]).
+Tensor binary_packed(const Tensor& a, const c10::optional<Tensor>& b, double scale, int64_t period, bool mul) {
+  require_device(a, mul ? "mul" : "add");
+  const bool has_b = b.has_value() && b->defined();
+  TORCH_CHECK(mul || has_b, "add: the second operand is missing");
+  TORCH_CHECK(a.is_contiguous() && (!has_b || (b->is_contiguous() && b->scalar_type() == a.scalar_type() &&
+                                               b->device() == a.device())),
+              mul ? "mul" : "add", ": both operands must have the same dtype and device");
+  TORCH_CHECK(!has_b || (period > 0 && b->numel() >= period), "packed binary op: operand shorter than its period");
+  c10::hip::HIPGuard guard(a.device().index());
+  Tensor out = at::empty_like(a);
+  if (a.numel() == 0) return out;
+  const int dt = dtype_code(a.scalar_type());
+  if (mul) {
+    check(nt_mul_packed(a.const_data_ptr(), opt_ptr(b), scale, out.data_ptr(), a.numel(), period, dt, stream_of(a)));
+  } else {
+    check(nt_add_packed(a.const_data_ptr(), b->const_data_ptr(), scale, out.data_ptr(), a.numel(), period, dt,
+                        stream_of(a)));
+  }
+  return out;
+}
+
+Tensor softmax_rows(const Tensor& x, const Tensor& offsets, const Tensor& row_offsets, int64_t total_rows, bool log) {
+  require_device(x, log ? "log_softmax" : "softmax");
+  TORCH_CHECK(x.is_contiguous() && offsets.scalar_type() == at::kLong && row_offsets.scalar_type() == at::kLong &&
+                  offsets.device() == x.device() && row_offsets.device() == x.device() &&
+                  offsets.numel() == row_offsets.numel() && offsets.numel() >= 1,
+              "softmax: offsets and row offsets must be int64 [B + 1] tensors on the buffer's device");
+  c10::hip::HIPGuard guard(x.device().index());
+  Tensor out = at::empty_like(x);
+  if (x.numel() == 0) return out;
+  check(nt_softmax_rows(x.const_data_ptr(), out.data_ptr(), offsets.const_data_ptr<int64_t>(),
+                        row_offsets.const_data_ptr<int64_t>(), offsets.numel() - 1, total_rows, log ? 1 : 0,
+                        dtype_code(x.scalar_type()), stream_of(x)));
+  return out;
+}
+
+Tensor activation_packed(const Tensor& x, int64_t act) {
+  require_device(x, "activation");
+  TORCH_CHECK(x.is_contiguous() && (act == 1 || act == 2), "activation: relu (1) or gelu (2) of a contiguous buffer");
+  c10::hip::HIPGuard guard(x.device().index());
+  Tensor out = at::empty_like(x);
+  if (x.numel() == 0) return out;
+  check(nt_activation_packed(x.const_data_ptr(), out.data_ptr(), x.numel(), static_cast<int>(act),
+                             dtype_code(x.scalar_type()), stream_of(x)));
+  return out;
+}
+
 // ---- consumers of the offsets array ---------------------------------------------
 
 // After a kernel that may have counted out-of-range indices: the running count
@@ -975,6 +1050,10 @@ TORCH_LIBRARY(nestedtensor, m) {
         "Tensor? mirror) -> Tensor");
   m.def("packed_sequence_lowered(Tensor buffer, Tensor lengths, Tensor row_offsets, int row_elems) -> "
         "(Tensor, Tensor, Tensor, Tensor)");
+  m.def("layer_norm_packed(Tensor x, Tensor? residual, Tensor? weight, Tensor? bias, int n, float eps) -> Tensor");
+  m.def("binary_packed(Tensor a, Tensor? b, float scale, int period, bool mul) -> Tensor");
+  m.def("softmax_rows(Tensor x, Tensor offsets, Tensor row_offsets, int total_rows, bool log) -> Tensor");
+  m.def("activation_packed(Tensor x, int act) -> Tensor");
   m.def("linear_packed(Tensor x, Tensor weight, Tensor? bias, int act) -> Tensor");
   m.def("mha_self_packed(Tensor x, Tensor schedule, int num_heads, int head_dim, Tensor in_proj_weight, "
         "Tensor? in_proj_bias, float scaling, Tensor out_proj_weight, Tensor? out_proj_bias) -> Tensor");
@@ -992,6 +1071,10 @@ TORCH_LIBRARY_IMPL(nestedtensor, CUDA, m) {
   m.impl("nt_from_padded_tensor", nt_from_padded_tensor_op);
   m.impl("linear_packed", linear_packed);
   m.impl("mha_self_packed", mha_self_packed);
+  m.impl("layer_norm_packed", layer_norm_packed);
+  m.impl("binary_packed", binary_packed);
+  m.impl("softmax_rows", softmax_rows);
+  m.impl("activation_packed", activation_packed);
   m.impl("embedding_packed", embedding_packed);
   m.impl("embedding_bag_packed", embedding_bag_packed);
   m.impl("packed_sequence_lowered", packed_sequence_lowered);

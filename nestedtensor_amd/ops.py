@@ -27,6 +27,10 @@ _remove_padding = _C.ops.remove_padding.default
 _build_mask = _C.ops.build_mask.default
 _linear_packed = _C.ops.linear_packed.default
 _mha_self_packed = _C.ops.mha_self_packed.default
+_layer_norm_packed = _C.ops.layer_norm_packed.default
+_binary_packed = _C.ops.binary_packed.default
+_softmax_rows = _C.ops.softmax_rows.default
+_activation_packed = _C.ops.activation_packed.default
 _embedding_packed = _C.ops.embedding_packed.default
 _embedding_bag_packed = _C.ops.embedding_bag_packed.default
 _packed_sequence_lowered = _C.ops.packed_sequence_lowered.default
@@ -350,12 +354,7 @@ def activation(impl, kind):
     storage layout does not matter."""
     buf = impl.buffer
     _C.require_device(buf, kind)
-    out = torch.empty_like(buf)
-    if buf.numel() > 0:
-        with _C.on_device(buf.device):
-            _C.check(_C.lib.nt_activation_packed(_C.ptr(buf), _C.ptr(out), buf.numel(), _ACTS[kind],
-                                                 _C.dtype_code(buf.dtype), _C.current_stream(buf.device)))
-    return impl.with_buffer(out)
+    return impl.with_buffer(_activation_packed(buf, _ACTS[kind]))
 
 
 def _check_mha_inputs(query, key, value):
@@ -530,15 +529,11 @@ def layer_norm(impl, normalized_shape, weight=None, bias=None, eps=1e-5, residua
         if not torch.equal(residual.sizes, impl.sizes) or residual.buffer.dtype != buf.dtype:
             raise RuntimeError("layer_norm: the residual must have the nested size and dtype of the input")
         res_buf = residual.buffer
-    out = torch.empty_like(buf)
-    rows = buf.numel() // n if n > 0 else 0
+    if n == 0 or buf.numel() == 0:
+        return impl.with_buffer(torch.empty_like(buf))
     weight = weight.contiguous() if weight is not None else None
     bias = bias.contiguous() if bias is not None else None
-    with _C.on_device(buf.device):
-        _C.check(_C.lib.nt_layer_norm(_C.ptr(buf), _C.ptr(res_buf), _C.ptr(weight), _C.ptr(bias),
-                                      _C.ptr(out), rows, n, float(eps), _C.dtype_code(buf.dtype),
-                                      _C.current_stream(buf.device)))
-    return impl.with_buffer(out)
+    return impl.with_buffer(_layer_norm_packed(buf, res_buf, weight, bias, n, float(eps)))
 
 
 def add(impl, other, alpha=1):
@@ -568,12 +563,7 @@ def add(impl, other, alpha=1):
                                   "are on the packed path.")
     if b.dtype != buf.dtype or b.device != buf.device:
         raise RuntimeError("add: both operands must have the same dtype and device")
-    out = torch.empty_like(buf)
-    if buf.numel() > 0:
-        with _C.on_device(buf.device):
-            _C.check(_C.lib.nt_add_packed(_C.ptr(buf), _C.ptr(b), float(alpha), _C.ptr(out), buf.numel(),
-                                          period, _C.dtype_code(buf.dtype), _C.current_stream(buf.device)))
-    return impl.with_buffer(out)
+    return impl.with_buffer(_binary_packed(buf, b, float(alpha), period, False))
 
 
 def softmax(impl, dim, dtype=None, log=False):
@@ -596,16 +586,10 @@ def softmax(impl, dim, dtype=None, log=False):
     if dtype is not None and dtype != buf.dtype:
         buf = buf.to(dtype)
         impl = impl.with_buffer(buf)
-    out = torch.empty_like(buf)
-    B, D = impl.B, impl.D
     if buf.numel() == 0:
-        return impl.with_buffer(out)
+        return impl.with_buffer(torch.empty_like(buf))
     row_offsets, total_rows = impl.last_dim_rows()
-    with _C.on_device(buf.device):
-        _C.check(_C.lib.nt_softmax_rows(_C.ptr(buf), _C.ptr(out), _C.ptr(impl.offsets_dev()),
-                                        _C.ptr(row_offsets), B, total_rows, 1 if log else 0,
-                                        _C.dtype_code(buf.dtype), _C.current_stream(buf.device)))
-    return impl.with_buffer(out)
+    return impl.with_buffer(_softmax_rows(buf, impl.offsets_dev(), row_offsets, total_rows, bool(log)))
 
 
 def mul(impl, other):
@@ -634,12 +618,7 @@ def mul(impl, other):
     buf = impl.buffer
     if b is not None and (b.dtype != buf.dtype or b.device != buf.device):
         raise RuntimeError("mul: both operands must have the same dtype and device")
-    out = torch.empty_like(buf)
-    if buf.numel() > 0:
-        with _C.on_device(buf.device):
-            _C.check(_C.lib.nt_mul_packed(_C.ptr(buf), _C.ptr(b), scale, _C.ptr(out), buf.numel(), period,
-                                          _C.dtype_code(buf.dtype), _C.current_stream(buf.device)))
-    return impl.with_buffer(out)
+    return impl.with_buffer(_binary_packed(buf, b, scale, period, True))
 
 
 def matmul(impl, other):
