@@ -996,6 +996,140 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> packed_sequence_lowered(const Tensor&
   return std::make_tuple(data, batch_sizes, sorted_dev, rank_dev);
 }
 
+// One projection of the packed rows x [T, K] with rows [r0, r0 + n) of W and of the bias.
+Tensor project_rows(const Tensor& x, const Tensor& W, const Tensor& bias, int64_t r0, int64_t n, void* stream) {
+  const int64_t T = x.size(0), K = x.size(1);
+  Tensor out = at::empty({T, n}, x.options());
+  if (T == 0) return out;
+  const char* w = static_cast<const char*>(W.const_data_ptr()) + r0 * K * static_cast<int64_t>(W.element_size());
+  const char* b = bias.defined() ? static_cast<const char*>(bias.const_data_ptr()) + r0 * static_cast<int64_t>(bias.element_size())
+                                 : nullptr;
+  check(nt_linear_act(x.const_data_ptr(), x.stride(0), w, b, out.data_ptr(), n, T, n, K, 0, dtype_code(x.scalar_type()),
+                      stream));
+  return out;
+}
+
+void check_mha_operands(const Tensor& xq, const Tensor& xk, const Tensor& xv, int64_t E, const Tensor& W,
+                        const Tensor& b_in, const Tensor& Wo, const Tensor& b_out) {
+  const at::ScalarType st = xq.scalar_type();
+  for (const Tensor* t : {&xq, &xk, &xv}) {
+    TORCH_CHECK(t->dim() == 2 && t->size(1) == E && t->stride(1) == 1 && t->scalar_type() == st &&
+                    t->device() == xq.device(),
+                "mha: query, key and value must be [tokens, num_heads * head_dim] views of one dtype and device");
+  }
+  TORCH_CHECK(W.dim() == 2 && W.size(0) == 3 * E && W.size(1) == E,
+              "in_proj_weight must have shape [3 * embed_dim, embed_dim].");
+  TORCH_CHECK(W.scalar_type() == st && Wo.scalar_type() == st && (!b_in.defined() || b_in.scalar_type() == st) &&
+                  (!b_out.defined() || b_out.scalar_type() == st),
+              "linear: input, weight and bias must have the same dtype");
+  TORCH_CHECK(Wo.dim() == 2 && Wo.size(1) == E, "linear: weight of shape ", Wo.sizes(),
+              " does not match input feature size ", E);
+}
+
+// Attention between different nested tensors (or with an embedding size the fused
+// projection does not tile), f16 / bf16, head_dim 32 / 64 / 128 (min_mha,
+// mha.cpp:42-65): three projections, the value one written transposed, the
+// attention kernel with one key sequence per query sequence, output projection.
+Tensor mha_cross_packed(const Tensor& xq, const Tensor& xk, const Tensor& xv, const Tensor& schedule, int64_t num_heads,
+                        int64_t head_dim, const Tensor& in_proj_weight, const c10::optional<Tensor>& in_proj_bias,
+                        double scaling, const Tensor& out_proj_weight, const c10::optional<Tensor>& out_proj_bias) {
+  require_device(xq, "multi-head attention");
+  const int64_t E = num_heads * head_dim;
+  const Tensor W = in_proj_weight.contiguous(), Wo = out_proj_weight.contiguous();
+  Tensor b_in, b_out;
+  if (in_proj_bias.has_value() && in_proj_bias->defined()) b_in = in_proj_bias->contiguous();
+  if (out_proj_bias.has_value() && out_proj_bias->defined()) b_out = out_proj_bias->contiguous();
+  check_mha_operands(xq, xk, xv, E, W, b_in, Wo, b_out);
+  TORCH_CHECK(schedule.scalar_type() == at::kInt && schedule.dim() == 2 && schedule.size(1) == 8 &&
+                  schedule.is_contiguous() && schedule.device() == xq.device(),
+              "mha: schedule must be a contiguous int32 [n_work, 8] tensor on the input's device");
+  const int64_t Tq = xq.size(0), Tk = xk.size(0), N = Wo.size(0);
+  TORCH_CHECK(xv.size(0) == Tk, "key and value must have the same nested size.");
+  c10::hip::HIPGuard guard(xq.device().index());
+  void* stream = stream_of(xq);
+  const int dt = dtype_code(xq.scalar_type());
+  Tensor out = at::empty({Tq, N}, xq.options());
+  if (Tq == 0) return out;
+  Tensor q = project_rows(xq, W, b_in, 0, E, stream);
+  Tensor k = project_rows(xk, W, b_in, E, E, stream);
+  const int64_t ldvt = (Tk + 72 + 7) / 8 * 8;
+  Tensor vt = at::empty({E, ldvt}, xq.options());
+  const int64_t es = static_cast<int64_t>(xq.element_size());
+  check(nt_linear_transposed(xv.const_data_ptr(), xv.stride(0),
+                             static_cast<const char*>(W.const_data_ptr()) + 2 * E * E * es,
+                             b_in.defined() ? static_cast<const char*>(b_in.const_data_ptr()) + 2 * E * es : nullptr,
+                             vt.data_ptr(), ldvt, Tk, E, E, dt, stream));
+  Tensor attn = at::empty({Tq, E}, xq.options());
+  check(nt_varlen_attention_vt(q.const_data_ptr(), E, k.const_data_ptr(), E, vt.const_data_ptr(), ldvt, attn.data_ptr(), E,
+                               schedule.const_data_ptr<int32_t>(), schedule.size(0), num_heads, head_dim, Tk,
+                               static_cast<float>(scaling), dt, stream));
+  check(nt_linear_act(attn.const_data_ptr(), E, Wo.const_data_ptr(), b_out.defined() ? b_out.const_data_ptr() : nullptr,
+                      out.data_ptr(), N, Tq, N, E, 0, dt, stream));
+  return out;
+}
+
+// The same layer with V row-major: fp32 with head_dim 32 / 64 / 128 from the work
+// list (`schedule`), anything else over the device row offsets on a padded grid.
+// `same`: query, key and value are one nested tensor (one [T, 3E] projection).
+Tensor mha_rowmajor_packed(const Tensor& xq, const Tensor& xk, const Tensor& xv, bool same,
+                           const c10::optional<Tensor>& schedule, const Tensor& q_offsets, const Tensor& kv_offsets,
+                           int64_t max_q, int64_t num_heads, int64_t head_dim, const Tensor& in_proj_weight,
+                           const c10::optional<Tensor>& in_proj_bias, double scaling, const Tensor& out_proj_weight,
+                           const c10::optional<Tensor>& out_proj_bias) {
+  require_device(xq, "multi-head attention");
+  const int64_t E = num_heads * head_dim;
+  const Tensor W = in_proj_weight.contiguous(), Wo = out_proj_weight.contiguous();
+  Tensor b_in, b_out;
+  if (in_proj_bias.has_value() && in_proj_bias->defined()) b_in = in_proj_bias->contiguous();
+  if (out_proj_bias.has_value() && out_proj_bias->defined()) b_out = out_proj_bias->contiguous();
+  check_mha_operands(xq, xk, xv, E, W, b_in, Wo, b_out);
+  const int64_t Tq = xq.size(0), N = Wo.size(0), B = q_offsets.numel() - 1;
+  TORCH_CHECK(q_offsets.scalar_type() == at::kLong && kv_offsets.scalar_type() == at::kLong &&
+                  kv_offsets.numel() == q_offsets.numel() && q_offsets.device() == xq.device() &&
+                  kv_offsets.device() == xq.device(),
+              "mha: row offsets must be int64 [B + 1] tensors on the input's device");
+  c10::hip::HIPGuard guard(xq.device().index());
+  void* stream = stream_of(xq);
+  const int dt = dtype_code(xq.scalar_type());
+  Tensor out = at::empty({Tq, N}, xq.options());
+  if (Tq == 0) return out;
+  Tensor q, k, v;
+  int64_t qc = 0, kc = 0, vc = 0, ld = E;
+  if (same) {
+    q = project_rows(xq, W, b_in, 0, 3 * E, stream);     // [T, 3E]
+    k = q;
+    v = q;
+    kc = E;
+    vc = 2 * E;
+    ld = 3 * E;
+  } else {
+    q = project_rows(xq, W, b_in, 0, E, stream);
+    k = project_rows(xk, W, b_in, E, E, stream);
+    v = project_rows(xv, W, b_in, 2 * E, E, stream);
+  }
+  const int64_t es = static_cast<int64_t>(xq.element_size());
+  const char* qp = static_cast<const char*>(q.const_data_ptr()) + qc * es;
+  const char* kp = static_cast<const char*>(k.const_data_ptr()) + kc * es;
+  const char* vp = static_cast<const char*>(v.const_data_ptr()) + vc * es;
+  Tensor attn = at::empty({Tq, E}, xq.options());
+  const bool listed = schedule.has_value() && schedule->defined() && xq.scalar_type() == at::kFloat &&
+                      (head_dim == 32 || head_dim == 64 || head_dim == 128);
+  if (listed) {
+    TORCH_CHECK(schedule->scalar_type() == at::kInt && schedule->dim() == 2 && schedule->size(1) == 8 &&
+                    schedule->is_contiguous() && schedule->device() == xq.device(),
+                "mha: schedule must be a contiguous int32 [n_work, 8] tensor on the input's device");
+    check(nt_varlen_attention_scheduled(qp, ld, kp, ld, vp, ld, attn.data_ptr(), E, schedule->const_data_ptr<int32_t>(),
+                                        schedule->size(0), num_heads, head_dim, static_cast<float>(scaling), dt, stream));
+  } else {
+    check(nt_varlen_attention(qp, ld, kp, ld, vp, ld, attn.data_ptr(), E, q_offsets.const_data_ptr<int64_t>(),
+                              kv_offsets.const_data_ptr<int64_t>(), B, num_heads, head_dim, max_q,
+                              static_cast<float>(scaling), dt, stream));
+  }
+  check(nt_linear_act(attn.const_data_ptr(), E, Wo.const_data_ptr(), b_out.defined() ? b_out.const_data_ptr() : nullptr,
+                      out.data_ptr(), N, Tq, N, E, 0, dt, stream));
+  return out;
+}
+
 }  // namespace
 
 // Schemas.  The first block are the reference's operators, names and argument
@@ -1057,6 +1191,12 @@ TORCH_LIBRARY(nestedtensor, m) {
   m.def("linear_packed(Tensor x, Tensor weight, Tensor? bias, int act) -> Tensor");
   m.def("mha_self_packed(Tensor x, Tensor schedule, int num_heads, int head_dim, Tensor in_proj_weight, "
         "Tensor? in_proj_bias, float scaling, Tensor out_proj_weight, Tensor? out_proj_bias) -> Tensor");
+  m.def("mha_cross_packed(Tensor xq, Tensor xk, Tensor xv, Tensor schedule, int num_heads, int head_dim, "
+        "Tensor in_proj_weight, Tensor? in_proj_bias, float scaling, Tensor out_proj_weight, "
+        "Tensor? out_proj_bias) -> Tensor");
+  m.def("mha_rowmajor_packed(Tensor xq, Tensor xk, Tensor xv, bool same, Tensor? schedule, Tensor q_offsets, "
+        "Tensor kv_offsets, int max_q, int num_heads, int head_dim, Tensor in_proj_weight, Tensor? in_proj_bias, "
+        "float scaling, Tensor out_proj_weight, Tensor? out_proj_bias) -> Tensor");
 }
 
 // "CUDA" is the dispatch key of the HIP device on PyTorch-ROCm.
@@ -1071,6 +1211,8 @@ TORCH_LIBRARY_IMPL(nestedtensor, CUDA, m) {
   m.impl("nt_from_padded_tensor", nt_from_padded_tensor_op);
   m.impl("linear_packed", linear_packed);
   m.impl("mha_self_packed", mha_self_packed);
+  m.impl("mha_cross_packed", mha_cross_packed);
+  m.impl("mha_rowmajor_packed", mha_rowmajor_packed);
   m.impl("layer_norm_packed", layer_norm_packed);
   m.impl("binary_packed", binary_packed);
   m.impl("softmax_rows", softmax_rows);

@@ -27,6 +27,8 @@ _remove_padding = _C.ops.remove_padding.default
 _build_mask = _C.ops.build_mask.default
 _linear_packed = _C.ops.linear_packed.default
 _mha_self_packed = _C.ops.mha_self_packed.default
+_mha_cross_packed = _C.ops.mha_cross_packed.default
+_mha_rowmajor_packed = _C.ops.mha_rowmajor_packed.default
 _layer_norm_packed = _C.ops.layer_norm_packed.default
 _binary_packed = _C.ops.binary_packed.default
 _softmax_rows = _C.ops.softmax_rows.default
@@ -366,11 +368,6 @@ def _check_mha_inputs(query, key, value):
         raise RuntimeError("value needs to be 3 dim.")
 
 
-def _offset_ptr(t, col):
-    import ctypes
-    return ctypes.c_void_p(t.data_ptr() + col * t.element_size())
-
-
 def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_bias, scaling,
                out_proj_weight, out_proj_bias):
     """Nested multi-head attention on packed buffers.  Semantics of min_mha
@@ -391,7 +388,6 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
     if not torch.equal(key.sizes, value.sizes):
         raise RuntimeError("key and value must have the same nested size.")
     _C.require_device(query.buffer, "multi-head attention")
-    dev = query.buffer.device
     dtype = query.buffer.dtype
     W = in_proj_weight.contiguous()
     if tuple(W.shape) != (3 * E, E):
@@ -400,9 +396,7 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
     same = (key is query or key.buffer.data_ptr() == query.buffer.data_ptr()) and \
         (value is query or value.buffer.data_ptr() == query.buffer.data_ptr()) and \
         torch.equal(key.sizes, query.sizes)
-    T_tokens = xq.size(0)
     max_q = int(query.sizes[:, 0].max()) if query.B > 0 else 0
-    attn = torch.empty((T_tokens, E), dtype=dtype, device=dev)
     mfma_path = head_dim in (32, 64, 128) and dtype in (torch.float16, torch.bfloat16)
     fused = same and mfma_path and (2 * E) % 128 == 0
     if in_proj_bias is not None:
@@ -418,58 +412,25 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
         out = _mha_self_packed(xq, query.attention_schedule(), num_heads, head_dim, W, in_proj_bias,
                                float(scaling), out_proj_weight, out_proj_bias)
         return query.with_buffer(out.reshape(-1))
-    elif mfma_path and bool((key.sizes[:, 0] > 0).all()):
+    xk, xv = key.buffer.reshape(-1, E), value.buffer.reshape(-1, E)
+    if mfma_path and bool((key.sizes[:, 0] > 0).all()):
         # cross-attention (or an embedding size the fused projection does not tile),
         # head_dim 32 / 64 / 128: three projections (the value one written
         # transposed), then the same attention kernel with one key sequence per
-        # query sequence
-        b = in_proj_bias
-        T_kv = key.buffer.numel() // E
-        q_t = linear(xq, W[0:E], None if b is None else b[0:E])
-        k_t = linear(key.buffer.reshape(-1, E), W[E:2 * E], None if b is None else b[E:2 * E])
-        ldvt = (T_kv + 72 + 7) // 8 * 8
-        vt = torch.empty((E, ldvt), dtype=dtype, device=dev)
-        xv = value.buffer.reshape(-1, E)
-        bv = None if b is None else b[2 * E:].contiguous()
-        with _C.on_device(dev):
-            stream = _C.current_stream(dev)
-            _C.check(_C.lib.nt_linear_transposed(
-                _C.ptr(xv), xv.stride(0), _C.ptr(W[2 * E:]), _C.ptr(bv), _C.ptr(vt), ldvt, T_kv, E, E,
-                _C.dtype_code(dtype), stream))
-            sched = query.attention_schedule(kv=key)
-            _C.check(_C.lib.nt_varlen_attention_vt(
-                _C.ptr(q_t), E, _C.ptr(k_t), E, _C.ptr(vt), ldvt, _C.ptr(attn), E,
-                _C.ptr(sched), sched.size(0), num_heads, head_dim, T_kv,
-                float(scaling), _C.dtype_code(dtype), stream))
-    else:
-        if same:
-            qkv = linear(xq, W, in_proj_bias)                       # [T, 3E]
-            q_t, k_t, v_t = qkv, qkv, qkv
-            qc, kc, vc = 0, E, 2 * E
-            ldq = ldk = ldv = 3 * E
-        else:
-            b = in_proj_bias
-            q_t = linear(xq, W[0:E], None if b is None else b[0:E])
-            k_t = linear(key.buffer.reshape(-1, E), W[E:2 * E], None if b is None else b[E:2 * E])
-            v_t = linear(value.buffer.reshape(-1, E), W[2 * E:], None if b is None else b[2 * E:])
-            qc = kc = vc = 0
-            ldq = ldk = ldv = E
-        with _C.on_device(dev):
-            if dtype == torch.float32 and head_dim in (32, 64, 128):
-                # fp32 on the fp32 matrix instruction, from the work list: only tiles
-                # that exist, longest key sequences first
-                sched = query.attention_schedule(kv=None if same else key)
-                _C.check(_C.lib.nt_varlen_attention_scheduled(
-                    _offset_ptr(q_t, qc), ldq, _offset_ptr(k_t, kc), ldk, _offset_ptr(v_t, vc), ldv,
-                    _C.ptr(attn), E, _C.ptr(sched), sched.size(0), num_heads, head_dim, float(scaling),
-                    _C.dtype_code(dtype), _C.current_stream(dev)))
-            else:
-                _C.check(_C.lib.nt_varlen_attention(
-                    _offset_ptr(q_t, qc), ldq, _offset_ptr(k_t, kc), ldk, _offset_ptr(v_t, vc), ldv,
-                    _C.ptr(attn), E, _C.ptr(query.row_offsets_dev()), _C.ptr(key.row_offsets_dev()),
-                    query.B, num_heads, head_dim, max_q, float(scaling), _C.dtype_code(dtype),
-                    _C.current_stream(dev)))
-    out = linear(attn, out_proj_weight, out_proj_bias)
+        # query sequence: five launches issued by one call into the extension
+        out = _mha_cross_packed(xq, xk, xv, query.attention_schedule(kv=key), num_heads, head_dim, W,
+                                in_proj_bias, float(scaling), out_proj_weight, out_proj_bias)
+        return query.with_buffer(out.reshape(-1))
+    # V row-major: fp32 with head_dim 32 / 64 / 128 on the fp32 matrix instruction from
+    # the work list (only tiles that exist, longest key sequences first), anything else
+    # (other head dims, key sequences without keys) on the generic kernels over the
+    # device row offsets
+    sched = None
+    if dtype == torch.float32 and head_dim in (32, 64, 128):
+        sched = query.attention_schedule(kv=None if same else key)
+    out = _mha_rowmajor_packed(xq, xk, xv, same, sched, query.row_offsets_dev(), key.row_offsets_dev(), max_q,
+                               num_heads, head_dim, W, in_proj_bias, float(scaling), out_proj_weight,
+                               out_proj_bias)
     return query.with_buffer(out.reshape(-1))
 
 
