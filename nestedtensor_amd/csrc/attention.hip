@@ -432,6 +432,17 @@ __global__ __launch_bounds__(256, (HD > 64 ? 2 : NT_ATTN_WAVES_PER_EU)) void var
   float l_run = 0.0f;   // this lane's share of the row's denominator
 
   const int ntiles = (L + kKTile - 1) / kKTile;
+  // A workgroup's life is its number of key tiles, and three workgroups share a
+  // SIMD: the launch ends when the longest sequences do.  Their wavefronts get the
+  // higher issue priority, so they run near the speed of a SIMD of their own while
+  // the short ones fill what is left.
+  if (ntiles >= 7) {
+    __builtin_amdgcn_s_setprio(3);
+  } else if (ntiles >= 5) {
+    __builtin_amdgcn_s_setprio(2);
+  } else if (ntiles >= 3) {
+    __builtin_amdgcn_s_setprio(1);
+  }
   const T* kbase = K + begin * ldk + h * HD;
   const T* vbase = Vt + (int64_t)h * HD * ldvt + begin;
 
@@ -545,19 +556,15 @@ __global__ __launch_bounds__(256, (HD > 64 ? 2 : NT_ATTN_WAVES_PER_EU)) void var
 #pragma unroll
     for (int e = 0; e < 16; ++e) m_tile = fmaxf(m_tile, sa[1][e]);
     m_tile = max_across_halves(m_tile);
-    if (partial) {
-      // last tile, fewer than 64 keys: the K rows past L are copies of row L - 1
-      // (they cannot have raised the maximum); their probabilities become zero
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          // key of LDS row 32 kb + 8 (e/4) + 4 g + e%4: bits 2 and 3 exchanged
-          const int key = 32 * kb + 16 * (e >> 3) + 8 * g + 4 * ((e >> 2) & 1) + (e & 3);
-          if (key >= n_last) sa[kb][e] = -INFINITY;
-        }
-    }
-    if (first || __any(m_tile > kLazyMaxLog2)) {   // wavefront-uniform
+    // (last tile, fewer than 64 keys: the K rows past L are copies of row L - 1, so
+    // they cannot have raised the maximum, and their V^T columns are zero, so they add
+    // nothing to the output; what they add to the denominator is taken out below)
+    //
+    // The reference maximum starts at 0 and moves only when a tile's maximum leaves
+    // [-2^3, 2^3] powers of two around it (first tile: either way, later only
+    // upwards): for scores of ordinary size it never moves, and no tile pays the
+    // 48 subtractions of a move.
+    if (__any(first ? fabsf(m_tile) > kLazyMaxLog2 : m_tile > kLazyMaxLog2)) {   // wavefront-uniform
       // raise (first tile: set) the reference maximum of every row by delta
       const float delta = first ? m_tile : fmaxf(m_tile, 0.0f);
 #pragma unroll
@@ -613,6 +620,22 @@ __global__ __launch_bounds__(256, (HD > 64 ? 2 : NT_ATTN_WAVES_PER_EU)) void var
           NT_FENCE();
         }
       }
+    }
+    if (partial) {
+      // The keys past L: their K rows are copies of row L - 1, so each of them has
+      // exactly the probability of the last valid key, and the highest key this lane
+      // half holds (8 g + 55, the last accumulator) is one of them whenever the half
+      // holds any.  The lane half holds keys [8 g + 16 j, 8 g + 16 j + 8), j = 0..3.
+      int extra = 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        int over = 8 * g + 16 * j + 8 - n_last;
+        over = over < 0 ? 0 : (over > 8 ? 8 : over);
+        extra += over;
+      }
+      typename AT::Half last4;
+      __builtin_memcpy(&last4, &pw[3][2], 8);
+      l_run -= (float)extra * (float)last4[3];
     }
   };
   // Tile t + 1 travels global -> registers while tile t is computed, and goes

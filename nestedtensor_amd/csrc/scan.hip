@@ -165,17 +165,17 @@ constexpr int kMaxDevices = 64;
 static std::atomic<int64_t*> g_scratch_ptr[kMaxDevices];
 
 // Device address of `scratch` on the current device, or nullptr with the error
-// text set.  The first call on a device asks the runtime; later calls read the
+// text set and its code in *rc.  The first call on a device asks the runtime; later calls read the
 // cached pointer (threads that race on the first call store the same value).
-static int64_t* scratch_on_current_device() {
+static int64_t* scratch_on_current_device(int* rc) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) {
-    fail(NT_ERR_HIP, "offsets_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+    *rc = fail(NT_ERR_HIP, "offsets_noalloc: hipGetDevice: %s", hipGetErrorString(e));
     return nullptr;
   }
   if (dev < 0 || dev >= kMaxDevices) {
-    fail(NT_ERR_UNSUPPORTED, "offsets_noalloc: device index %d is not in [0, %d)", dev, kMaxDevices);
+    *rc = fail(NT_ERR_UNSUPPORTED, "offsets_noalloc: device index %d is not in [0, %d)", dev, kMaxDevices);
     return nullptr;
   }
   int64_t* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
@@ -183,7 +183,7 @@ static int64_t* scratch_on_current_device() {
   void* addr = nullptr;
   e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
   if (e != hipSuccess || addr == nullptr) {
-    fail(NT_ERR_HIP, "offsets_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    *rc = fail(NT_ERR_HIP, "offsets_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
     return nullptr;
   }
   p = static_cast<int64_t*>(addr);
@@ -226,8 +226,9 @@ extern "C" int nt_offsets_from_sizes_noalloc(const int64_t* sizes, int64_t B, in
   }
   // Nothing in the scratch has to start at zero: the first launch writes the
   // sum of every tile before the second one reads it.
-  int64_t* ws = scratch_on_current_device();
-  if (ws == nullptr) return NT_ERR_HIP;
+  int rc = NT_OK;
+  int64_t* ws = scratch_on_current_device(&rc);
+  if (ws == nullptr) return rc;
   SizesProd load{sizes, D};
   return run_scan(load, B, offsets, ws, (size_t)kNoAllocMaxTiles * sizeof(int64_t),
                   (hipStream_t)stream);

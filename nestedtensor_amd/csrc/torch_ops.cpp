@@ -23,6 +23,7 @@
 #include <torch/library.h>
 
 #include <algorithm>
+#include <chrono>
 #include <cstring>
 #include <tuple>
 #include <vector>
@@ -43,6 +44,14 @@ inline void check(int rc) {
 inline void require_device(const Tensor& t, const char* what) {
   TORCH_CHECK(t.is_cuda(), "nestedtensor_amd: ", what, " runs on the HIP device only; got a tensor on ",
               t.device(), ". Move the nested tensor with .to('cuda') first.");
+}
+
+// Every pointer a kernel dereferences must be device memory of the input's
+// device: a weight or bias left on the host would be read by the GPU as a stray
+// address (a memory-access fault, not an exception).
+inline void require_same_device(const Tensor& t, const Tensor& like, const char* what, const char* name) {
+  TORCH_CHECK(!t.defined() || t.device() == like.device(), what, ": ", name, " is on ", t.device(),
+              " but the input is on ", like.device(), ". Move the module with .to('cuda') first.");
 }
 
 inline void* stream_of(const Tensor& t) {
@@ -355,12 +364,21 @@ void wait_for_stream(hipStream_t stream) {
     if (!flag_t.defined()) {
       flag_t = at::zeros({16}, at::TensorOptions().dtype(at::kInt).pinned_memory(true));
     }
-    volatile uint32_t* flag = reinterpret_cast<volatile uint32_t*>(flag_t.data_ptr());
+    uint32_t* flag = reinterpret_cast<uint32_t*>(flag_t.data_ptr());
     const uint32_t want = ++seq;
-    if (hipStreamWriteValue32(stream, const_cast<uint32_t*>(flag), want, 0) == hipSuccess) {
-      for (int spin = 0; spin < (1 << 22); ++spin) {
-        if (*flag == want) return;
+    if (hipStreamWriteValue32(stream, flag, want, 0) == hipSuccess) {
+      // Poll for at most 200 microseconds (an acquire load: the counts the kernel wrote
+      // to pinned memory are read after it), then hand the wait to the runtime.  The
+      // write-value operation follows the kernel in stream order; that the kernel's
+      // own stores to host memory are visible by then is what the blocking
+      // synchronise below guarantees in any case, and it runs whenever the flag
+      // has not shown up in time.
+      const auto t0 = std::chrono::steady_clock::now();
+      for (int spin = 0;; ++spin) {
+        if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) == want) return;
         __builtin_ia32_pause();
+        if ((spin & 255) == 255 &&
+            std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(200)) break;
       }
     } else {
       (void)hipGetLastError();
@@ -456,6 +474,10 @@ bool leading_box(const int32_t* c, const int64_t* dims, int64_t nd, int64_t* ext
 // mask, which only the non-prefix path needs.
 template <class CountRows, class ByteMask>
 Lowered from_rows(const Tensor& tensor, int64_t mask_dims, CountRows count_rows, ByteMask byte_mask) {
+  // a mask row lives below the batch dim: the level tables below index [mask_dims - 2]
+  TORCH_CHECK(mask_dims >= 2 && mask_dims <= tensor.dim(),
+              "nested_tensor_from_tensor_mask: the mask needs a batch dim and at least one more (got ", mask_dims,
+              " mask dims for a tensor of ", tensor.dim(), " dims)");
   const int64_t B = tensor.size(0);
   const at::IntArrayRef shape = tensor.sizes();
   const int64_t M = shape[mask_dims - 1];
@@ -717,6 +739,21 @@ std::tuple<Tensor, Tensor> merge_tensor_mask(const Tensor& tensor, const Tensor&
 
 // ---- packed projections and nested multi-head attention -------------------------
 
+// Weights and biases of an attention layer against the input x [T, E]: on x's
+// device (a module left on the host would hand the kernels host pointers), biases
+// of the length the kernels read (3 E for the in-projection, N for the output).
+void check_mha_weights(const Tensor& x, int64_t E, const Tensor& W, const Tensor& b_in, const Tensor& Wo,
+                       const Tensor& b_out) {
+  require_same_device(W, x, "mha", "in_proj_weight");
+  require_same_device(b_in, x, "mha", "in_proj_bias");
+  require_same_device(Wo, x, "mha", "out_proj_weight");
+  require_same_device(b_out, x, "mha", "out_proj_bias");
+  TORCH_CHECK(!b_in.defined() || b_in.numel() == 3 * E, "in_proj_bias must have 3 * embed_dim = ", 3 * E,
+              " elements, got ", b_in.defined() ? b_in.numel() : 0);
+  TORCH_CHECK(!b_out.defined() || b_out.numel() == Wo.size(0), "out_proj_bias must have ", Wo.size(0),
+              " elements, got ", b_out.defined() ? b_out.numel() : 0);
+}
+
 // y = act(x @ weight.T + bias) on a 2-D row-major view (nt_linear_act): the packed
 // fast path of NestedTensor_matmul (matmul.cpp:13-41) with the packed bias add
 // (BinaryOps.cpp:97-107) and, optionally, relu / gelu (activation.cpp:11-19, 34-46)
@@ -733,6 +770,10 @@ Tensor linear_packed(const Tensor& x, const Tensor& weight_in, const c10::option
   if (bias_in.has_value() && bias_in->defined()) bias = bias_in->contiguous();
   TORCH_CHECK(weight.scalar_type() == x.scalar_type() && (!bias.defined() || bias.scalar_type() == x.scalar_type()),
               "linear: input, weight and bias must have the same dtype");
+  require_same_device(weight, x, "linear", "weight");
+  require_same_device(bias, x, "linear", "bias");
+  TORCH_CHECK(!bias.defined() || bias.numel() == N, "linear: bias of ", bias.defined() ? bias.numel() : 0,
+              " elements does not match the ", N, " output features");
   c10::hip::HIPGuard guard(x.device().index());
   Tensor out = at::empty({M, N}, x.options());
   check(nt_linear_act(x.const_data_ptr(), x.stride(0), weight.const_data_ptr(),
@@ -766,6 +807,7 @@ Tensor mha_self_packed(const Tensor& x, const Tensor& schedule, int64_t num_head
               "linear: input, weight and bias must have the same dtype");
   TORCH_CHECK(Wo.dim() == 2 && Wo.size(1) == E, "linear: weight of shape ", Wo.sizes(),
               " does not match input feature size ", E);
+  check_mha_weights(x, E, W, b_in, Wo, b_out);
   TORCH_CHECK(schedule.scalar_type() == at::kInt && schedule.dim() == 2 && schedule.size(1) == 8 &&
                   schedule.is_contiguous() && schedule.device() == x.device(),
               "mha: schedule must be a contiguous int32 [n_work, 8] tensor on the input's device");
@@ -809,6 +851,10 @@ Tensor layer_norm_packed(const Tensor& x, const c10::optional<Tensor>& residual,
   }
   TORCH_CHECK(!residual.has_value() || !residual->defined() || residual->numel() == x.numel(),
               "layer_norm: the residual must have the size of the input");
+  for (const auto* t : {&weight, &bias}) {
+    TORCH_CHECK(!t->has_value() || !(*t)->defined() || (*t)->numel() == n,
+                "layer_norm: weight and bias must have ", n, " elements");
+  }
   c10::hip::HIPGuard guard(x.device().index());
   Tensor out = at::empty_like(x);
   check(nt_layer_norm(x.const_data_ptr(), opt_ptr(residual), opt_ptr(weight), opt_ptr(bias), out.data_ptr(),
@@ -1024,6 +1070,7 @@ void check_mha_operands(const Tensor& xq, const Tensor& xk, const Tensor& xv, in
               "linear: input, weight and bias must have the same dtype");
   TORCH_CHECK(Wo.dim() == 2 && Wo.size(1) == E, "linear: weight of shape ", Wo.sizes(),
               " does not match input feature size ", E);
+  check_mha_weights(xq, E, W, b_in, Wo, b_out);
 }
 
 // Attention between different nested tensors (or with an embedding size the fused

@@ -698,15 +698,18 @@ def conv2d(impl, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
 # the kernels write zero rows for such indices and count them in a counter that
 # lives on the device for the life of the process (it only ever grows).  How the
 # count reaches the host is a setting:
-#   "deferred"  (default) after each call the counter is copied, asynchronously,
-#               into pinned host memory; the next embedding / embedding_bag call
-#               and check_index_errors() look at that copy and raise IndexError
-#               for whatever has arrived.  No call waits for the device, and the
-#               ops can be captured in a HIP graph.
-#   "immediate" every call waits for its own count and raises before returning.
+#   "immediate" (default) every call waits for its own count and raises before
+#               returning, like an index error of the reference's host path.  Under
+#               stream capture nothing can be waited for; a captured call behaves
+#               as in "deferred".
+#   "deferred"  after each call the counter is copied, asynchronously, into pinned
+#               host memory; the next embedding / embedding_bag call and
+#               check_index_errors() look at that copy and raise IndexError for
+#               whatever has arrived.  No call waits for the device: the setting
+#               for serving loops that validate their indices elsewhere.
 #   "off"       indices are trusted; nothing is copied.
 _INDEX_CHECK_MODES = ("deferred", "immediate", "off")
-_index_check_mode = "deferred"
+_index_check_mode = "immediate"
 _index_counters = {}      # device index -> [device int32[1], pinned int32[1], count already reported]
 
 
@@ -758,13 +761,14 @@ def _oob_begin(device, what):
     if _index_check_mode == "off":
         return None
     slot = _index_counter(device)
-    if _index_check_mode == "deferred" and not torch.cuda.is_current_stream_capturing():
+    if not torch.cuda.is_current_stream_capturing():
+        # what earlier deferred (or captured) calls have left
         _report_index_errors(slot, what + " (an earlier call)")
     return slot
 
 
 def _oob_end(slot, what):
-    if _index_check_mode == "immediate":
+    if _index_check_mode == "immediate" and not torch.cuda.is_current_stream_capturing():
         torch.cuda.current_stream(slot[0].device).synchronize()
         _report_index_errors(slot, what)
 

@@ -57,11 +57,28 @@ def test_out_of_range_indices_immediate(op):
 
 @pytest.mark.parametrize("op", ["embedding", "embedding_bag"])
 def test_out_of_range_indices_deferred(op):
-    # the default: the call itself returns (zero rows for the bad indices, no wait
-    # for the device); the count is raised by check_index_errors() or by the next call
+    # opt-in: the call itself returns (zero rows for the bad indices, no wait for the
+    # device); the count is raised by check_index_errors() or by the next call
     fn = getattr(torch.nn.functional, op)
     bad, good, w = _bad_and_good()
-    assert nt.set_index_check("deferred") == "deferred"
+    previous = nt.set_index_check("deferred")
+    try:
+        _deferred_reports(op, fn, bad, good, w)
+    finally:
+        nt.set_index_check(previous)
+
+
+def test_out_of_range_indices_raise_by_default():
+    # without any setting a bad index raises from the call that met it, as the
+    # reference's host embedding does
+    bad, good, w = _bad_and_good()
+    with pytest.raises(IndexError, match="2 index value"):
+        torch.nn.functional.embedding(bad, w)
+    torch.nn.functional.embedding(good, w)
+    nt.check_index_errors()
+
+
+def _deferred_reports(op, fn, bad, good, w):
     nt.check_index_errors()
     out = fn(bad, w)
     dense = out.to_padded_tensor(0) if op == "embedding" else out
@@ -126,7 +143,8 @@ def test_embedding_ops_under_hip_graph_replays(op):
         exp = buf(fn(a, w, **kw))
         torch.cuda.synchronize()
         assert torch.equal(got, exp), "replay %d differs from the eager call" % rep
-    # an out-of-range index met during a replay is reported like any other
+    # an out-of-range index met during a replay (nothing waits inside a graph) is
+    # reported by the next check
     a._impl.buffer[3] = V + 7
     graph.replay()
     with pytest.raises(IndexError, match="1 index value"):

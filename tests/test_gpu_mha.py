@@ -17,6 +17,7 @@ pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda", 0)
 
 FP32_REL = 1e-5
+FP32_ELEM_ABS = 1e-5
 HALF_ABS = 2e-2
 
 
@@ -39,6 +40,11 @@ def check(got_nt, exp_parts, dtype, exp64=None):
     if dtype == torch.float32:
         scale = max(exp.abs().max().item(), 1e-30)
         assert err / scale <= FP32_REL, (err, scale)
+        # and element by element, the way the reference's own tests compare
+        # (assertEqual at 1e-5, test/utils_test_case.py:21,102-118) together with the
+        # 1e-5 relative bound of the target: |a - b| <= 1e-5 + 1e-5 |b|
+        excess = ((got - exp).abs() - (FP32_ELEM_ABS + FP32_REL * exp.abs())).max().item()
+        assert excess <= 0.0, "worst element exceeds 1e-5 + 1e-5 |b| by %g" % excess
     else:
         assert err <= HALF_ABS, err
     if exp64 is not None:
@@ -249,6 +255,40 @@ def test_mha_input_errors():
     irregular = nt.nested_tensor([torch.randn(3, 4), torch.randn(2, 5)], device=DEV)
     with pytest.raises(RuntimeError, match="query's third dimension must be regular."):
         torch.ops.nestedtensor.min_mha(2, 2, 0.0, False, irregular, a, a, W, bi, 1.0, Wo, bo)
+
+
+def test_weights_on_the_host_raise_before_any_launch():
+    # a module left on the host must raise, not hand the kernels a host pointer
+    H, hd = 2, 64
+    E = H * hd
+    for dtype in (torch.float16, torch.float32):
+        xs, W_in, b_in, W_out, b_out = make_case(E, [5, 9], 3, dtype)
+        a = nt.nested_tensor(xs, device=DEV, dtype=dtype)
+        dev = [t.to(DEV) for t in (W_in, b_in, W_out, b_out)]
+        host = [W_in, b_in, W_out, b_out]
+        for i in range(4):
+            w = list(dev)
+            w[i] = host[i]
+            with pytest.raises(RuntimeError, match="is on cpu"):
+                torch.ops.nestedtensor.min_mha(H, hd, 0.0, False, a, a, a, w[0], w[1], hd ** -0.5, w[2], w[3])
+        # cross-attention takes the operator with three projections
+        k = nt.nested_tensor([torch.randn(7, E).to(dtype), torch.randn(3, E).to(dtype)], device=DEV, dtype=dtype)
+        with pytest.raises(RuntimeError, match="is on cpu"):
+            torch.ops.nestedtensor.min_mha(H, hd, 0.0, False, a, k, k, dev[0], dev[1], hd ** -0.5, W_out, dev[3])
+        # biases of the wrong length are refused too
+        with pytest.raises(RuntimeError, match="in_proj_bias must have"):
+            torch.ops.nestedtensor.min_mha(H, hd, 0.0, False, a, a, a, dev[0], dev[1][:E], hd ** -0.5, dev[2], dev[3])
+        with pytest.raises(RuntimeError, match="out_proj_bias must have"):
+            torch.ops.nestedtensor.min_mha(H, hd, 0.0, False, a, a, a, dev[0], dev[1], hd ** -0.5, dev[2], dev[3][:5])
+    a = nt.nested_tensor([torch.randn(4, 8), torch.randn(2, 8)], device=DEV)
+    with pytest.raises(RuntimeError, match="is on cpu"):
+        torch.nn.functional.linear(a, torch.randn(16, 8))
+    with pytest.raises(RuntimeError, match="is on cpu"):
+        torch.nn.functional.linear(a, torch.randn(16, 8, device=DEV), torch.randn(16))
+    with pytest.raises(RuntimeError, match="bias of 3 elements"):
+        torch.nn.functional.linear(a, torch.randn(16, 8, device=DEV), torch.randn(3, device=DEV))
+    with pytest.raises(RuntimeError, match="weight and bias must have 8 elements"):
+        torch.ops.nestedtensor.layer_norm_packed(a._impl.buffer, None, torch.ones(4, device=DEV), None, 8, 1e-5)
 
 
 def _c3():

@@ -534,6 +534,16 @@ def test_from_padded_value_comparison_semantics():
     bits_equal(got._impl.buffer, exp.buffer)
 
 
+def test_dense_to_nested_operators_refuse_a_tensor_without_rows():
+    # the registered operators can be called directly; a 1-D tensor has no mask rows
+    # below the batch dim
+    t = torch.arange(6.0, device=DEV)
+    with pytest.raises(RuntimeError, match="batch dim and at least one more"):
+        torch.ops.nestedtensor.nt_from_padded_tensor(t, -1.0, 1)
+    with pytest.raises(RuntimeError, match="batch dim and at least one more"):
+        torch.ops.nestedtensor.from_padded_value_lowered(t, -1.0, 1)
+
+
 def test_from_padded_value_non_prefix_takes_compaction_path():
     t = torch.tensor([[[1.0, -1.0, 2.0, -1.0], [3.0, -1.0, 4.0, -1.0]],
                       [[5.0, 6.0, -1.0, -1.0], [7.0, 8.0, -1.0, -1.0]]])
