@@ -11,16 +11,20 @@ in HBM before the timed region.  `value` is the algorithmic bytes of the whole
 step (pad: valid read + padded written; un-pad: valid read + valid written)
 divided by the step time.
 
-The same JSON line carries
+The LAST line of the output is the headline JSON record.  It carries
   roofline     - the dominant kernel (row_kernel<2, pad>): algorithmic bytes per
-                 launch / mean launch time from HIP events, against 8 TB/s;
+                 launch / mean launch time from HIP events, against 8 TB/s; and in
+                 roofline.mha the second half of the metric: the C3 attention
+                 layer's tokens/s and fraction of the dense fp16 MFMA peak;
   cpu_baseline - the CPU oracle (the reference's CPU algorithm restated) timed on
-                 a bounded sample of the same workload on the host cores;
-  mha          - nested BERT-base self-attention (configuration C3) tokens/s and
-                 its MFMA roofline fraction;
-  rows         - the remaining rows of the path (to_tensor_mask, to_mask,
-                 nested_tensor_from_tensor_mask / _from_padded_tensor, pack, the
-                 offsets scan, C4 attention) on configurations C1, C2 and C4.
+                 a bounded sample of the same workload on the host cores (and in
+                 cpu_baseline.mha the oracle's attention layer on the C3 batch);
+  mha          - the C3 leg in full: per-kernel times, the same layer from a HIP
+                 graph, the whole encoder layer, and the reference benchmark's own
+                 comparison, torch's dense nn.MultiheadAttention on the padded batch.
+A line before it, {"rows": ...}, holds the remaining rows of the path
+(to_tensor_mask, to_mask, nested_tensor_from_tensor_mask / _from_padded_tensor,
+pack, the offsets scan, C4 attention, ...) on configurations C1, C2 and C4.
 
 Every row is the median over timed batches of calls, with the slowest batch
 and the mean beside it.  All device legs run first; what the CPU oracle times
@@ -33,6 +37,7 @@ and print only the sizes the counters are to be set against:
 
 import argparse
 import contextlib
+import ctypes
 import gc
 import json
 import os
@@ -423,6 +428,43 @@ def bench_mha_c3(args, torch, dev, later):
         graph_ms = "graph capture failed: %r" % (exc,)
     T = sum(lens)
     flops = 8 * T * E * E + 4 * E * sum(L * L for L in lens)
+    # the three launches one by one through the C ABI (each timed as batches of
+    # five with an event between batches, like the layer): what each costs when the
+    # device has nothing else queued
+    kernel_us = _mha_kernel_times(torch, dev, a, dW_in, db_in, dW_out, db_out, H, hd)
+    # The reference's own benchmark method (benchmarks/mha_cuda.py:26-83): the same
+    # batch, padded to the longest sequence, through torch's dense
+    # nn.MultiheadAttention with a key-padding mask on the same GPU.  Context, not a
+    # target: the dense layer computes the padded tokens too.
+    dense = None
+    try:
+        mha = torch.nn.MultiheadAttention(E, H, bias=True, batch_first=True, device=dev, dtype=torch.float16)
+        with torch.no_grad():
+            mha.in_proj_weight.copy_(dW_in)
+            mha.in_proj_bias.copy_(db_in)
+            mha.out_proj.weight.copy_(dW_out)
+            mha.out_proj.bias.copy_(db_out)
+        mha.eval()
+        Lmax = max(lens)
+        x_pad = a.to_padded_tensor(0)
+        kpm = torch.arange(Lmax, device=dev)[None, :] >= torch.tensor(lens, device=dev)[:, None]
+
+        def dense_layer():
+            with torch.no_grad():
+                return mha(x_pad, x_pad, x_pad, key_padding_mask=kpm, need_weights=False)[0]
+
+        y_dense = dense_layer()
+        ms_dense = _time_gpu(torch, dense_layer, iters=30, warmup=3)
+        got_pad = out.to_padded_tensor(0)
+        valid = ~kpm
+        dense = dict(what="torch.nn.MultiheadAttention (dense, batch_first, key_padding_mask) on the batch padded to "
+                          "[%d, %d, %d], same GPU, fp16" % (len(lens), Lmax, E),
+                     ms=float(ms_dense), ms_max=ms_dense.max, speedup=float(ms_dense) / float(ms),
+                     padded_tokens=len(lens) * Lmax, valid_tokens=T,
+                     max_abs_diff_on_valid_tokens=float((y_dense[valid].float() - got_pad[valid].float()).abs().max()))
+        del mha, x_pad, y_dense, got_pad
+    except Exception as exc:      # report, do not hide
+        dense = "dense comparison failed: %r" % (exc,)
     # the whole encoder layer on the packed layout: attention, residual + layer norm,
     # feed-forward 768 -> 3072 (gelu in the GEMM epilogue) -> 768, residual + layer norm
     from nestedtensor_amd import ops as _ops
@@ -458,7 +500,7 @@ def bench_mha_c3(args, torch, dev, later):
     res = dict(workload="C3: nested BERT-base self-attention, fp16, B=32, L~U[32,512], d=768, 12x64",
                tokens=T, ms_per_layer=float(ms), ms_per_layer_max=ms.max, ms_per_layer_mean=ms.mean,
                timing=ms.fields()["timing"], ms_per_layer_hip_graph=graph_ms,
-               tokens_per_s=T / (ms * 1e-3), flops=flops,
+               tokens_per_s=T / (ms * 1e-3), flops=flops, kernel_us=kernel_us, dense_padded_torch=dense,
                roofline=dict(bound="mfma", achieved=flops / (ms * 1e-3) / 1e12, peak=MFMA_F16_PEAK_TFLOPS,
                              unit="TFLOP/s", frac=flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS))
     if ms_enc is not None:
@@ -485,6 +527,44 @@ def bench_mha_c3(args, torch, dev, later):
             res["cpu_baseline"] = dict(value=T / best, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
                                        sample="full C3 layer, oracle min_mha in fp16 on the host, best of 2")
         later.append(_cpu_layer)
+    return res
+
+
+def _mha_kernel_times(torch, dev, a, W_in, b_in, W_out, b_out, H, hd):
+    """Microseconds of each of the three launches of the fused self-attention
+    layer (nt_linear_qkv, nt_varlen_attention_vt, nt_linear_act), issued through
+    the C ABI on torch's current stream with the operator's own buffers' shapes."""
+    from nestedtensor_amd import _C
+    impl = a._impl
+    E = H * hd
+    x = impl.buffer.reshape(-1, E)
+    T = x.size(0)
+    ldvt = (T + 72 + 7) // 8 * 8
+    qk = torch.empty(T, 2 * E, device=dev, dtype=x.dtype)
+    vt = torch.zeros(E, ldvt, device=dev, dtype=x.dtype)
+    attn = torch.empty(T, E, device=dev, dtype=x.dtype)
+    out = torch.empty(T, E, device=dev, dtype=x.dtype)
+    sched = impl.attention_schedule()
+    stream = _C.current_stream(dev)
+    dt = _C.dtype_code(x.dtype)
+
+    def qkv():
+        _C.check(_C.lib.nt_linear_qkv(_C.ptr(x), E, _C.ptr(W_in), _C.ptr(b_in), _C.ptr(qk), 2 * E, _C.ptr(vt), ldvt,
+                                      T, E, E, dt, stream))
+
+    def attention():
+        _C.check(_C.lib.nt_varlen_attention_vt(_C.ptr(qk), 2 * E, ctypes.c_void_p(qk.data_ptr() + 2 * E), 2 * E,
+                                               _C.ptr(vt), ldvt, _C.ptr(attn), E, _C.ptr(sched), sched.size(0), H, hd,
+                                               T, hd ** -0.5, dt, stream))
+
+    def out_proj():
+        _C.check(_C.lib.nt_linear_act(_C.ptr(attn), E, _C.ptr(W_out), _C.ptr(b_out), _C.ptr(out), E, T, E, E, 0, dt,
+                                      stream))
+
+    res = {}
+    for name, fn in (("qkv_projection", qkv), ("attention", attention), ("out_projection", out_proj)):
+        res[name] = float(_time_gpu(torch, fn, iters=50, warmup=5)) * 1e3
+    res["sum"] = sum(res.values())
     return res
 
 
@@ -927,6 +1007,23 @@ def main():
         for job in later:
             job()
         line["cpu_baseline"] = cpu_baseline_c5(torch)
+    # The metric has two halves; `value` is the first (C5 pad + un-pad GB/s).  The
+    # second, the C3 attention layer, rides inside `roofline` and `cpu_baseline`
+    # as well, next to the figures of the first half.
+    mha = line.get("mha")
+    if isinstance(mha, dict):
+        r = mha["roofline"]
+        line["roofline"]["mha"] = dict(bound="mfma", achieved=r["achieved"], peak=r["peak"], unit=r["unit"],
+                                       frac=r["frac"], ms_per_layer=mha["ms_per_layer"],
+                                       tokens_per_s=mha["tokens_per_s"], kernel_us=mha["kernel_us"],
+                                       workload=mha["workload"])
+        if "cpu_baseline" in mha and "cpu_baseline" in line:
+            line["cpu_baseline"]["mha"] = mha["cpu_baseline"]
+    # the per-operator rows go out first, on a line of their own; the last line of
+    # the output is the headline record
+    rows = line.pop("rows", None)
+    if rows is not None:
+        print(json.dumps({"rows": rows}))
     print(json.dumps(line))
 
 
