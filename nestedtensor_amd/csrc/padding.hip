@@ -168,6 +168,23 @@ __device__ __forceinline__ void move_row(char* d, const char* s, int64_t valid, 
   }
 }
 
+// Every argument the row decode may touch, fetched in ONE batch of scalar loads at
+// the top of a kernel.  Left to the compiler they are fetched piecemeal
+// behind the decode's branches, each a round trip of its own, and a workgroup here
+// lives for one 4 KiB tile (C5 pad: 2.4 % of the launch).  The statement depends on
+// all of them and yields a zero the compiler cannot see through, which the caller
+// adds to its row index so that the statement is kept.  It is neither volatile nor
+// a memory clobber: behind a volatile statement the loads through offsets / sizes
+// stop being scalar loads.
+__device__ __forceinline__ int args_in_one_batch(const RowParams& p) {
+  int zero;
+  asm("s_mov_b32 %0, 0"
+      : "=s"(zero)
+      : "s"(p.src), "s"(p.dst), "s"(p.offsets), "s"(p.sizes), "s"(p.D), "s"(p.nrag), "s"(p.M0), "s"(p.M1),
+        "s"(p.M2), "s"(p.inner), "s"(p.nrows));
+  return __builtin_amdgcn_readfirstlane(zero);
+}
+
 // One row of work, decoded: bytes [0, valid) of d come from s, bytes [valid, total)
 // are padding (kOnes: ones / zeros, s unused).
 struct RowDesc {
@@ -178,7 +195,12 @@ struct RowDesc {
 
 // Decode row `row` (scalar arithmetic, uniform over the lanes that share the row).
 // Returns false when the row has nothing to move.
-template <int EB, int MODE>
+// ONE_RAGGED: the launch has one ragged dim (a row is a whole constituent): a kernel
+// of its own without the divisions of the other two cases, so that the decode is
+// a few straight-line instructions from the kernel's entry.  A workgroup lives for
+// one 4 KiB tile; with the general decode the one-ragged-dim path sat behind a far
+// branch and cost the C5 pad launch 2.4 %.
+template <int EB, int MODE, bool ONE_RAGGED>
 __device__ __forceinline__ bool decode_row(const RowParams& p, int64_t row, RowDesc& r) {
   if (MODE == kPack) {
     const int64_t off = p.offsets[row];
@@ -190,7 +212,7 @@ __device__ __forceinline__ bool decode_row(const RowParams& p, int64_t row, RowD
   }
   int64_t b, src_off = 0, last;
   bool inside = true;
-  if (p.nrag == 1) {
+  if (ONE_RAGGED || p.nrag == 1) {
     b = row;
     last = p.sizes[b * p.D];
   } else if (p.nrag == 2) {
@@ -211,7 +233,7 @@ __device__ __forceinline__ bool decode_row(const RowParams& p, int64_t row, RowD
     last = sz[2];
     src_off = (i0 * sz[1] + i1) * last;
   }
-  const int64_t Mlast = p.nrag == 1 ? p.M0 : (p.nrag == 2 ? p.M1 : p.M2);
+  const int64_t Mlast = (ONE_RAGGED || p.nrag == 1) ? p.M0 : (p.nrag == 2 ? p.M1 : p.M2);
   const int64_t row_bytes = Mlast * p.inner * EB;
   const int64_t valid = inside ? last * p.inner * EB : 0;
   if (MODE == kOnes) {
@@ -237,13 +259,14 @@ __device__ __forceinline__ bool decode_row(const RowParams& p, int64_t row, RowD
 
 // WAVE_ROWS: rows of at most 1 KiB -- every wavefront of the workgroup takes a row
 // of its own (4 rows per workgroup) instead of 192 lanes idling on one row.
-template <int EB, int MODE, bool WAVE_ROWS>
+template <int EB, int MODE, bool WAVE_ROWS, bool ONE_RAGGED>
 __global__ __launch_bounds__(256) void row_kernel(RowParams p) {
   constexpr int kT = WAVE_ROWS ? 64 : 256;
-  const int64_t row = WAVE_ROWS ? row_index() * 4 + (threadIdx.x >> 6) : row_index();
+  const int after_args = args_in_one_batch(p);
+  const int64_t row = (WAVE_ROWS ? row_index() * 4 + (threadIdx.x >> 6) : row_index()) + after_args;
   if (row >= p.nrows) return;
   RowDesc r;
-  if (!decode_row<EB, MODE>(p, row, r)) return;
+  if (!decode_row<EB, MODE, ONE_RAGGED>(p, row, r)) return;
   constexpr int kMove = MODE == kPack ? kUnpad : (MODE == kPadMask ? kPad : MODE);
   move_row<EB, kMove, kT>(r.d, r.s, r.valid, r.total, p.pad);
   if (MODE == kPadMask) {
@@ -354,9 +377,10 @@ __device__ __forceinline__ void move_rows(const RowDesc (&r)[NR], const bool (&o
 template <int EB, int MODE, int kT, int NR>
 __global__ __launch_bounds__(256) void row_batch_kernel(RowParams p) {
   constexpr int kGroups = 256 / kT;
+  const int after_args = args_in_one_batch(p);
   const int tid = threadIdx.x & (kT - 1);
   const int64_t group = ((int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x) * kGroups + (threadIdx.x / kT);
-  const int64_t row0 = group * NR;
+  const int64_t row0 = group * NR + after_args;
   if (row0 >= p.nrows) return;
   // Row decode in three steps so that the size-table and offset loads of all NR
   // rows are in flight together (one memory round trip, not NR): coordinates of
@@ -452,9 +476,10 @@ __global__ __launch_bounds__(256) void row_batch_kernel(RowParams p) {
 template <int EB, int MODE, int kT>
 __global__ __launch_bounds__(256) void row_group_kernel(RowParams p, int rows_per_group) {
   constexpr int kGroups = 256 / kT;
+  const int after_args = args_in_one_batch(p);
   const int tid = threadIdx.x & (kT - 1);
   const int64_t group = ((int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x) * kGroups + (threadIdx.x / kT);
-  const int64_t row0 = group * rows_per_group;
+  const int64_t row0 = group * rows_per_group + after_args;
   if (row0 >= p.nrows) return;
   const int64_t count = p.nrows - row0 < rows_per_group ? p.nrows - row0 : rows_per_group;
   // coordinates of the first row: (b, i0) for two ragged dims, (b, i0, i1) for three
@@ -653,13 +678,21 @@ static int launch_rows_t(int eb, const RowParams& p, int64_t max_row_bytes, hipS
   dim3 grid((unsigned)grid_rows, (unsigned)gy, 1);
 #endif
   dim3 block(256, 1, 1);
+#define NT_ROW_CASE(EB)                                                                               \
+  if (p.nrag == 1 || MODE == kPack) {                                                                 \
+    hipLaunchKernelGGL((row_kernel<EB, MODE, WAVE_ROWS, true>), grid, block, 0, stream, p);           \
+  } else {                                                                                            \
+    hipLaunchKernelGGL((row_kernel<EB, MODE, WAVE_ROWS, false>), grid, block, 0, stream, p);          \
+  }                                                                                                   \
+  break;
   switch (eb) {
-    case 1: hipLaunchKernelGGL((row_kernel<1, MODE, WAVE_ROWS>), grid, block, 0, stream, p); break;
-    case 2: hipLaunchKernelGGL((row_kernel<2, MODE, WAVE_ROWS>), grid, block, 0, stream, p); break;
-    case 4: hipLaunchKernelGGL((row_kernel<4, MODE, WAVE_ROWS>), grid, block, 0, stream, p); break;
-    case 8: hipLaunchKernelGGL((row_kernel<8, MODE, WAVE_ROWS>), grid, block, 0, stream, p); break;
+    case 1: NT_ROW_CASE(1)
+    case 2: NT_ROW_CASE(2)
+    case 4: NT_ROW_CASE(4)
+    case 8: NT_ROW_CASE(8)
     default: return fail(NT_ERR_INVALID_ARGUMENT, "elem_bytes must be 1, 2, 4 or 8, got %d", eb);
   }
+#undef NT_ROW_CASE
   return check_launch("row_kernel");
 }
 
