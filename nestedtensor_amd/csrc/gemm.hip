@@ -29,18 +29,6 @@
 //            finds V^T tiles key-contiguous.
 #include "nt_common.h"
 
-// Compile-time tuning knobs.
-// Measurement aid, never set in a product build: bits that take one ingredient
-// out of the K loop of the global -> LDS path so that its cost can be read off a
-// depth sweep (results are then wrong).  1: no MFMA, 2: no global -> LDS loads,
-// 4: fragments read once instead of every step, 8: no barrier.
-#ifndef NT_GEMM_ABLATE
-#define NT_GEMM_ABLATE 0
-#endif
-#ifndef NT_GEMM_FORCE_CFG
-#define NT_GEMM_FORCE_CFG (-1)           // 0, 1, 2: always that tile shape (experiments)
-#endif
-
 namespace nt {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -98,12 +86,19 @@ struct GemmCfg {
   static constexpr int kPerB = kBN * kChunksPerRow / kThreads;   // W pieces per thread
   static constexpr int kPerThread = kPerA + kPerB;
   static constexpr int kBufBytes = (kBM + kBN) * kLdsRow;
-  // direct global -> LDS loads: unpadded rows, as many K tiles resident as fit (at most 4)
-  static constexpr int kDmaTileBytes = (kBM + kBN) * BKB_;
-  static constexpr int kDmaBufs = (160 * 1024 - 2048) / kDmaTileBytes > 4 ? 4 : (160 * 1024 - 2048) / kDmaTileBytes;
+  // direct global -> LDS loads: unpadded rows, the K tiles of A and of W in a ring
+  // each, three tiles deep if that fits and two otherwise.  (A third tile for only
+  // one of the operands, which fits beside two whole tiles of the 256x192 shape, was
+  // measured for either operand: no change, the K loop is not waiting for latency.)
+  static constexpr int kATileBytes = kBM * BKB_;
+  static constexpr int kBTileBytes = kBN * BKB_;
+  static constexpr int kLdsBudget = 160 * 1024 - 2048;
+  static constexpr bool kThreeOfBoth = 3 * (kATileBytes + kBTileBytes) <= kLdsBudget;
+  static constexpr int kBufsB = kThreeOfBoth ? 3 : 2;
+  static constexpr int kBufsA = kThreeOfBoth ? 3 : 2;
+  static constexpr int kRingBytes = kBufsA * kATileBytes + kBufsB * kBTileBytes;
   // tile buffers (kernels for a ragged K use two padded, register-staged buffers)
-  static constexpr int kLdsBytes =
-      kDmaBufs * kDmaTileBytes > 2 * kBufBytes ? kDmaBufs * kDmaTileBytes : 2 * kBufBytes;
+  static constexpr int kLdsBytes = kRingBytes > 2 * kBufBytes ? kRingBytes : 2 * kBufBytes;
   static_assert((kBM * kChunksPerRow) % kThreads == 0 && (kBN * kChunksPerRow) % kThreads == 0,
                 "tile pieces must divide among the threads");
 };
@@ -229,44 +224,62 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
     // between them; in the other direction the rule for this file is that nothing
     // makes the compiler keep a value of its own in M0 across these statements (no
     // LDS-direct builtin, no dynamic register indexing, no sendmsg).
-    static_assert(Cfg::kRowBytes == 128 && Cfg::kBM % 8 == 0, "1 KiB blocks of eight rows");
-    constexpr int kN = Cfg::kPerThread;
+    static_assert(Cfg::kRowBytes == 128 && Cfg::kBM % 64 == 0 && Cfg::kBN % 64 == 0,
+                  "1 KiB blocks of eight rows, a whole number of them per wavefront");
     constexpr int kWaves = Cfg::kThreads / 64;
-    const char* gptr[kN];
+    constexpr int kNA = Cfg::kBM / 8 / kWaves;      // 1 KiB blocks of an A tile per wavefront
+    constexpr int kNW = Cfg::kBN / 8 / kWaves;      // ... of a W tile
+    constexpr int kRA = Cfg::kBufsA, kRW = Cfg::kBufsB;
+    static_assert(kRA >= 2 && kRW >= 2 && kRA - kRW <= 1 && kRW - kRA <= 1, "the wait below counts on the issue order");
+    constexpr bool kWLast = kRW > kRA;              // the deeper ring is issued last in an iteration
+    constexpr int kInFlight = (kRA - 2) * kNA + (kRW - 2) * kNW;   // loads that may be outstanding at a barrier
+    static_assert(kInFlight <= 63, "vmcnt is a 6-bit counter");
+    const char* aptr[kNA];
+    const char* wptr[kNW];
 #pragma unroll
-    for (int i = 0; i < kN; ++i) {
-      const int blk = i * kWaves + wave;
-      const int r = blk * 8 + (lane >> 3);
+    for (int i = 0; i < kNA; ++i) {
+      const int r = (i * kWaves + wave) * 8 + (lane >> 3);
       const int c = (lane & 7) ^ ((r >> 1) & 7);
-      if (blk * 8 < Cfg::kBM) {          // uniform per (wave, i)
-        int64_t row = m0 + r;
-        row = row < a.M ? row : a.M - 1;
-        gptr[i] = reinterpret_cast<const char*>(a.A + row * a.lda + c * kPer);
-      } else {
-        int64_t row = n0 + r - Cfg::kBM;
-        row = row < a.N ? row : a.N - 1;
-        gptr[i] = reinterpret_cast<const char*>(a.W + row * a.K + c * kPer);
-      }
+      int64_t row = m0 + r;
+      row = row < a.M ? row : a.M - 1;
+      aptr[i] = reinterpret_cast<const char*>(a.A + row * a.lda + c * kPer);
+    }
+#pragma unroll
+    for (int i = 0; i < kNW; ++i) {
+      const int r = (i * kWaves + wave) * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ ((r >> 1) & 7);
+      int64_t row = n0 + r;
+      row = row < a.N ? row : a.N - 1;
+      wptr[i] = reinterpret_cast<const char*>(a.W + row * a.K + c * kPer);
     }
     const unsigned lds_base = (unsigned)reinterpret_cast<uintptr_t>(lds);
-    constexpr int kNB = Cfg::kDmaBufs;
-    static_assert(kNB >= 2 && (kNB - 2) * kN <= 63, "vmcnt is a 6-bit counter");
-    auto dma_tile = [&](int buf, int64_t kt_in) {
+    constexpr int kWRing = kRA * Cfg::kATileBytes;          // the W ring lies behind the A ring
+    auto dma_a = [&](int buf, int64_t kt_in) {
       const int64_t kt = kt_in >= nk ? nk - 1 : kt_in;    // past the end: re-read, never used
-      if (NT_GEMM_ABLATE & 2) return;
 #pragma unroll
-      for (int i = 0; i < kN; ++i) {
+      for (int i = 0; i < kNA; ++i) {
         const unsigned dst = __builtin_amdgcn_readfirstlane(
-            lds_base + (unsigned)(buf * Cfg::kDmaTileBytes + (i * kWaves + wave) * 1024));
-        const char* src = gptr[i] + kt * Cfg::kRowBytes;
+            lds_base + (unsigned)(buf * Cfg::kATileBytes + (i * kWaves + wave) * 1024));
+        const char* src = aptr[i] + kt * Cfg::kRowBytes;
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                     :: "v"(src), "s"(dst) : "memory");
+      }
+    };
+    auto dma_w = [&](int buf, int64_t kt_in) {
+      const int64_t kt = kt_in >= nk ? nk - 1 : kt_in;
+#pragma unroll
+      for (int i = 0; i < kNW; ++i) {
+        const unsigned dst = __builtin_amdgcn_readfirstlane(
+            lds_base + (unsigned)(kWRing + buf * Cfg::kBTileBytes + (i * kWaves + wave) * 1024));
+        const char* src = wptr[i] + kt * Cfg::kRowBytes;
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                      :: "v"(src), "s"(dst) : "memory");
       }
     };
     const int sw = (l32 >> 1) & 7;
-    auto read_frags = [&](Frag* fa, Frag* fb, int buf, int s) {
-      const char* a_base = lds + buf * Cfg::kDmaTileBytes + (wm * WM * 32 + l32) * 128;
-      const char* b_base = lds + buf * Cfg::kDmaTileBytes + (Cfg::kBM + wn * WN * 32 + l32) * 128;
+    auto read_frags = [&](Frag* fa, Frag* fb, int abuf, int wbuf, int s) {
+      const char* a_base = lds + abuf * Cfg::kATileBytes + (wm * WM * 32 + l32) * 128;
+      const char* b_base = lds + kWRing + wbuf * Cfg::kBTileBytes + (wn * WN * 32 + l32) * 128;
       const int off = s * MM::kK * (int)sizeof(T) + g * kFragBytes;   // byte offset in the row
       const int koff = ((((off >> 4) ^ sw)) << 4) | (off & 15);
 #pragma unroll
@@ -276,54 +289,69 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& a, int64_t m0, int6
       for (int j = 0; j < WN; ++j)
         fb[j] = *reinterpret_cast<const Frag*>(b_base + j * 32 * 128 + koff);
     };
-    // K tiles kt + 1 .. kt + kNB - 1 are resident or in flight while tile kt is
-    // multiplied; the loads of the newest kNB - 2 tiles may still be outstanding
-    // when the barrier publishes tile kt + 1 (loads complete in order).
+    // While K tile kt is multiplied, the tiles kt + 1 .. kt + kRA - 1 of A and
+    // kt + 1 .. kt + kRW - 1 of W are resident or in flight.  Loads complete in the
+    // order of issue and every iteration issues the tile of the deeper ring last,
+    // so when at most kInFlight loads are outstanding, tile kt + 1 of both has landed.
+    // Prologue: tiles in the order the loop would have issued them.
 #pragma unroll
-    for (int j = 0; j < kNB - 1; ++j) dma_tile(j, j);
-    asm volatile("s_waitcnt vmcnt(%0)" :: "n"((kNB - 2) * kN) : "memory");
-    __syncthreads();
-    int buf = 0;
-    Frag fa[2][WM], fb[2][WN];
-    if (NT_GEMM_ABLATE & 4) {
-      read_frags(fa[0], fb[0], 0, 0);
-      read_frags(fa[1], fb[1], 0, 1);
+    for (int j = 0; j < (kRA > kRW ? kRA : kRW) - 1; ++j) {
+      if (!kWLast && j < kRW - 1) dma_w(j, j);
+      if (j < kRA - 1) dma_a(j, j);
+      if (kWLast && j < kRW - 1) dma_w(j, j);
     }
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kInFlight) : "memory");
+    __syncthreads();
+    int abuf = 0, wbuf = 0;
+    Frag fa[2][WM], fb[2][WN];
     for (int64_t kt = 0; kt < nk; ++kt) {
-      const int buf_new = buf == 0 ? kNB - 1 : buf - 1;    // == (kt + kNB - 1) % kNB, free since the last barrier
-      dma_tile(buf_new, kt + kNB - 1);
-      if (NT_GEMM_ABLATE & 4) {
-        asm volatile("" : "+v"(fa[0][0]), "+v"(fb[0][0]), "+v"(fa[1][0]), "+v"(fb[1][0]));
-      } else {
-        read_frags(fa[0], fb[0], buf, 0);
-      }
+      // (kt + kR - 1) % kR: free since the last barrier
+      // This iteration's loads (the tile of the shallower ring first) are not issued
+      // in one burst: a DMA load occupies the issuing wavefront until the memory
+      // path has taken its 64 addresses, so a burst keeps every wavefront of the
+      // workgroup from its matrix instructions at the same time.  They are dealt out
+      // behind the k-steps instead.
+      const int a_new = abuf == 0 ? kRA - 1 : abuf - 1;     // (kt + kR - 1) % kR: free since the last barrier
+      const int w_new = wbuf == 0 ? kRW - 1 : wbuf - 1;
+      const int64_t a_kt = kt + kRA - 1 >= nk ? nk - 1 : kt + kRA - 1;   // past the end: re-read, never used
+      const int64_t w_kt = kt + kRW - 1 >= nk ? nk - 1 : kt + kRW - 1;
+      auto dma_one = [&](int idx) {
+        const bool is_w = kWLast ? idx >= kNA : idx < kNW;
+        const int i = kWLast ? (is_w ? idx - kNA : idx) : (is_w ? idx : idx - kNW);
+        const unsigned off = is_w ? (unsigned)(kWRing + w_new * Cfg::kBTileBytes) : (unsigned)(a_new * Cfg::kATileBytes);
+        const unsigned dst = __builtin_amdgcn_readfirstlane(lds_base + off + (unsigned)((i * kWaves + wave) * 1024));
+        const char* src = is_w ? wptr[i] + w_kt * Cfg::kRowBytes : aptr[i] + a_kt * Cfg::kRowBytes;
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                     :: "v"(src), "s"(dst) : "memory");
+      };
+      constexpr int kLoads = kNA + kNW;
+      read_frags(fa[0], fb[0], abuf, wbuf, 0);
 #pragma unroll
       for (int s = 0; s < kSteps; ++s) {
-        if (s + 1 < kSteps && !(NT_GEMM_ABLATE & 4)) read_frags(fa[(s + 1) & 1], fb[(s + 1) & 1], buf, s + 1);
-        if (NT_GEMM_ABLATE & 1) {
-          asm volatile("" ::"v"(fa[s & 1][0]), "v"(fb[s & 1][0]), "v"(fa[s & 1][WM - 1]), "v"(fb[s & 1][WN - 1]));
-        } else {
+        if (s + 1 < kSteps) read_frags(fa[(s + 1) & 1], fb[(s + 1) & 1], abuf, wbuf, s + 1);
 #pragma unroll
-          for (int i = 0; i < WM; ++i)
+        for (int i = 0; i < WM; ++i)
 #pragma unroll
-            for (int jj = 0; jj < WN; ++jj) {
-              if (VT_OUT) {
-                acc[i][jj] = MM::run(fa[s & 1][i], fb[s & 1][jj], acc[i][jj]);
-              } else {
-                acc[i][jj] = MM::run(fb[s & 1][jj], fa[s & 1][i], acc[i][jj]);
-              }
+          for (int jj = 0; jj < WN; ++jj) {
+            if (VT_OUT) {
+              acc[i][jj] = MM::run(fa[s & 1][i], fb[s & 1][jj], acc[i][jj]);
+            } else {
+              acc[i][jj] = MM::run(fb[s & 1][jj], fa[s & 1][i], acc[i][jj]);
             }
-        }
+          }
+#pragma unroll
+        for (int idx = s * kLoads / kSteps; idx < (s + 1) * kLoads / kSteps; ++idx) dma_one(idx);
         __builtin_amdgcn_sched_barrier(0);
       }
-      asm volatile("s_waitcnt vmcnt(%0)" :: "n"((kNB - 2) * kN) : "memory");
-      if (!(NT_GEMM_ABLATE & 8)) __syncthreads();
-      buf = buf + 1 == kNB ? 0 : buf + 1;
+      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kInFlight) : "memory");
+      __syncthreads();
+      abuf = abuf + 1 == kRA ? 0 : abuf + 1;
+      wbuf = wbuf + 1 == kRW ? 0 : wbuf + 1;
     }
-    // The last kNB - 1 iterations issued clamped re-reads of the last K tile; up to
-    // (kNB - 2) * kN of them per lane may still be in flight, and their LDS
-    // destinations overlap the strips of the epilogue.  Drain them, workgroup-wide.
-    if (kNB > 2) {
+    // The last iterations issued clamped re-reads of the last K tile; up to
+    // kInFlight of them per lane may still be in flight, and their LDS destinations
+    // overlap the strips of the epilogue.  Drain them, workgroup-wide.
+    if (kInFlight > 0) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
     }
@@ -581,7 +609,6 @@ static int pick_cfg(int64_t M, int64_t N, int64_t n_split, int* which) {
   double best_cost = 0.0;
   for (int c = 0; c < 3; ++c) {
     if (n_split % bn[c] != 0) continue;          // a tile must not straddle the K | V boundary
-    if (NT_GEMM_FORCE_CFG >= 0 && c != NT_GEMM_FORCE_CFG) continue;
     const int64_t tiles = ((M + 255) / 256) * ((N + bn[c] - 1) / bn[c]);
     const double whole = (double)((tiles + num_cus - 1) / num_cus);
     const double fluid = (double)tiles / num_cus;
