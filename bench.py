@@ -345,7 +345,43 @@ def mha_probe(args, torch, dev):
                                   wavefront_key_tiles=count * q_tiles * 4 * k_tiles * H,
                                   flops=4 * E * count * length * length))
             out["attention_length_sweep"] = sweep
+    out["instruction_rates"] = instruction_rates()
     print(json.dumps(out))
+
+
+def instruction_rates():
+    """Nanoseconds a SIMD spends per wavefront-wide instruction (every SIMD of the
+    chip loaded alike, 1 to 3 wavefronts per SIMD), from libnt_probe.so: the
+    transcendental and conversion instructions of the softmax against v_fma_f32,
+    the matrix instruction, 16-byte LDS reads, and three mixed streams (16 matrix
+    instructions with 128 multiply-adds and / or 32 exponentials per iteration)
+    whose time beside the sum of their parts says how much of the vector work
+    runs in the shadow of the matrix pipe."""
+    path = os.path.join(ROOT, "nestedtensor_amd", "libnt_probe.so")
+    if not os.path.exists(path):
+        return "libnt_probe.so is not built (make -C nestedtensor_amd/csrc)"
+    lib = ctypes.CDLL(path)
+    lib.nt_probe_rate.restype = ctypes.c_int
+    lib.nt_probe_rate.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float),
+                                  ctypes.POINTER(ctypes.c_int)]
+    names = ["v_fma_f32", "v_exp_f32", "v_exp_f16", "v_cvt_pk_f16_f32", "v_dot2_f32_f16", "v_max3_f32 (2 x v_max)",
+             "v_mfma_f32_32x32x16_f16", "ds_read_b128", "16 mfma + 128 fma (per iteration)",
+             "16 mfma + 32 exp (per iteration)", "16 mfma + 128 fma + 32 exp (per iteration)"]
+    iters = 2000
+    res = {}
+    for kind, name in enumerate(names):
+        row = {}
+        for waves in (1, 2, 3):
+            ms, per = ctypes.c_float(), ctypes.c_int()
+            rc = lib.nt_probe_rate(kind, waves, iters, ctypes.byref(ms), ctypes.byref(per))
+            if rc != 0:
+                row["%d_waves_per_simd" % waves] = "probe failed (%d)" % rc
+                continue
+            # the SIMD runs `waves` wavefronts, each `iters * per` instructions
+            row["%d_waves_per_simd" % waves] = round(ms.value * 1e6 / (iters * per.value * waves), 3)
+        res[name] = row
+    res["unit"] = "ns per instruction (mixed rows: per iteration) and SIMD"
+    return res
 
 
 def cpu_baseline_c5(torch, n_sample=128):

@@ -229,6 +229,17 @@ int nt_linear_qkv(const void* A, int64_t lda, const void* W, const void* bias, v
                   int64_t ldqk, void* Vt, int64_t ldvt, int64_t M, int64_t E, int64_t K,
                   int dtype, void* stream);
 
+/* The key and value projections of cross-attention in one launch, for keys and
+ * values that are the same tensor (the usual `memory` of a decoder layer):
+ * [Kp | V] = A * W^T + bias with W [2E, K] (rows [E, 3E) of an in-projection
+ * weight); Kp is written row-major into Kout[M, E] (row stride ldk), V transposed
+ * into Vt[e][m] (row stride ldvt >= M; nt_varlen_attention_vt wants >= M + 72).
+ * E must be a multiple of 128.  Replaces the `k` and `v` matmuls and bias adds of
+ * min_mha (nestedtensor/csrc/mha.cpp:45-54) when key and value are one buffer: A
+ * is read once instead of twice. */
+int nt_linear_kv(const void* A, int64_t lda, const void* W, const void* bias, void* Kout, int64_t ldk,
+                 void* Vt, int64_t ldvt, int64_t M, int64_t E, int64_t K, int dtype, void* stream);
+
 /* Ct[n][m] = (A[M, K] * W[N, K]^T + bias[N])[m][n]: nt_linear with the result
  * written transposed (row stride ldct >= M).  The value projection of
  * cross-attention (nestedtensor/csrc/mha.cpp:48-54, the `v` matmul and bias add)

@@ -57,6 +57,8 @@ SIGNATURES = {
                              _int, _int, _c_void_p]),
     "nt_linear_qkv": (_int, [_c_void_p, _i64, _c_void_p, _c_void_p, _c_void_p, _i64, _c_void_p, _i64, _i64,
                              _i64, _i64, _int, _c_void_p]),
+    "nt_linear_kv": (_int, [_c_void_p, _i64, _c_void_p, _c_void_p, _c_void_p, _i64, _c_void_p, _i64, _i64,
+                            _i64, _i64, _int, _c_void_p]),
     "nt_linear_transposed": (_int, [_c_void_p, _i64, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _i64,
                                     _int, _c_void_p]),
     "nt_varlen_attention_vt": (_int, [_c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64,

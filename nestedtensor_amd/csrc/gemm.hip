@@ -744,6 +744,35 @@ extern "C" int nt_linear_qkv(const void* A, int64_t lda, const void* W, const vo
 #undef NT_QKV_CASE
 }
 
+extern "C" int nt_linear_kv(const void* A, int64_t lda, const void* W, const void* bias, void* Kout,
+                            int64_t ldk, void* Vt, int64_t ldvt, int64_t M, int64_t E, int64_t K, int dtype,
+                            void* stream) {
+  int rc = check_linear(A, lda, W, Kout, ldk, M, 2 * E, K);
+  if (rc != NT_OK) return rc;
+  if (ldk < E || ldvt < M) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "linear_kv: ldk %lld < E or ldvt %lld < M", (long long)ldk, (long long)ldvt);
+  }
+  if (M == 0 || E == 0) return NT_OK;
+  if (!Vt) return fail(NT_ERR_INVALID_ARGUMENT, "linear_kv: Vt is NULL");
+  hipStream_t s = (hipStream_t)stream;
+  // the fused in-projection's kernel with the row-major | transposed boundary at column E
+#define NT_KV_CASE(TYPE)                                                        \
+  {                                                                             \
+    GemmArgs<TYPE> a = make_args<TYPE>(A, lda, W, bias, Kout, ldk, M, 2 * E, K); \
+    a.Vt = static_cast<TYPE*>(Vt);                                              \
+    a.ldvt = ldvt;                                                              \
+    a.n_split = E;                                                              \
+    return launch_linear<TYPE>(a, true, s);                                     \
+  }
+  switch (dtype) {
+    case NT_F32: NT_KV_CASE(float)
+    case NT_F16: NT_KV_CASE(_Float16)
+    case NT_BF16: NT_KV_CASE(__bf16)
+    default: return fail(NT_ERR_INVALID_ARGUMENT, "linear_kv: unknown dtype %d", dtype);
+  }
+#undef NT_KV_CASE
+}
+
 extern "C" int nt_linear_transposed(const void* A, int64_t lda, const void* W, const void* bias,
                                     void* Ct, int64_t ldct, int64_t M, int64_t N, int64_t K, int dtype,
                                     void* stream) {

@@ -1098,14 +1098,26 @@ Tensor mha_cross_packed(const Tensor& xq, const Tensor& xk, const Tensor& xv, co
   Tensor out = at::empty({Tq, N}, xq.options());
   if (Tq == 0) return out;
   Tensor q = project_rows(xq, W, b_in, 0, E, stream);
-  Tensor k = project_rows(xk, W, b_in, E, E, stream);
   const int64_t ldvt = (Tk + 72 + 7) / 8 * 8;
   Tensor vt = at::empty({E, ldvt}, xq.options());
   const int64_t es = static_cast<int64_t>(xq.element_size());
-  check(nt_linear_transposed(xv.const_data_ptr(), xv.stride(0),
-                             static_cast<const char*>(W.const_data_ptr()) + 2 * E * E * es,
-                             b_in.defined() ? static_cast<const char*>(b_in.const_data_ptr()) + 2 * E * es : nullptr,
-                             vt.data_ptr(), ldvt, Tk, E, E, dt, stream));
+  Tensor k;
+  if (xk.const_data_ptr() == xv.const_data_ptr() && xk.stride(0) == xv.stride(0) && E % 128 == 0) {
+    // key and value are one buffer (the `memory` of a decoder layer): both
+    // projections in one launch, the buffer read once
+    k = at::empty({Tk, E}, xq.options());
+    if (Tk > 0) {
+      check(nt_linear_kv(xk.const_data_ptr(), xk.stride(0), static_cast<const char*>(W.const_data_ptr()) + E * E * es,
+                         b_in.defined() ? static_cast<const char*>(b_in.const_data_ptr()) + E * es : nullptr,
+                         k.data_ptr(), E, vt.data_ptr(), ldvt, Tk, E, E, dt, stream));
+    }
+  } else {
+    k = project_rows(xk, W, b_in, E, E, stream);
+    check(nt_linear_transposed(xv.const_data_ptr(), xv.stride(0),
+                               static_cast<const char*>(W.const_data_ptr()) + 2 * E * E * es,
+                               b_in.defined() ? static_cast<const char*>(b_in.const_data_ptr()) + 2 * E * es : nullptr,
+                               vt.data_ptr(), ldvt, Tk, E, E, dt, stream));
+  }
   Tensor attn = at::empty({Tq, E}, xq.options());
   check(nt_varlen_attention_vt(q.const_data_ptr(), E, k.const_data_ptr(), E, vt.const_data_ptr(), ldvt, attn.data_ptr(), E,
                                schedule.const_data_ptr<int32_t>(), schedule.size(0), num_heads, head_dim, Tk,

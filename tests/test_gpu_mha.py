@@ -241,6 +241,30 @@ def test_linear_transposed(M, N, K, dtype):
     assert bool((ct[:, M:] == 7.0).all())          # nothing is written past column M
 
 
+@pytest.mark.parametrize("M,E,K", [(300, 128, 128), (777, 256, 64), (5, 384, 200)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_linear_kv_one_launch(M, E, K, dtype):
+    # key projection row-major and value projection transposed from one launch
+    # (mha.cpp:45-54 for key and value that are one tensor), against float64
+    from nestedtensor_amd import _C
+    g = torch.Generator().manual_seed(23)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    w = (torch.randn(2 * E, K, generator=g) * 0.2).to(dtype)
+    b = torch.randn(2 * E, generator=g).to(dtype)
+    ld = (M + 72 + 7) // 8 * 8
+    kp = torch.full((M, E), 7.0, dtype=dtype, device=DEV)
+    vt = torch.full((E, ld), 7.0, dtype=dtype, device=DEV)
+    xd, wd, bd = x.to(DEV), w.to(DEV), b.to(DEV)
+    _C.check(_C.lib.nt_linear_kv(_C.ptr(xd), K, _C.ptr(wd), _C.ptr(bd), _C.ptr(kp), E, _C.ptr(vt), ld, M, E, K,
+                                 _C.dtype_code(dtype), _C.current_stream(DEV)))
+    ref = x.double() @ w.double().t() + b.double()
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    scale = max(1.0, ref.abs().max().item())
+    assert (kp.double().cpu() - ref[:, :E]).abs().max().item() <= tol * scale
+    assert (vt[:, :M].double().cpu() - ref[:, E:].t()).abs().max().item() <= tol * scale
+    assert bool((vt[:, M:] == 7.0).all())          # nothing is written past column M
+
+
 def test_mha_input_errors():
     a = nt.nested_tensor([torch.randn(3, 4), torch.randn(2, 4)], device=DEV)
     b2 = nt.nested_tensor([torch.randn(3), torch.randn(2)], device=DEV)
