@@ -61,14 +61,16 @@ METRIC = "ragged->padded HBM GB/s + nested BERT MHA tokens/s (B=32, L<=512, d=76
 
 
 @contextlib.contextmanager
-def _no_gc():
+def _no_gc(collect=True):
     """Timed regions run with Python's cyclic collector off (and collected just
-    before).  A full collection walks every tracked object of the interpreter,
-    about 40 ms with torch imported, and starts whenever the allocation counters
-    say so: inside a loop of 20-microsecond calls it is a stall of two thousand
-    calls' worth that has nothing to do with the call being timed."""
+    before, unless the caller has done that ahead of its warm-up).  A full
+    collection walks every tracked object of the interpreter, about 40 ms with
+    torch imported, and starts whenever the allocation counters say so: inside a
+    loop of 20-microsecond calls it is a stall of two thousand calls' worth that
+    has nothing to do with the call being timed."""
     was = gc.isenabled()
-    gc.collect()
+    if collect:
+        gc.collect()
     gc.disable()
     try:
         yield
@@ -152,6 +154,12 @@ def bench_c5(args, torch, dev):
         _C.check(_C.lib.nt_remove_padding(_C.ptr(padded_buf), _C.ptr(unpacked_buf), _C.ptr(m["offsets"]),
                                           _C.ptr(m["sizes"]), m["impl"].B, 2, 1, m["ext"], eb, stream))
 
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(len(meta) * args.steps)]
+    step_start = torch.cuda.Event(enable_timing=True)
+    step_end = torch.cuda.Event(enable_timing=True)
+    # (the collector runs here, before the warm-up, not between it and the timed steps:
+    # its 40 ms would be an idle spell after which the device's clocks start low)
+    gc.collect()
     # warm-up, with the size-independent parity property of the full-size run:
     # un-pad(pad(x)) == x bit-exact, and the padding region reads as the pad value
     for w in range(max(args.warmup, 1)):
@@ -168,12 +176,7 @@ def bench_c5(args, torch, dev):
                 b_short = int(torch.argmin(lens))
                 assert bool((pv[b_short, int(lens[b_short]):] == 0).all()), "padding region is not the pad value"
     torch.cuda.synchronize()
-
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(len(meta) * args.steps)]
-    step_start = torch.cuda.Event(enable_timing=True)
-    step_end = torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    with _no_gc():
+    with _no_gc(collect=False):
         t0 = time.perf_counter()
         step_start.record()
         i = 0
@@ -298,6 +301,23 @@ def mha_probe(args, torch, dev):
         out[tag] = dict(tokens=T, embed=E, heads=H, sum_L2=sum(L * L for L in lens),
                         flops_in_proj=2 * T * E * 3 * E, flops_out_proj=2 * T * E * E,
                         flops_attention=4 * E * sum(L * L for L in lens))
+        if dtype != torch.float32:
+            # the same layer with the planned attention kernel (two more dispatches of the
+            # projections and two of varlen_attention_planned_kernel), and both timed
+            def layer():
+                return op(H, 64, 0.0, False, a, a, a, W_in, b_in, 64 ** -0.5, W_out, b_out)
+            out[tag]["layer_us_work_list"] = round(_event_us(torch, layer), 2)
+            nt.set_attention_kernel("planned")
+            try:
+                for _ in range(2):
+                    layer()
+                torch.cuda.synchronize()
+                out[tag]["layer_us_planned"] = round(_event_us(torch, layer), 2)
+            finally:
+                nt.set_attention_kernel("work_list")
+            # and the default once more, so that a drift of the clocks between the two
+            # measurements above would show
+            out[tag]["layer_us_work_list_again"] = round(_event_us(torch, layer), 2)
         if tag == "C3":
             x = a._impl.buffer.reshape(T, E)
             for _ in range(2):
@@ -340,13 +360,44 @@ def mha_probe(args, torch, dev):
                         _C.ptr(qk), 2 * E, kptr, 2 * E, _C.ptr(vt), ldvt, _C.ptr(o), E, _C.ptr(sched),
                         sched.size(0), H, 64, Tn, 0.125, _C.dtype_code(dtype), _C.current_stream(dev)))
                 torch.cuda.synchronize()
+                plan = impl.attention_plan(H, 64)
+                n_wg = torch.cuda.get_device_properties(dev).multi_processor_count
+
+                def work_list():
+                    _C.check(_C.lib.nt_varlen_attention_vt(
+                        _C.ptr(qk), 2 * E, kptr, 2 * E, _C.ptr(vt), ldvt, _C.ptr(o), E, _C.ptr(sched),
+                        sched.size(0), H, 64, Tn, 0.125, _C.dtype_code(dtype), _C.current_stream(dev)))
+
+                def planned():
+                    _C.check(_C.lib.nt_varlen_attention_planned(
+                        _C.ptr(qk), 2 * E, kptr, 2 * E, _C.ptr(vt), ldvt, _C.ptr(o), E, _C.ptr(plan), n_wg,
+                        H, 64, Tn, 0.125, _C.dtype_code(dtype), _C.current_stream(dev)))
+                for _ in range(2):
+                    planned()
+                torch.cuda.synchronize()
                 q_tiles, k_tiles = (length + 127) // 128, (length + 63) // 64
                 sweep.append(dict(sequences=count, length=length, workgroups=count * q_tiles * H,
                                   wavefront_key_tiles=count * q_tiles * 4 * k_tiles * H,
-                                  flops=4 * E * count * length * length))
+                                  flops=4 * E * count * length * length,
+                                  us_work_list=round(_event_us(torch, work_list), 2),
+                                  us_planned=round(_event_us(torch, planned), 2)))
             out["attention_length_sweep"] = sweep
     out["instruction_rates"] = instruction_rates()
     print(json.dumps(out))
+
+
+def _event_us(torch, fn, iters=20, warmup=3):
+    """Mean time of one call of fn in microseconds, from events on the current
+    stream around `iters` back-to-back calls."""
+    for _ in range(warmup):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1000.0 / iters
 
 
 def instruction_rates():
@@ -436,6 +487,7 @@ def bench_mha_c3(args, torch, dev, later):
 
     out = layer()
     ms = _time_gpu(torch, layer, iters=50, warmup=5)
+    ms_drained = _time_gpu(torch, layer, iters=50, warmup=5, from_idle=True)
     iters = 50
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     # the same three launches replayed from a HIP graph (no host work between them)
@@ -449,16 +501,7 @@ def bench_mha_c3(args, torch, dev, later):
             with torch.cuda.graph(graph, stream=side):
                 gout = layer()
         torch.cuda.current_stream().wait_stream(side)
-        for _ in range(5):
-            graph.replay()
-        torch.cuda.synchronize()
-        with _no_gc():
-            e0.record()
-            for _ in range(iters):
-                graph.replay()
-            e1.record()
-            torch.cuda.synchronize()
-        graph_ms = e0.elapsed_time(e1) / iters
+        graph_ms = float(_time_gpu(torch, graph.replay, iters=iters, warmup=5))
         assert torch.equal(gout._impl.buffer, out._impl.buffer)
     except Exception as exc:      # report, do not hide
         graph_ms = "graph capture failed: %r" % (exc,)
@@ -535,7 +578,8 @@ def bench_mha_c3(args, torch, dev, later):
     flops_enc = flops + 16 * T * E * E
     res = dict(workload="C3: nested BERT-base self-attention, fp16, B=32, L~U[32,512], d=768, 12x64",
                tokens=T, ms_per_layer=float(ms), ms_per_layer_max=ms.max, ms_per_layer_mean=ms.mean,
-               timing=ms.fields()["timing"], ms_per_layer_hip_graph=graph_ms,
+               timing=ms.fields()["timing"] + ", queued behind 30 ms of the same calls",
+               ms_per_layer_queue_drained_first=float(ms_drained), ms_per_layer_hip_graph=graph_ms,
                tokens_per_s=T / (ms * 1e-3), flops=flops, kernel_us=kernel_us, dense_padded_torch=dense,
                roofline=dict(bound="mfma", achieved=flops / (ms * 1e-3) / 1e12, peak=MFMA_F16_PEAK_TFLOPS,
                              unit="TFLOP/s", frac=flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS))
@@ -575,7 +619,7 @@ def _mha_kernel_times(torch, dev, a, W_in, b_in, W_out, b_out, H, hd):
     E = H * hd
     x = impl.buffer.reshape(-1, E)
     T = x.size(0)
-    ldvt = (T + 72 + 7) // 8 * 8
+    ldvt = (T + 72 + 63) // 64 * 64
     qk = torch.empty(T, 2 * E, device=dev, dtype=x.dtype)
     vt = torch.zeros(E, ldvt, device=dev, dtype=x.dtype)
     attn = torch.empty(T, E, device=dev, dtype=x.dtype)
@@ -615,16 +659,33 @@ class Ms(float):
                     timing="median / max / mean over %d batches of %d calls" % (self.batches, self.per))
 
 
-def _time_gpu(torch, fn, iters=20, warmup=3, per=5):
+def _time_gpu(torch, fn, iters=20, warmup=3, per=5, warm_s=0.03, from_idle=False):
     """`iters` calls of fn (rounded up to whole batches of `per`), an event
     between batches.  Events are not put between single calls: an event costs
-    the device a few microseconds, which is the size of the smallest rows."""
-    for _ in range(warmup):
-        fn()
-    batches = max(3, -(-iters // per))
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(batches + 1)]
-    torch.cuda.synchronize()
+    the device a few microseconds, which is the size of the smallest rows.
+    The untimed calls go on for at least `warm_s` seconds of queued work, and
+    the timed batches follow them at once (the collector runs BEFORE the untimed
+    calls: its 40 ms are an idle spell for the device): after an idle spell the
+    device takes about 15 ms of continuous load to reach the clocks it then
+    holds, and a 100 us layer timed over its first fifty calls reads 10 to 15 %
+    slower than in a loop that keeps the device busy.  from_idle=True drains the
+    queue before the timed batches (the device then starts each call as the
+    host issues it)."""
     with _no_gc():
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(per):
+            fn()
+        torch.cuda.synchronize()
+        per_call = max((time.perf_counter() - t0) / per, 1e-6)
+        batches = max(3, -(-iters // per))
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(batches + 1)]
+        for _ in range(min(int(warm_s / per_call), 4000)):
+            fn()
+        if from_idle:
+            torch.cuda.synchronize()
         ev[0].record()
         for b in range(batches):
             for _ in range(per):

@@ -268,6 +268,39 @@ int nt_varlen_attention_vt(const void* q, int64_t ldq, const void* k, int64_t ld
                            int64_t n_work, int64_t num_heads, int64_t head_dim,
                            int64_t total_kv_tokens, float scale, int dtype, void* stream);
 
+/* The same attention from a PLAN instead of a work list (head_dim 64, f16 / bf16):
+ * persistent workgroups, one per compute unit, twelve wavefronts each, that bring a
+ * sequence's K and V^T tiles into LDS with direct global -> LDS loads, 256 keys per
+ * step, and give every wavefront one block of 32 query rows: K / V^T are read once
+ * per 384 query rows, there is one barrier per 256 keys, and short sequences share
+ * a workgroup.  An alternative to nt_varlen_attention_vt with the same results to
+ * rounding; on the attention benchmarks of this library it is the slower of the two
+ * (the host layer uses it only on request).  Replaces the same reference chain as
+ * nt_varlen_attention_vt (nestedtensor/csrc/cuda/mha.cpp:59-105, the masked softmax
+ * of nestedtensor/csrc/cuda/attention.cu:182-482), with the semantics of the
+ * per-sequence loop of min_mha (nestedtensor/csrc/mha.cpp:58-65).
+ *
+ * nt_attention_plan builds the plan on the HOST from the query and key lengths
+ * of the B sequences (host int64 arrays; a sequence with queries must have
+ * keys) for `num_heads` heads and `n_workgroups` workgroups (<= 0: the compute
+ * units of the current device).  It returns the number of int32 the plan holds,
+ * or minus an NT_ERR_* code, and writes the plan when `plan` is not NULL and
+ * `capacity` (in int32) suffices: call it once with NULL to size the buffer.
+ * plan[0] is the number of workgroups to launch.  The caller copies the plan to
+ * device memory; it depends on the lengths, the head count and the workgroup
+ * count only, so it can be kept for as long as the nested size lives. */
+int64_t nt_attention_plan(const int64_t* q_lens, const int64_t* k_lens, int64_t B, int64_t num_heads,
+                          int64_t head_dim, int64_t n_workgroups, int32_t* plan, int64_t capacity);
+
+/* Operands as nt_varlen_attention_vt (Q, K row-major with 16-byte aligned K rows,
+ * V transposed with ldvt >= total_kv_tokens + 72); `plan` is the DEVICE copy of
+ * what nt_attention_plan built for these sequences and head count, n_workgroups
+ * its plan[0].  The kernel cannot check the plan against the buffers. */
+int nt_varlen_attention_planned(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* vt,
+                                int64_t ldvt, void* out, int64_t ldo, const int32_t* plan,
+                                int64_t n_workgroups, int64_t num_heads, int64_t head_dim,
+                                int64_t total_kv_tokens, float scale, int dtype, void* stream);
+
 /* nt_varlen_attention (V row-major) driven by the work list of
  * nt_varlen_attention_vt instead of a padded grid: one workgroup per (item,
  * head), so only query tiles that exist are launched and the long sequences

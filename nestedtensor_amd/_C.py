@@ -63,6 +63,9 @@ SIGNATURES = {
                                     _int, _c_void_p]),
     "nt_varlen_attention_vt": (_int, [_c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64,
                                       _c_void_p, _i64, _i64, _i64, _i64, _f32, _int, _c_void_p]),
+    "nt_attention_plan": (_i64, [_c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _c_void_p, _i64]),
+    "nt_varlen_attention_planned": (_int, [_c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64,
+                                           _c_void_p, _i64, _i64, _i64, _i64, _f32, _int, _c_void_p]),
     "nt_varlen_attention_scheduled": (_int, [_c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64,
                                              _c_void_p, _i64, _i64, _i64, _f32, _int, _c_void_p]),
     "nt_varlen_attention": (_int, [_c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64, _c_void_p, _i64,

@@ -21,7 +21,7 @@ from .nested.nested import transpose_nchw_nhwc
 from .nested.nested import transpose_nhwc_nchw
 from .nested.nested import linear_act
 
-from .ops import set_index_check
+from .ops import set_attention_kernel, set_index_check
 from .ops import check_index_errors
 
 from . import nested

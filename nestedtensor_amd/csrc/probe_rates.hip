@@ -63,8 +63,9 @@ __global__ __launch_bounds__(256) void rate_kernel(float* out, int iters) {
         h[j][0] = r;
       }
       if (OTHER == kCvtPk) {
-        float2v x = {v[j], v[(j + 1) & 15]};
-        h[j] = __builtin_convertvector(x, half2v);
+        // (as an asm statement: the operands do not change in the loop, and the
+        // compiler would hoist a plain conversion out of it)
+        asm volatile("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(h[j]) : "v"(v[j]), "v"(v[(j + 1) & 15]));
       }
       if (OTHER == kDot2) v[j] = __builtin_amdgcn_fdot2(h[j], h[(j + 1) & 15], v[j], false);
       if (OTHER == kMax3) v[j] = __builtin_fmaxf(__builtin_fmaxf(v[j], v[(j + 1) & 15]), v[(j + 2) & 15]);

@@ -782,10 +782,67 @@ Tensor linear_packed(const Tensor& x, const Tensor& weight_in, const c10::option
   return out;
 }
 
+// The attention kernels that read V transposed.  A two-dimensional `schedule` is the
+// work list of nt_varlen_attention_vt ([n_work, 8]); a one-dimensional one is the
+// device copy of a plan of nt_attention_plan, for the kernel that streams the keys
+// of a sequence through LDS (head_dim 64 only).
+int compute_units_of(const c10::Device& device) {
+  int n = 0;
+  TORCH_CHECK(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device.index()) == hipSuccess && n > 0,
+              "attention: cannot query the compute units of ", device);
+  return n;
+}
+
+void check_attention_schedule(const Tensor& schedule, const Tensor& x) {
+  TORCH_CHECK(schedule.scalar_type() == at::kInt && schedule.is_contiguous() && schedule.device() == x.device() &&
+                  ((schedule.dim() == 2 && schedule.size(1) == 8) || (schedule.dim() == 1 && schedule.size(0) >= 4)),
+              "mha: schedule must be a contiguous int32 [n_work, 8] work list or a one-dimensional plan on the "
+              "input's device");
+}
+
+void launch_attention_vt(const void* q, int64_t ldq, const void* k, int64_t ldk, const Tensor& vt, int64_t ldvt,
+                         Tensor& attn, int64_t E, const Tensor& schedule, int64_t num_heads, int64_t head_dim,
+                         int64_t total_kv, double scaling, int dt, void* stream) {
+  if (schedule.dim() == 1) {
+    TORCH_CHECK(head_dim == 64, "mha: the planned attention kernel covers head_dim 64 only");
+    // the plan was made for one workgroup per compute unit of this device (attention_plan
+    // below); a workgroup beyond the plan's own count returns at once
+    check(nt_varlen_attention_planned(q, ldq, k, ldk, vt.const_data_ptr(), ldvt, attn.data_ptr(), E,
+                                      schedule.const_data_ptr<int32_t>(), compute_units_of(attn.device()), num_heads,
+                                      head_dim, total_kv, static_cast<float>(scaling), dt, stream));
+    return;
+  }
+  check(nt_varlen_attention_vt(q, ldq, k, ldk, vt.const_data_ptr(), ldvt, attn.data_ptr(), E,
+                               schedule.const_data_ptr<int32_t>(), schedule.size(0), num_heads, head_dim, total_kv,
+                               static_cast<float>(scaling), dt, stream));
+}
+
+// Plan of the planned attention kernel for sequences of the given query and key
+// lengths (host int64 tensors), copied to `device`.
+Tensor attention_plan(const Tensor& q_lens, const Tensor& k_lens, int64_t num_heads, int64_t head_dim,
+                      c10::Device device) {
+  TORCH_CHECK(q_lens.device().is_cpu() && k_lens.device().is_cpu() && q_lens.scalar_type() == at::kLong &&
+                  k_lens.scalar_type() == at::kLong && q_lens.dim() == 1 && k_lens.dim() == 1 &&
+                  q_lens.numel() == k_lens.numel(),
+              "attention_plan: the lengths must be host int64 vectors of one size");
+  TORCH_CHECK(device.is_cuda(), "attention_plan: the plan is for a GPU");
+  const Tensor ql = q_lens.contiguous(), kl = k_lens.contiguous();
+  const int64_t B = ql.numel();
+  const int n_wg = compute_units_of(device);
+  const int64_t n = nt_attention_plan(ql.const_data_ptr<int64_t>(), kl.const_data_ptr<int64_t>(), B, num_heads, head_dim,
+                                      n_wg, nullptr, 0);
+  TORCH_CHECK(n > 0, "attention_plan: ", nt_last_error());
+  Tensor plan = at::empty({n}, at::TensorOptions().dtype(at::kInt));
+  const int64_t m = nt_attention_plan(ql.const_data_ptr<int64_t>(), kl.const_data_ptr<int64_t>(), B, num_heads, head_dim,
+                                      n_wg, plan.data_ptr<int32_t>(), n);
+  TORCH_CHECK(m == n, "attention_plan: ", nt_last_error());
+  return plan.to(device);
+}
+
 // Self-attention layer on the packed token buffer x [T, E] (min_mha, mha.cpp:18-69;
 // bt_min_mha, cuda/mha.cpp:22-107, passes no out bias): fused QKV projection with V
 // written transposed, attention over each sequence's own keys, output projection.
-// `schedule` is the device work list of nt_varlen_attention_vt.
+// `schedule` is the device work list of nt_varlen_attention_vt, or a plan (launch_attention_vt).
 Tensor mha_self_packed(const Tensor& x, const Tensor& schedule, int64_t num_heads, int64_t head_dim,
                        const Tensor& in_proj_weight, const c10::optional<Tensor>& in_proj_bias, double scaling,
                        const Tensor& out_proj_weight, const c10::optional<Tensor>& out_proj_bias) {
@@ -808,11 +865,9 @@ Tensor mha_self_packed(const Tensor& x, const Tensor& schedule, int64_t num_head
   TORCH_CHECK(Wo.dim() == 2 && Wo.size(1) == E, "linear: weight of shape ", Wo.sizes(),
               " does not match input feature size ", E);
   check_mha_weights(x, E, W, b_in, Wo, b_out);
-  TORCH_CHECK(schedule.scalar_type() == at::kInt && schedule.dim() == 2 && schedule.size(1) == 8 &&
-                  schedule.is_contiguous() && schedule.device() == x.device(),
-              "mha: schedule must be a contiguous int32 [n_work, 8] tensor on the input's device");
+  check_attention_schedule(schedule, x);
   const int64_t T = x.size(0), N = Wo.size(0);
-  const int64_t ldvt = (T + 72 + 7) / 8 * 8;   // rows readable 72 elements past the last token
+  const int64_t ldvt = (T + 72 + 63) / 64 * 64;   // rows readable 72 elements past the last token, 128-byte aligned
   c10::hip::HIPGuard guard(x.device().index());
   void* stream = stream_of(x);
   const int dt = dtype_code(st);
@@ -824,9 +879,8 @@ Tensor mha_self_packed(const Tensor& x, const Tensor& schedule, int64_t num_head
   check(nt_linear_qkv(x.const_data_ptr(), x.stride(0), W.const_data_ptr(), b_in.defined() ? b_in.const_data_ptr() : nullptr,
                       qk.data_ptr(), 2 * E, vt.data_ptr(), ldvt, T, E, E, dt, stream));
   const char* kptr = static_cast<const char*>(qk.const_data_ptr()) + E * static_cast<int64_t>(x.element_size());
-  check(nt_varlen_attention_vt(qk.const_data_ptr(), 2 * E, kptr, 2 * E, vt.const_data_ptr(), ldvt, attn.data_ptr(), E,
-                               schedule.const_data_ptr<int32_t>(), schedule.size(0), num_heads, head_dim, T,
-                               static_cast<float>(scaling), dt, stream));
+  launch_attention_vt(qk.const_data_ptr(), 2 * E, kptr, 2 * E, vt, ldvt, attn, E, schedule, num_heads, head_dim, T,
+                      scaling, dt, stream);
   check(nt_linear_act(attn.const_data_ptr(), E, Wo.const_data_ptr(), b_out.defined() ? b_out.const_data_ptr() : nullptr,
                       out.data_ptr(), N, T, N, E, 0, dt, stream));
   return out;
@@ -1087,9 +1141,7 @@ Tensor mha_cross_packed(const Tensor& xq, const Tensor& xk, const Tensor& xv, co
   if (in_proj_bias.has_value() && in_proj_bias->defined()) b_in = in_proj_bias->contiguous();
   if (out_proj_bias.has_value() && out_proj_bias->defined()) b_out = out_proj_bias->contiguous();
   check_mha_operands(xq, xk, xv, E, W, b_in, Wo, b_out);
-  TORCH_CHECK(schedule.scalar_type() == at::kInt && schedule.dim() == 2 && schedule.size(1) == 8 &&
-                  schedule.is_contiguous() && schedule.device() == xq.device(),
-              "mha: schedule must be a contiguous int32 [n_work, 8] tensor on the input's device");
+  check_attention_schedule(schedule, xq);
   const int64_t Tq = xq.size(0), Tk = xk.size(0), N = Wo.size(0);
   TORCH_CHECK(xv.size(0) == Tk, "key and value must have the same nested size.");
   c10::hip::HIPGuard guard(xq.device().index());
@@ -1098,7 +1150,7 @@ Tensor mha_cross_packed(const Tensor& xq, const Tensor& xk, const Tensor& xv, co
   Tensor out = at::empty({Tq, N}, xq.options());
   if (Tq == 0) return out;
   Tensor q = project_rows(xq, W, b_in, 0, E, stream);
-  const int64_t ldvt = (Tk + 72 + 7) / 8 * 8;
+  const int64_t ldvt = (Tk + 72 + 63) / 64 * 64;
   Tensor vt = at::empty({E, ldvt}, xq.options());
   const int64_t es = static_cast<int64_t>(xq.element_size());
   Tensor k;
@@ -1119,9 +1171,8 @@ Tensor mha_cross_packed(const Tensor& xq, const Tensor& xk, const Tensor& xv, co
                                vt.data_ptr(), ldvt, Tk, E, E, dt, stream));
   }
   Tensor attn = at::empty({Tq, E}, xq.options());
-  check(nt_varlen_attention_vt(q.const_data_ptr(), E, k.const_data_ptr(), E, vt.const_data_ptr(), ldvt, attn.data_ptr(), E,
-                               schedule.const_data_ptr<int32_t>(), schedule.size(0), num_heads, head_dim, Tk,
-                               static_cast<float>(scaling), dt, stream));
+  launch_attention_vt(q.const_data_ptr(), E, k.const_data_ptr(), E, vt, ldvt, attn, E, schedule, num_heads, head_dim, Tk,
+                      scaling, dt, stream);
   check(nt_linear_act(attn.const_data_ptr(), E, Wo.const_data_ptr(), b_out.defined() ? b_out.const_data_ptr() : nullptr,
                       out.data_ptr(), N, Tq, N, E, 0, dt, stream));
   return out;
@@ -1248,6 +1299,7 @@ TORCH_LIBRARY(nestedtensor, m) {
   m.def("softmax_rows(Tensor x, Tensor offsets, Tensor row_offsets, int total_rows, bool log) -> Tensor");
   m.def("activation_packed(Tensor x, int act) -> Tensor");
   m.def("linear_packed(Tensor x, Tensor weight, Tensor? bias, int act) -> Tensor");
+  m.def("attention_plan(Tensor q_lens, Tensor k_lens, int num_heads, int head_dim, Device device) -> Tensor");
   m.def("mha_self_packed(Tensor x, Tensor schedule, int num_heads, int head_dim, Tensor in_proj_weight, "
         "Tensor? in_proj_bias, float scaling, Tensor out_proj_weight, Tensor? out_proj_bias) -> Tensor");
   m.def("mha_cross_packed(Tensor xq, Tensor xk, Tensor xv, Tensor schedule, int num_heads, int head_dim, "
@@ -1286,6 +1338,7 @@ TORCH_LIBRARY_IMPL(nestedtensor, CUDA, m) {
 // element) for any device and raises for host tensors otherwise.
 TORCH_LIBRARY_IMPL(nestedtensor, CompositeExplicitAutograd, m) {
   m.impl("merge_tensor_mask", merge_tensor_mask);
+  m.impl("attention_plan", attention_plan);   // host lengths in, device plan out
   m.impl("nt_from_tensor_mask", nt_from_tensor_mask_op);
   m.impl("from_tensor_mask_lowered", from_tensor_mask_lowered);
 }

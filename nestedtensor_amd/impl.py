@@ -25,7 +25,7 @@ from . import _C
 
 class NestedTensorImpl:
     __slots__ = ("buffer", "sizes", "_opt_sizes", "_sizes_dev", "_offsets_dev",
-                 "_row_offsets_dev", "_max_sizes", "_attn_schedule", "_last_dim_rows", "_has_empty", "channels_last")
+                 "_row_offsets_dev", "_max_sizes", "_attn_schedule", "_attn_plan", "_last_dim_rows", "_has_empty", "channels_last")
 
     def __init__(self, buffer, sizes, channels_last=False):
         """buffer: 1-D contiguous tensor; sizes: CPU int64 [B, D], or 0-d for an
@@ -47,6 +47,7 @@ class NestedTensorImpl:
         self._row_offsets_dev = None
         self._max_sizes = None
         self._attn_schedule = None
+        self._attn_plan = None
         self._last_dim_rows = None
         self._has_empty = None
 
@@ -179,6 +180,21 @@ class NestedTensorImpl:
         self._attn_schedule = (kv.sizes, sched)      # holds kv.sizes, so the identity test stays valid
         return sched
 
+    def attention_plan(self, num_heads, head_dim, kv=None):
+        """Plan of the planned attention kernel (nt_attention_plan) for this nested
+        size, `num_heads` heads and the compute units of the buffer's device: an
+        int32 vector on the device, cached like the work list.
+        kv: the nested tensor of the keys (None: self-attention)."""
+        if kv is None or kv.sizes is self.sizes:
+            kv = self
+        cached = self._attn_plan
+        if cached is not None and cached[0] is kv.sizes and cached[1] == (num_heads, head_dim):
+            return cached[2]
+        plan = _C.ops.attention_plan.default(self.sizes[:, 0].contiguous(), kv.sizes[:, 0].contiguous(),
+                                             num_heads, head_dim, self.buffer.device)
+        self._attn_plan = (kv.sizes, (num_heads, head_dim), plan)
+        return plan
+
     def adopt_device_metadata(self, sizes_dev, offsets_dev):
         """Take over device copies of the nested size and of the element offsets
         that a conversion has already built for this nested size."""
@@ -201,6 +217,7 @@ class NestedTensorImpl:
             out._offsets_dev = self._offsets_dev
             out._row_offsets_dev = self._row_offsets_dev
             out._attn_schedule = self._attn_schedule
+            out._attn_plan = self._attn_plan
             out._last_dim_rows = self._last_dim_rows
         return out
 

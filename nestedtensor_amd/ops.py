@@ -359,6 +359,29 @@ def activation(impl, kind):
     return impl.with_buffer(_activation_packed(buf, _ACTS[kind]))
 
 
+_attention_kernel = "work_list"
+
+
+def set_attention_kernel(kind):
+    """Which kernel runs f16 / bf16 attention with head_dim 64: "work_list" (the
+    default: one small workgroup per 128 query rows of a head, the faster one on every
+    measured batch) or "planned" (persistent workgroups that stream a sequence's
+    keys through LDS from a host-made plan).  Same results to rounding; other head
+    dims always take the work list.  Returns the previous setting."""
+    global _attention_kernel
+    if kind not in ("work_list", "planned"):
+        raise ValueError("attention kernel must be 'work_list' or 'planned', not %r" % (kind,))
+    previous, _attention_kernel = _attention_kernel, kind
+    return previous
+
+
+def _attention_work(query, key, num_heads, head_dim):
+    """The device-side description of the attention work for the selected kernel."""
+    if _attention_kernel == "planned" and head_dim == 64:
+        return query.attention_plan(num_heads, head_dim, kv=key)
+    return query.attention_schedule(kv=key)
+
+
 def _check_mha_inputs(query, key, value):
     if query.dim() != 3:
         raise RuntimeError("query needs to be 3 dim.")
@@ -409,7 +432,7 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
         # self-attention, head_dim 32 / 64 / 128: Q|K row-major + V transposed straight out of
         # the projection GEMM, attention reads both without any re-layout pass, then the
         # output projection: three launches, issued by one call into the extension
-        out = _mha_self_packed(xq, query.attention_schedule(), num_heads, head_dim, W, in_proj_bias,
+        out = _mha_self_packed(xq, _attention_work(query, None, num_heads, head_dim), num_heads, head_dim, W, in_proj_bias,
                                float(scaling), out_proj_weight, out_proj_bias)
         return query.with_buffer(out.reshape(-1))
     xk, xv = key.buffer.reshape(-1, E), value.buffer.reshape(-1, E)
@@ -418,7 +441,7 @@ def mha_packed(num_heads, head_dim, query, key, value, in_proj_weight, in_proj_b
         # head_dim 32 / 64 / 128: three projections (the value one written
         # transposed), then the same attention kernel with one key sequence per
         # query sequence: five launches issued by one call into the extension
-        out = _mha_cross_packed(xq, xk, xv, query.attention_schedule(kv=key), num_heads, head_dim, W,
+        out = _mha_cross_packed(xq, xk, xv, _attention_work(query, key, num_heads, head_dim), num_heads, head_dim, W,
                                 in_proj_bias, float(scaling), out_proj_weight, out_proj_bias)
         return query.with_buffer(out.reshape(-1))
     # V row-major: fp32 with head_dim 32 / 64 / 128 on the fp32 matrix instruction from
