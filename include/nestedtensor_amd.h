@@ -143,6 +143,14 @@ int64_t nt_pack_table_max_entries(void);
 int nt_pack_table(const int64_t* table_host, int64_t B, int64_t D, void* packed, int64_t* table_dev,
                   int elem_bytes, void* stream);
 
+/* A small table of host int64 (a nested size and its offsets, at most
+ * nt_pack_table_max_entries() entries) to device memory, carried by the kernel
+ * arguments of a one-workgroup launch: ordered on `stream` like any kernel, no
+ * staging buffer, no copy engine.  Replaces the metadata upload the reference
+ * does with Tensor::to(kCUDA, ..., non_blocking) before its padding kernels
+ * (nestedtensor/csrc/masking.cpp:471-472, 578-579). */
+int nt_upload_table(const int64_t* table_host, int64_t n, int64_t* table_dev, void* stream);
+
 /* ---- mask -> nested size, compaction ----------------------------------- */
 
 /* Row statistics of a byte mask viewed as [R, M] (nonzero = true):
@@ -153,6 +161,28 @@ int nt_pack_table(const int64_t* table_host, int64_t B, int64_t D, void* packed,
  * .item<bool>() on the host (nestedtensor/csrc/masking.cpp:190-201). */
 int nt_mask_row_counts(const uint8_t* mask, int64_t R, int64_t M, int32_t* counts,
                        uint8_t* prefix, void* stream);
+
+/* The nested size straight from the row statistics, when the mask is that of a
+ * padded tensor.  counts / prefix (device) are the statistics of B constituents
+ * of rows_per rows each, the rows of a constituent indexed row-major by the nd
+ * row dims `row_dims_host` (host int64, their product is rows_per; nd <=
+ * nt_leading_boxes_max_dims()).  boxes (device or device-visible host memory)
+ * receives max_dims + 2 int32 per constituent: {ok, w, extent[0 .. max_dims)}:
+ * ok = 1 iff every row keeps exactly its first w entries or nothing, and the rows
+ * that keep something are those whose index is below extent[k] in every row dim
+ * k; the constituent's size is then (extent[0 .. nd), w), as the reference's walk
+ * over the mask finds it (nestedtensor/csrc/masking.cpp:203-222).  ok = 0: the
+ * caller has to look at the statistics itself.
+ * done (may be NULL): a word in device-visible host memory that receives
+ * done_value, with system-wide release, once every line of boxes is written, so
+ * that a host thread polling it (acquire) can read boxes from host memory without
+ * a stream synchronisation.  arrivals (needed with done): a device word that is
+ * zero when the launch starts and is left zero; launches that share it must not
+ * overlap. */
+int64_t nt_leading_boxes_max_dims(void);
+int nt_leading_boxes(const int32_t* counts, const uint8_t* prefix, int64_t B, int64_t rows_per,
+                     const int64_t* row_dims_host, int64_t nd, int32_t* boxes, uint32_t* done,
+                     uint32_t done_value, uint32_t* arrivals, void* stream);
 
 /* The same statistics for the mask `data != padding` of a dense tensor viewed as
  * [R, M] elements of type elem_type, without materialising the mask; the

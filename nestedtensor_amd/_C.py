@@ -45,7 +45,11 @@ SIGNATURES = {
     "nt_pack": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _int, _c_void_p]),
     "nt_pack_table_max_entries": (_i64, []),
     "nt_pack_table": (_int, [_c_void_p, _i64, _i64, _c_void_p, _c_void_p, _int, _c_void_p]),
+    "nt_upload_table": (_int, [_c_void_p, _i64, _c_void_p, _c_void_p]),
     "nt_mask_row_counts": (_int, [_c_void_p, _i64, _i64, _c_void_p, _c_void_p, _c_void_p]),
+    "nt_leading_boxes_max_dims": (_i64, []),
+    "nt_leading_boxes": (_int, [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _i64, _c_void_p, _c_void_p, ctypes.c_uint32,
+                                _c_void_p, _c_void_p]),
     "nt_value_row_counts": (_int, [_c_void_p, _int, ctypes.c_double, _i64, _i64, _c_void_p, _c_void_p,
                                    _c_void_p]),
     "nt_compact_rows": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _c_void_p, _c_void_p]),

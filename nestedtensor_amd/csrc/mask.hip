@@ -15,6 +15,7 @@
 namespace nt {
 
 constexpr int kRowsPerBlock = 4;  // wavefronts per workgroup of the row kernels
+constexpr int kBoxMaxDims = 6;    // row dims of a constituent that leading_box_kernel walks
 
 // Predicates: a mask byte is kept if non-zero; a data element is kept if it
 // differs from the padding value with the comparison of its type (so NaN != x is
@@ -29,6 +30,36 @@ struct NotEqual {
   C pad;
   __device__ __forceinline__ bool operator()(T x) const { return (C)x != pad; }
 };
+
+// Bit j of the result: entry j of a lane's 16 bytes is kept.
+template <typename P, int VEC>
+__device__ __forceinline__ uint32_t lane_flags(const u32x4& raw, const P& pred) {
+  typename P::type v[VEC];
+  __builtin_memcpy(v, &raw, 16);
+  uint32_t flags = 0;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    if (pred(v[j])) flags |= 1u << j;
+  }
+  return flags;
+}
+// Sixteen mask bytes, four at a time in 32-bit arithmetic instead of sixteen
+// compares and selects: bit 7 of every byte of t says "byte is non-zero" (the add
+// carries into bit 7 exactly when one of the low seven bits is set), and the
+// multiplication gathers the four bits, shifted down to bits 0 / 8 / 16 / 24, into
+// bits 24..27 (the partial products land on ten different bit positions, so
+// nothing carries).
+template <>
+__device__ __forceinline__ uint32_t lane_flags<NonZeroByte, 16>(const u32x4& raw, const NonZeroByte&) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  uint32_t flags = 0;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const uint32_t t = (((w[k] & 0x7f7f7f7fu) + 0x7f7f7f7fu) | w[k]) & 0x80808080u;
+    flags |= (((t >> 7) * 0x01020408u) >> 24) << (4 * k);
+  }
+  return flags;
+}
 
 // counts[r] = kept entries of row r; prefix[r] = 1 iff the kept entries are
 // exactly the first counts[r] entries of the row.  A wavefront takes NR
@@ -68,17 +99,17 @@ __global__ __launch_bounds__(kWave * kRowsPerBlock) void row_counts_kernel(
     // element-wise tail) and drops the low VEC - exist flags: what is left are the
     // flags of entries i0 .. M - 1.  The vector path is only taken for M >= VEC.
     const int64_t ld = (VEC == 1 || here >= VEC) ? i0 : M - VEC;
-    T v[NR][VEC];
+    T v1[NR];         // VEC == 1
+    u32x4 raw[NR];    // otherwise
 #pragma unroll
     for (int r = 0; r < NR; ++r) {
       if (row0 + r >= R) continue;
       const T* m = data + (row0 + r) * M;
       if (VEC == 1) {
-        if (i0 < M) v[r][0] = m[i0];
+        if (i0 < M) v1[r] = m[i0];
       } else {
         // any alignment: the part runs in unaligned-access mode
-        u32x4 raw = load16_unaligned(reinterpret_cast<const char*>(m + ld));
-        __builtin_memcpy(v[r], &raw, 16);
+        raw[r] = load16_unaligned(reinterpret_cast<const char*>(m + ld));
       }
     }
     const uint64_t present = __ballot(exist > 0);
@@ -87,12 +118,9 @@ __global__ __launch_bounds__(kWave * kRowsPerBlock) void row_counts_kernel(
       if (row0 + r >= R) continue;
       uint32_t flags = 0;
       if (VEC == 1) {
-        if (exist > 0 && pred(v[r][0])) flags = 1u;
+        if (exist > 0 && pred(v1[r])) flags = 1u;
       } else {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          if (pred(v[r][j])) flags |= 1u << j;
-        }
+        flags = lane_flags<P, VEC>(raw[r], pred);
         flags = exist == VEC ? flags : (exist > 0 ? flags >> (VEC - exist) : 0u);
       }
       const int cnt = __popc(flags);
@@ -208,6 +236,75 @@ __global__ __launch_bounds__(kWave * kRowsPerBlock) void compact_rows_kernel(
   }
 }
 
+// Per constituent: do the row statistics describe a LEADING BOX (every row keeps
+// the same leading w entries or nothing, and the rows that keep something are the
+// rows whose index is below an extent in every row dim)?  That is what the mask
+// of a padded tensor looks like, and then the nested size is (extents, w) and
+// nothing else of the statistics has to leave the device.  One workgroup per
+// constituent: the extents are counted along the axes through the origin, then
+// every row is compared with what the box predicts.
+struct BoxDims {
+  int64_t d[kBoxMaxDims];
+};
+__global__ __launch_bounds__(256) void leading_box_kernel(const int32_t* __restrict__ counts,
+                                                          const uint8_t* __restrict__ prefix, int64_t rows_per,
+                                                          BoxDims dims, int nd, int32_t* __restrict__ out,
+                                                          uint32_t* done, uint32_t done_value, uint32_t* arrivals) {
+  __shared__ int s_ext[kBoxMaxDims];
+  __shared__ int s_bad;
+  const int64_t b = blockIdx.x;
+  const int32_t* c = counts + b * rows_per;
+  const uint8_t* pf = prefix + b * rows_per;
+  const int t = threadIdx.x;
+  if (t < kBoxMaxDims) s_ext[t] = 0;
+  if (t == 0) s_bad = 0;
+  __syncthreads();
+  const int32_t w = c[0];
+  int64_t stride = rows_per;
+  for (int k = 0; k < nd; ++k) {
+    stride /= dims.d[k];                 // rows per step along dim k
+    int n = 0;
+    for (int64_t j = t; j < dims.d[k]; j += 256) n += c[j * stride] != 0;
+    if (n) atomicAdd(&s_ext[k], n);
+  }
+  __syncthreads();
+  int bad = 0;
+  for (int64_t r = t; r < rows_per; r += 256) {
+    int64_t rest = r;
+    bool inside = true;
+    for (int k = nd - 1; k >= 0; --k) {
+      const int64_t i = rest % dims.d[k];
+      rest /= dims.d[k];
+      inside = inside && i < s_ext[k];
+    }
+    bad |= (c[r] != (inside ? w : 0)) | (pf[r] != 1);
+  }
+  if (bad) s_bad = 1;
+  __syncthreads();
+  if (t == 0) {
+    // an empty box is described as all zeros (the rows' extents along the axes are
+    // zero already when w is)
+    out[b * (kBoxMaxDims + 2)] = s_bad ? 0 : 1;
+    out[b * (kBoxMaxDims + 2) + 1] = w;
+  }
+  if (t < kBoxMaxDims) out[b * (kBoxMaxDims + 2) + 2 + t] = t < nd ? s_ext[t] : 1;
+  if (done == nullptr) return;
+  // The workgroup that arrives last tells the host (which polls `done`) that every
+  // constituent's line is written: each workgroup makes its line visible system-wide
+  // before it counts itself in, and the last one publishes after it has seen the
+  // others' arrivals.  The counter is left at zero for the next launch.
+  __threadfence_system();
+  __syncthreads();
+  if (t == 0) {
+    const uint32_t before = atomicAdd(arrivals, 1u);
+    if (before == gridDim.x - 1) {
+      atomicExch(arrivals, 0u);
+      __threadfence_system();
+      __hip_atomic_store(done, done_value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+  }
+}
+
 static int pick_unit(const void* a, const void* b, int64_t chunk_bytes) {
   uintptr_t x = (uintptr_t)a | (uintptr_t)b | (uintptr_t)chunk_bytes;
   if ((x & 15) == 0) return 16;
@@ -227,6 +324,33 @@ extern "C" int nt_mask_row_counts(const uint8_t* mask, int64_t R, int64_t M, int
   if (R == 0) return NT_OK;
   if (!counts || (M > 0 && !mask)) return fail(NT_ERR_INVALID_ARGUMENT, "mask_row_counts: NULL pointer");
   return launch_row_counts(mask, R, M, NonZeroByte(), counts, prefix, (hipStream_t)stream);
+}
+
+extern "C" int64_t nt_leading_boxes_max_dims(void) { return kBoxMaxDims; }
+
+extern "C" int nt_leading_boxes(const int32_t* counts, const uint8_t* prefix, int64_t B, int64_t rows_per,
+                                const int64_t* row_dims_host, int64_t nd, int32_t* boxes, uint32_t* done,
+                                uint32_t done_value, uint32_t* arrivals, void* stream) {
+  if (B < 0 || rows_per < 1 || nd < 0 || nd > kBoxMaxDims || (nd > 0 && !row_dims_host)) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "leading_boxes: bad shape (B=%lld rows=%lld dims=%lld)", (long long)B,
+                (long long)rows_per, (long long)nd);
+  }
+  if (B == 0) return NT_OK;
+  if (B > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "leading_boxes: too many constituents");
+  if (!counts || !prefix || !boxes || (done && !arrivals)) {
+    return fail(NT_ERR_INVALID_ARGUMENT, "leading_boxes: NULL pointer");
+  }
+  BoxDims dims;
+  int64_t prod = 1;
+  for (int64_t k = 0; k < kBoxMaxDims; ++k) {
+    dims.d[k] = k < nd ? row_dims_host[k] : 1;
+    if (dims.d[k] < 1 || dims.d[k] > 0x7fffffffLL) return fail(NT_ERR_INVALID_ARGUMENT, "leading_boxes: bad row dim");
+    prod *= dims.d[k];
+  }
+  if (prod != rows_per) return fail(NT_ERR_INVALID_ARGUMENT, "leading_boxes: row dims do not multiply to the rows");
+  hipLaunchKernelGGL(leading_box_kernel, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, counts, prefix,
+                     rows_per, dims, (int)nd, boxes, done, done_value, arrivals);
+  return check_launch("leading_box_kernel");
 }
 
 extern "C" int nt_value_row_counts(const void* data, int elem_type, double padding, int64_t R,

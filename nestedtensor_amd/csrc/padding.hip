@@ -897,9 +897,28 @@ __global__ __launch_bounds__(256) void pack_table_kernel(PackTable t, char* dst,
   const u32x4 zero = {0u, 0u, 0u, 0u};
   move_row<EB, kUnpad, 256>(dst + off * EB, reinterpret_cast<const char*>(t.v[B * D + B + 1 + row]), n, n, zero);
 }
+// The first n entries of a table that travelled in the kernel arguments, written
+// to device memory.
+__global__ __launch_bounds__(256) void table_store_kernel(PackTable t, int n, int64_t* out) {
+  for (int i = threadIdx.x; i < n; i += 256) out[i] = t.v[i];
+}
 }  // namespace nt
 
 extern "C" int64_t nt_pack_table_max_entries(void) { return nt::kPackTableMax; }
+
+extern "C" int nt_upload_table(const int64_t* table_host, int64_t n, int64_t* table_dev, void* stream) {
+  if (n == 0) return NT_OK;
+  if (n < 0 || !table_host || !table_dev) return fail(NT_ERR_INVALID_ARGUMENT, "bad upload_table args");
+  if (n > nt::kPackTableMax) {
+    return fail(NT_ERR_UNSUPPORTED, "table of %lld entries exceeds the %d that fit in kernel arguments",
+                (long long)n, nt::kPackTableMax);
+  }
+  nt::PackTable t;
+  for (int64_t i = 0; i < n; ++i) t.v[i] = table_host[i];
+  for (int64_t i = n; i < nt::kPackTableMax; ++i) t.v[i] = 0;
+  hipLaunchKernelGGL(nt::table_store_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, t, (int)n, table_dev);
+  return check_launch("table_store_kernel");
+}
 
 extern "C" int nt_pack_table(const int64_t* table_host, int64_t B, int64_t D, void* packed,
                              int64_t* table_dev, int elem_bytes, void* stream) {

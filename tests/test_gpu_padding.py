@@ -525,6 +525,119 @@ def test_mask_row_counts_and_prefix_flags(M):
         assert torch.equal(prefix.cpu(), exp_p), dtype
 
 
+@pytest.mark.parametrize("M", [16, 333, 1015, 4096])
+def test_mask_row_counts_take_any_nonzero_byte_as_true(M):
+    # a uint8 mask is true wherever it is non-zero (nested/masking.py:18-50 hands the
+    # mask to the kernels as it is): 0x80, 0x7f, 0x01 and 0xff bytes in every position
+    # of a lane's sixteen
+    g = torch.Generator().manual_seed(100 + M)
+    R = 64
+    values = torch.tensor([0, 0, 1, 2, 0x7f, 0x80, 0x81, 0xff], dtype=torch.uint8)
+    mask = values[torch.randint(0, values.numel(), (R, M), generator=g)]
+    for r in range(0, R, 4):                     # every fourth row: a prefix of odd bytes
+        n = int(torch.randint(0, M + 1, (1,), generator=g))
+        mask[r] = 0
+        mask[r, :n] = values[2 + torch.randint(0, 6, (n,), generator=g)]
+    exp_c, exp_p = _cpu_counts_prefix(mask != 0)
+    counts = torch.empty(R, dtype=torch.int32, device=DEV)
+    prefix = torch.empty(R, dtype=torch.uint8, device=DEV)
+    dmask = mask.to(DEV)
+    _C.check(_C.lib.nt_mask_row_counts(_C.ptr(dmask), R, M, _C.ptr(counts), _C.ptr(prefix), _C.current_stream(DEV)))
+    assert torch.equal(counts.cpu(), exp_c)
+    assert torch.equal(prefix.cpu(), exp_p)
+
+
+def _box_by_brute_force(c, pf, dims):
+    """(ok, w, extents) of one constituent's row statistics, every candidate box
+    tried: the definition nt_leading_boxes implements, not its algorithm."""
+    c = c.reshape(dims if dims else [1])
+    if not bool((pf == 1).all()):
+        return 0, int(c.flatten()[0]), None
+    w = int(c.flatten()[0])
+    if w == 0:
+        return (1 if int(c.abs().sum()) == 0 else 0), 0, [0] * len(dims)
+    import itertools
+    for ext in itertools.product(*[range(1, d + 1) for d in dims]):
+        box = torch.zeros_like(c)
+        box[tuple(slice(0, e) for e in ext)] = w
+        if torch.equal(box, c):
+            return 1, w, list(ext)
+    return 0, w, None
+
+
+@pytest.mark.parametrize("dims", [[], [5], [3, 4], [2, 3, 4], [300], [2, 260]])
+def test_leading_boxes_against_every_candidate_box(dims):
+    g = torch.Generator().manual_seed(len(dims) * 7 + sum(dims))
+    rows_per = 1
+    for d in dims:
+        rows_per *= d
+    cases = []
+    for trial in range(24):
+        w = int(torch.randint(1, 9, (1,), generator=g))
+        ext = [int(torch.randint(1, d + 1, (1,), generator=g)) for d in dims]
+        c = torch.zeros(dims if dims else [1], dtype=torch.int32)
+        c[tuple(slice(0, e) for e in ext)] = w
+        pf = torch.ones(rows_per, dtype=torch.uint8)
+        kind = trial % 6
+        if kind == 1:
+            c.zero_()                                              # an empty constituent
+        elif kind == 2 and rows_per > 1:
+            flat = c.flatten()
+            r = int(torch.randint(1, rows_per, (1,), generator=g))
+            flat[r] = w if int(flat[r]) == 0 else 0                # one row flipped
+            c = flat.reshape(c.shape)
+        elif kind == 3 and rows_per > 1:
+            flat = c.flatten()
+            flat[int(torch.randint(0, rows_per, (1,), generator=g))] += 1      # one row of another width
+            c = flat.reshape(c.shape)
+        elif kind == 4:
+            pf[int(torch.randint(0, rows_per, (1,), generator=g))] = 0        # a row that keeps no prefix
+        elif kind == 5 and dims:
+            c = c.flip(0)                                          # the box at the far end of the first dim
+        cases.append((c.flatten(), pf))
+    B = len(cases)
+    counts = torch.cat([c for c, _ in cases]).to(DEV)
+    prefix = torch.cat([p for _, p in cases]).to(DEV)
+    K = int(_C.lib.nt_leading_boxes_max_dims())
+    boxes = torch.full((B, K + 2), -7, dtype=torch.int32, device=DEV)
+    # the completion word lives in pinned host memory; the arrival counter on the device
+    done = torch.zeros(4, dtype=torch.int32).pin_memory()
+    arrivals = torch.zeros(1, dtype=torch.int32, device=DEV)
+    for value in (41, 42):                    # twice: the counter must be back at zero
+        boxes.fill_(-7)
+        _C.check(_C.lib.nt_leading_boxes(_C.ptr(counts), _C.ptr(prefix), B, rows_per, _C.i64_array(dims or [1]),
+                                         len(dims), _C.ptr(boxes), _C.ptr(done), value, _C.ptr(arrivals),
+                                         _C.current_stream(DEV)))
+        torch.cuda.synchronize()
+        assert int(done[0]) == value and int(arrivals.cpu()[0]) == 0
+    got = boxes.cpu()
+    n_ok = 0
+    for b, (c, pf) in enumerate(cases):
+        ok, w, ext = _box_by_brute_force(c, pf, dims)
+        assert int(got[b, 0]) == ok, (b, c, pf)
+        if ok:
+            n_ok += 1
+            assert int(got[b, 1]) == w
+            if w:
+                assert [int(v) for v in got[b, 2:2 + len(dims)]] == ext
+    assert 0 < n_ok < B or not dims
+
+
+def test_from_tensor_mask_falls_back_when_one_constituent_is_no_leading_box():
+    # two constituents keep a leading box, the third keeps a box that starts at
+    # column 1: same result as the reference's walk (masking.cpp:203-222)
+    g = torch.Generator().manual_seed(77)
+    t = torch.randn(3, 4, 6, generator=g)
+    m = torch.zeros(3, 4, 6, dtype=torch.bool)
+    m[0, :2, :3] = True
+    m[1, :4, :6] = True
+    m[2, :3, 1:5] = True
+    exp = oracle.nested_tensor_from_tensor_mask(t, m)
+    got = nt.nested_tensor_from_tensor_mask(t.to(DEV), m.to(DEV))
+    assert got.nested_size().unbind() == exp.nested_size()
+    bits_equal(got._impl.buffer, exp.buffer)
+
+
 def test_from_padded_value_comparison_semantics():
     # `tensor != padding` of torch: NaN is kept, -0.0 equals the padding 0.0
     t = torch.tensor([[1.0, float("nan"), 0.0, 0.0], [2.0, -0.0, 0.0, 0.0], [3.0, 4.0, 5.0, 6.0]])
