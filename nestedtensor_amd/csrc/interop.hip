@@ -407,6 +407,98 @@ __global__ __launch_bounds__(256) void transpose_ragged_kernel(
   }
 }
 
+// 64 x 64 tiles of 2-byte elements (fp16 / bf16 images) with 16-byte global accesses
+// on both sides.  The tile lies in LDS as dwords (two neighbouring columns each)
+// with an odd row stride: a lane of the transposed read takes one dword of eight
+// consecutive rows, which is conflict-free, and v_perm splits the eight dwords
+// into the 16-byte pieces of two output rows.  Where every output row of the
+// constituent is a whole number of 128-byte lines (rows % 64 == 0, e.g. NCHW ->
+// NHWC of 64 or 256 channels, where a tile's output is one contiguous block) the
+// stores are non-temporal: 4.9 -> 5.45 TB/s on 16 images [64, H, W].  Elsewhere a
+// tile writes 128-byte pieces that straddle lines, which only the L2 can merge
+// with the neighbouring tile's; non-temporal stores halve the rate there.
+__global__ __launch_bounds__(256) void transpose_u16_kernel(
+    const uint16_t* __restrict__ in, uint16_t* __restrict__ out, const int64_t* __restrict__ offsets,
+    const int64_t* __restrict__ rows, const int64_t* __restrict__ cols,
+    const int64_t* __restrict__ tile_offsets, int64_t B) {
+  constexpr int TR = 64, TC = 64, S = TC / 2 + 1;
+  __shared__ uint32_t tile[TR * S];
+  int64_t id = blockIdx.x;
+  {
+    const int64_t per_xcd = gridDim.x / 8;
+    if (id < per_xcd * 8) id = (id % 8) * per_xcd + id / 8;
+  }
+  const int64_t b = find_segment(tile_offsets, B, id);
+  const int64_t R = rows[b], C = cols[b];
+  const int64_t tiles_c = (C + TC - 1) / TC;
+  const int64_t local = id - tile_offsets[b];
+  const int64_t r0 = (local / tiles_c) * TR;
+  const int64_t c0 = (local % tiles_c) * TC;
+  const uint16_t* src = in + offsets[b];
+  uint16_t* dst = out + offsets[b];
+  {
+    const int k = threadIdx.x & 7;
+    const int lr = threadIdx.x >> 3;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+      const int r = lr + 32 * pass;
+      if (r0 + r < R) {
+        const uint16_t* p = src + (r0 + r) * C + c0 + 8 * k;
+        if (c0 + 8 * k + 8 <= C) {
+          const u32x4 bits = load16_unaligned(reinterpret_cast<const char*>(p));
+          uint32_t* t = &tile[r * S + 4 * k];
+          t[0] = bits.x;
+          t[1] = bits.y;
+          t[2] = bits.z;
+          t[3] = bits.w;
+        } else {
+          uint16_t* t16 = reinterpret_cast<uint16_t*>(&tile[r * S]) + 8 * k;
+          for (int j = 0; j < 8; ++j) t16[j] = c0 + 8 * k + j < C ? p[j] : (uint16_t)0;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // lane = (eight rows, one pair of columns)
+  const int lo = threadIdx.x & 7, cp = threadIdx.x >> 3;
+  uint32_t x[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) x[j] = tile[(8 * lo + j) * S + cp];
+  u32x4 even, odd;      // the pieces of output rows c and c + 1
+  even.x = __builtin_amdgcn_perm(x[1], x[0], 0x05040100u);
+  even.y = __builtin_amdgcn_perm(x[3], x[2], 0x05040100u);
+  even.z = __builtin_amdgcn_perm(x[5], x[4], 0x05040100u);
+  even.w = __builtin_amdgcn_perm(x[7], x[6], 0x05040100u);
+  odd.x = __builtin_amdgcn_perm(x[1], x[0], 0x07060302u);
+  odd.y = __builtin_amdgcn_perm(x[3], x[2], 0x07060302u);
+  odd.z = __builtin_amdgcn_perm(x[5], x[4], 0x07060302u);
+  odd.w = __builtin_amdgcn_perm(x[7], x[6], 0x07060302u);
+  const int64_t c = c0 + 2 * cp;
+  uint16_t* q = dst + c * R + r0 + 8 * lo;
+  if (r0 + 8 * lo + 8 <= R) {
+    // every piece is a whole aligned line when every output row starts on a line:
+    // rows of a multiple of 64 elements in a constituent that starts on one
+    const bool lines = (R & 63) == 0 && (reinterpret_cast<uintptr_t>(dst) & 127) == 0;
+    if (lines) {
+      if (c < C) __builtin_nontemporal_store(even, reinterpret_cast<u32x4*>(q));
+      if (c + 1 < C) __builtin_nontemporal_store(odd, reinterpret_cast<u32x4*>(q + R));
+    } else {
+      if (c < C) __builtin_memcpy(q, &even, 16);
+      if (c + 1 < C) __builtin_memcpy(q + R, &odd, 16);
+    }
+  } else {
+    uint16_t ve[8], vo[8];
+    __builtin_memcpy(ve, &even, 16);
+    __builtin_memcpy(vo, &odd, 16);
+    for (int j = 0; j < 8; ++j) {
+      if (r0 + 8 * lo + j < R) {
+        if (c < C) q[j] = ve[j];
+        if (c + 1 < C) q[R + j] = vo[j];
+      }
+    }
+  }
+}
+
 // Matrices with at most kTrNarrow rows (or columns): images of a few channels.  A
 // 64-wide tile would leave most of its lanes idle, so a workgroup takes a strip
 // of 256 * V columns (rows) of the long side instead, with V = 8 / sizeof(U), and
@@ -513,6 +605,12 @@ static int launch_transpose(const void* in, void* out, const int64_t* offsets, c
                          tile_offsets, B);
     }
     return check_launch("transpose_narrow_kernel");
+  }
+  if (sizeof(U) == 2 && tile_rows == 64 && tile_cols == 64) {
+    hipLaunchKernelGGL(transpose_u16_kernel, dim3((unsigned)total_tiles), dim3(256), 0, stream,
+                       static_cast<const uint16_t*>(in), static_cast<uint16_t*>(out), offsets, rows, cols,
+                       tile_offsets, B);
+    return check_launch("transpose_u16_kernel");
   }
   NT_TR_CASE(64, 64)
   NT_TR_CASE(64, 128)

@@ -25,7 +25,8 @@ from . import _C
 
 class NestedTensorImpl:
     __slots__ = ("buffer", "sizes", "_opt_sizes", "_sizes_dev", "_offsets_dev",
-                 "_row_offsets_dev", "_max_sizes", "_attn_schedule", "_attn_plan", "_last_dim_rows", "_has_empty", "channels_last")
+                 "_row_offsets_dev", "_max_sizes", "_attn_schedule", "_attn_plan", "_last_dim_rows", "_has_empty", "_transpose_meta",
+                 "channels_last")
 
     def __init__(self, buffer, sizes, channels_last=False):
         """buffer: 1-D contiguous tensor; sizes: CPU int64 [B, D], or 0-d for an
@@ -50,6 +51,7 @@ class NestedTensorImpl:
         self._attn_plan = None
         self._last_dim_rows = None
         self._has_empty = None
+        self._transpose_meta = None
 
     # ---- host metadata ----------------------------------------------------
     @property
@@ -219,6 +221,7 @@ class NestedTensorImpl:
             out._attn_schedule = self._attn_schedule
             out._attn_plan = self._attn_plan
             out._last_dim_rows = self._last_dim_rows
+            out._transpose_meta = self._transpose_meta
         return out
 
 

@@ -930,19 +930,27 @@ def _transpose_tile(max_rows, max_cols, elem_bytes):
     return 64, 64
 
 
-def _transpose_constituents(impl, rows, cols, new_sizes):
+def _transpose_constituents(impl, rows, cols, new_sizes, which):
     """Every constituent, seen as a row-major [rows[b], cols[b]] matrix, is
-    transposed in place of its slot of the packed buffer (nt_transpose_ragged)."""
+    transposed in place of its slot of the packed buffer (nt_transpose_ragged).
+    The device copy of (rows, cols, tile offsets) depends on the nested size and
+    the direction `which` only and is kept with the nested size."""
     buf = impl.buffer
     _C.require_device(buf, "transpose")
     B = impl.B
-    tr, tc = _transpose_tile(int(rows.max()) if B else 0, int(cols.max()) if B else 0, buf.element_size())
-    tiles = ((rows + tr - 1) // tr) * ((cols + tc - 1) // tc)
-    meta = torch.zeros((3, B + 1), dtype=torch.int64)
-    meta[0, :B], meta[1, :B] = rows, cols
-    meta[2, 1:] = torch.cumsum(tiles, 0)
-    total_tiles = int(meta[2, B])
-    meta_dev = meta.to(buf.device)
+    which = (which, buf.element_size())       # the tile shape depends on the element size
+    cached = impl._transpose_meta
+    if cached is not None and cached[0] == which and cached[1].device == buf.device:
+        _, meta_dev, total_tiles, tr, tc = cached
+    else:
+        tr, tc = _transpose_tile(int(rows.max()) if B else 0, int(cols.max()) if B else 0, buf.element_size())
+        tiles = ((rows + tr - 1) // tr) * ((cols + tc - 1) // tc)
+        meta = torch.zeros((3, B + 1), dtype=torch.int64)
+        meta[0, :B], meta[1, :B] = rows, cols
+        meta[2, 1:] = torch.cumsum(tiles, 0)
+        total_tiles = int(meta[2, B])
+        meta_dev = meta.to(buf.device)
+        impl._transpose_meta = (which, meta_dev, total_tiles, tr, tc)
     out = torch.empty_like(buf)
     if total_tiles:
         with _C.on_device(buf.device):
@@ -965,7 +973,7 @@ def transpose_nchw_nhwc(impl):
         raise RuntimeError("Expected first dimension to be regular.")
     s = impl.sizes
     return _transpose_constituents(impl, s[:, 0], s[:, 1] * s[:, 2],
-                                   torch.stack([s[:, 1], s[:, 2], s[:, 0]], 1).contiguous())
+                                   torch.stack([s[:, 1], s[:, 2], s[:, 0]], 1).contiguous(), "nchw_nhwc")
 
 
 def transpose_nhwc_nchw(impl):
@@ -978,7 +986,7 @@ def transpose_nhwc_nchw(impl):
         raise RuntimeError("Expected last dimension to be regular.")
     s = impl.sizes
     return _transpose_constituents(impl, s[:, 0] * s[:, 1], s[:, 2],
-                                   torch.stack([s[:, 2], s[:, 0], s[:, 1]], 1).contiguous())
+                                   torch.stack([s[:, 2], s[:, 0], s[:, 1]], 1).contiguous(), "nhwc_nchw")
 
 
 def is_contiguous(impl, memory_format=torch.contiguous_format):

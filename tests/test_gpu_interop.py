@@ -284,6 +284,26 @@ def test_transpose_ragged_every_tile_shape(dtype):
     assert rc != 0
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.int16])
+@pytest.mark.parametrize("first", [(64, 7, 9), (64, 1, 1)])
+def test_transpose_two_byte_elements_with_whole_line_rows(dtype, first):
+    """Two-byte elements take a kernel of their own, which stores whole cache lines
+    where every output row is a multiple of 64 elements in a constituent that starts
+    on a line (64 and 256 channels, NCHW -> NHWC) and ordinary pieces elsewhere: both
+    store paths in one batch, in both directions (transpose.cpp:122-204)."""
+    g = torch.Generator().manual_seed(31)
+    for ch in (64, 256, 192, 72):
+        shapes = [(ch,) + first[1:], (ch, 33, 65), (ch, 64, 64), (ch, 100, 3), (ch, 5, 129)]
+        ts = [torch.randint(-300, 300, s, generator=g).to(dtype) for s in shapes]
+        a = nt.nested_tensor(ts, device=DEV, dtype=dtype)
+        ref = oracle.ref_nested_tensor(ts, dtype=dtype)
+        a0 = nt.transpose_nchw_nhwc(a)
+        e0 = oracle.transpose_nchw_nhwc(ref)
+        assert torch.equal(a0._impl.buffer.cpu().view(torch.int16), e0.buffer.view(torch.int16)), ch
+        a2 = nt.transpose_nhwc_nchw(a0)
+        assert torch.equal(a2._impl.buffer.view(torch.int16), a._impl.buffer.view(torch.int16)), ch
+
+
 @pytest.mark.parametrize("dtype", [torch.uint8, torch.float16, torch.float32, torch.int64])
 @pytest.mark.parametrize("narrow", [1, 3, 4, 7, 16])
 def test_transpose_ragged_strips(dtype, narrow):
