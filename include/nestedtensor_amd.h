@@ -457,6 +457,27 @@ int nt_transpose_ragged(const void* in, void* out, const int64_t* offsets, const
                         int64_t total_tiles, int tile_rows, int tile_cols, int elem_bytes,
                         void* stream);
 
+/* Bias-free 1x1 convolution of B row-major images straight on the packed buffer:
+ * image b is x + pix_offsets[b] * c_in, a [c_in, P_b] matrix with the P_b = H_b W_b
+ * pixels contiguous, and the result y + pix_offsets[b] * c_out = weight[c_out,
+ * c_in] times it, [c_out, P_b].  pix_offsets (device int64 [B + 1]) are the
+ * cumulative pixel counts; tile_offsets (device int64 [B + 1]) the cumulative tile
+ * counts with ceil(P_b / t) + 1 tiles for image b, t = nt_conv1x1_tile_pixels()
+ * (a tile is one 128-byte line of every output row, and the rows' lines begin up
+ * to t - 1 pixels before a multiple of t); total_tiles their sum.  y must be
+ * 128-byte aligned.  f16 / bf16, fp32 accumulation; nt_conv1x1_supported() says
+ * whether a pair of depths is covered (c_in a multiple of 16 up to 128, c_out a
+ * multiple of 32 up to 512, and the weight plus two wavefronts' tiles must fit the
+ * 160 KiB of LDS), otherwise NT_ERR_UNSUPPORTED.  Replaces transpose_nchw_nhwc +
+ * matmul + transpose_nhwc_nchw of the reference's 1x1 path
+ * (nestedtensor/csrc/conv2d.cpp:33-75) by one launch that reads and writes every
+ * element once. */
+int nt_conv1x1_supported(int64_t c_in, int64_t c_out, int dtype);
+int64_t nt_conv1x1_tile_pixels(void);
+int nt_conv1x1_nchw(const void* x, const void* weight, void* y, const int64_t* pix_offsets,
+                    const int64_t* tile_offsets, int64_t B, int64_t total_tiles, int64_t c_in,
+                    int64_t c_out, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

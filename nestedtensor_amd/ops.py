@@ -685,6 +685,44 @@ def max_pool2d(impl, kernel_size, stride=None, padding=0, dilation=1, ceil_mode=
         ceil_mode=bool(ceil_mode))
 
 
+def _conv1x1_row_major(impl, w2d):
+    """The 1x1 convolution of row-major f16 / bf16 images as one launch on the packed
+    buffer (nt_conv1x1_nchw); None when the kernel does not cover the shape."""
+    buf = impl.buffer
+    c_out, c_in = w2d.shape
+    if impl.channels_last or buf.dtype not in (torch.float16, torch.bfloat16) or \
+            not _C.lib.nt_conv1x1_supported(c_in, c_out, _C.dtype_code(buf.dtype)):
+        return None
+    tn = int(_C.lib.nt_conv1x1_tile_pixels())
+    B = impl.B
+    if impl._transpose_meta is None:
+        impl._transpose_meta = {}
+    key = ("conv1x1", tn)
+    cached = impl._transpose_meta.get(key)
+    if cached is not None and cached[0].device == buf.device:
+        meta_dev, total_tiles = cached
+    else:
+        pix = impl.sizes[:, 1] * impl.sizes[:, 2]
+        meta = torch.zeros((2, B + 1), dtype=torch.int64)
+        meta[0, 1:] = torch.cumsum(pix, 0)
+        # a tile is one 128-byte line of every output row; the rows' lines start up to
+        # tn - 1 pixels before a multiple of tn, hence one tile more than ceil(P / tn)
+        meta[1, 1:] = torch.cumsum(torch.where(pix > 0, (pix + tn - 1) // tn + 1, pix), 0)
+        total_tiles = int(meta[1, B])
+        meta_dev = meta.to(buf.device)
+        impl._transpose_meta[key] = (meta_dev, total_tiles)
+    w2d = w2d.contiguous()
+    sizes = impl.sizes.clone()
+    sizes[:, 0] = c_out
+    out = torch.empty(int(sizes.prod(1).sum()), dtype=buf.dtype, device=buf.device)
+    if total_tiles:
+        with _C.on_device(buf.device):
+            _C.check(_C.lib.nt_conv1x1_nchw(_C.ptr(buf), _C.ptr(w2d), _C.ptr(out), _C.ptr(meta_dev[0]),
+                                            _C.ptr(meta_dev[1]), B, total_tiles, c_in, c_out,
+                                            _C.dtype_code(buf.dtype), _C.current_stream(buf.device)))
+    return NestedTensorImpl(out, sizes)
+
+
 def conv2d(impl, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
     """NestedTensor_conv2d, padded route (conv2d.cpp:77-92; the reference takes it
     for fp16).  Padding with 0 is exact: a convolution pads with zeros itself."""
@@ -705,6 +743,9 @@ def conv2d(impl, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
             sizes[:, 0] = c_out
             res = NestedTensorImpl(y.reshape(-1), sizes, channels_last=True)
             return res
+        y = _conv1x1_row_major(impl, weight.reshape(c_out, c_in))
+        if y is not None:
+            return y
         # NCHW -> NHWC on the packed buffer, [pixels, C_in] x W^T, and back (conv2d.cpp:61-73)
         nhwc = transpose_nchw_nhwc(impl)
         y = linear(nhwc.buffer.reshape(-1, c_in), weight.reshape(c_out, c_in), None)
@@ -939,9 +980,11 @@ def _transpose_constituents(impl, rows, cols, new_sizes, which):
     _C.require_device(buf, "transpose")
     B = impl.B
     which = (which, buf.element_size())       # the tile shape depends on the element size
-    cached = impl._transpose_meta
-    if cached is not None and cached[0] == which and cached[1].device == buf.device:
-        _, meta_dev, total_tiles, tr, tc = cached
+    if impl._transpose_meta is None:
+        impl._transpose_meta = {}
+    cached = impl._transpose_meta.get(which)
+    if cached is not None and cached[0].device == buf.device:
+        meta_dev, total_tiles, tr, tc = cached
     else:
         tr, tc = _transpose_tile(int(rows.max()) if B else 0, int(cols.max()) if B else 0, buf.element_size())
         tiles = ((rows + tr - 1) // tr) * ((cols + tc - 1) // tc)
@@ -950,7 +993,7 @@ def _transpose_constituents(impl, rows, cols, new_sizes, which):
         meta[2, 1:] = torch.cumsum(tiles, 0)
         total_tiles = int(meta[2, B])
         meta_dev = meta.to(buf.device)
-        impl._transpose_meta = (which, meta_dev, total_tiles, tr, tc)
+        impl._transpose_meta[which] = (meta_dev, total_tiles, tr, tc)
     out = torch.empty_like(buf)
     if total_tiles:
         with _C.on_device(buf.device):

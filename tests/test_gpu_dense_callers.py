@@ -105,3 +105,47 @@ def test_conv2d_1x1_runs_as_one_gemm(dtype):
         err = (got._impl.buffer.float().cpu() - ref.buffer).abs().max().item()
         scale = max(1.0, ref.buffer.abs().max().item())
         assert err <= (1e-5 if dtype == torch.float32 else 2e-2) * scale, err
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("c_in,c_out", [(16, 32), (64, 256), (64, 96), (128, 256), (32, 512), (48, 160), (128, 64)])
+def test_conv2d_1x1_row_major_in_one_launch(dtype, c_in, c_out, monkeypatch):
+    """Row-major f16 / bf16 images with depths the kernel covers take nt_conv1x1_nchw:
+    no transposes (conv2d.cpp:33-75 does two around its matmul), same numbers as the
+    per-constituent convolution.  Pixel counts around the 8-pixel pieces and the
+    64-pixel tiles, images of one pixel, and more tiles than workgroups."""
+    from nestedtensor_amd import ops
+
+    def boom(*a, **k):
+        raise AssertionError("this 1x1 convolution must not transpose")
+    monkeypatch.setattr(ops, "transpose_nchw_nhwc", boom)
+    shapes = [(c_in, 1, 1), (c_in, 1, 7), (c_in, 8, 8), (c_in, 5, 13), (c_in, 9, 7), (c_in, 16, 8), (c_in, 3, 43),
+              (c_in, 37, 50), (c_in, 250, 300)]
+    g = torch.Generator().manual_seed(c_in + c_out)
+    ts = [torch.randn(s, generator=g).to(dtype) for s in shapes]
+    w = (torch.randn(c_out, c_in, 1, 1, generator=g) * c_in ** -0.5).to(dtype)
+    a = nt.nested_tensor(ts, device=DEV, dtype=dtype)
+    got = torch.conv2d(a, w.to(DEV))
+    again = torch.conv2d(a, w.to(DEV))                       # the cached tile table
+    assert torch.equal(got._impl.buffer, again._impl.buffer)
+    ref = oracle.conv2d(oracle.ref_nested_tensor([t.float() for t in ts], dtype=torch.float32), w.float())
+    assert [tuple(x.shape) for x in got.unbind()] == [tuple(x.shape) for x in ref.unbind()]
+    assert torch.isfinite(got._impl.buffer).all()
+    err = (got._impl.buffer.float().cpu() - ref.buffer).abs().max().item()
+    scale = max(1.0, ref.buffer.abs().max().item())
+    assert err <= (1e-2 if dtype == torch.float16 else 4e-2) * scale, err
+    # exactly the packed GEMM's numbers: the channels-last route computes the same
+    # products in the same order of K
+    monkeypatch.undo()                                       # building a channels-last tensor transposes
+    cl = torch.conv2d(nt.nested_tensor(ts, device=DEV, dtype=dtype, channels_last=True), w.to(DEV))
+    diff = (cl.contiguous()._impl.buffer.float() - got._impl.buffer.float()).abs().max().item()
+    assert diff <= (4e-3 if dtype == torch.float16 else 3e-2) * scale, diff
+
+
+def test_conv2d_1x1_depths_outside_the_kernel_keep_the_transposes():
+    ts = [torch.randn(24, 9, 11).half(), torch.randn(24, 4, 4).half()]     # 24 input channels: not a multiple of 16
+    w = (torch.randn(40, 24, 1, 1) * 0.2).half()
+    a = nt.nested_tensor(ts, device=DEV, dtype=torch.float16)
+    got = torch.conv2d(a, w.to(DEV))
+    ref = oracle.conv2d(oracle.ref_nested_tensor([t.float() for t in ts], dtype=torch.float32), w.float())
+    assert (got._impl.buffer.float().cpu() - ref.buffer).abs().max().item() <= 2e-2 * max(1.0, ref.buffer.abs().max().item())
