@@ -457,6 +457,16 @@ int nt_transpose_ragged(const void* in, void* out, const int64_t* offsets, const
                         int64_t total_tiles, int tile_rows, int tile_cols, int elem_bytes,
                         void* stream);
 
+/* nt_transpose_ragged for 2-byte elements when the OUTPUT rows do not begin on
+ * 128-byte lines (NHWC -> NCHW of images whose H x W is no multiple of 64): every
+ * output row is written as whole lines from its own aligned window of the input
+ * rows.  Same operands; the tiles are counted differently: constituent b has
+ * (ceil(rows[b] / 64) + 1) * ceil(cols[b] / 64) tiles.  Same reference code
+ * (nestedtensor/csrc/transpose.cpp:183-204, cuda/transpose.cu). */
+int nt_transpose_ragged_lines(const void* in, void* out, const int64_t* offsets, const int64_t* rows,
+                              const int64_t* cols, const int64_t* tile_offsets, int64_t B,
+                              int64_t total_tiles, int elem_bytes, void* stream);
+
 /* Bias-free 1x1 convolution of B row-major images straight on the packed buffer:
  * image b is x + pix_offsets[b] * c_in, a [c_in, P_b] matrix with the P_b = H_b W_b
  * pixels contiguous, and the result y + pix_offsets[b] * c_out = weight[c_out,

@@ -86,6 +86,8 @@ SIGNATURES = {
     "nt_ragged_arange": (_int, [_c_void_p, _i64, _i64, _c_void_p, _c_void_p]),
     "nt_transpose_ragged": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64,
                                    _int, _int, _int, _c_void_p]),
+    "nt_transpose_ragged_lines": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64,
+                                         _int, _c_void_p]),
     "nt_conv1x1_tile_pixels": (_i64, []),
     "nt_conv1x1_supported": (_int, [_i64, _i64, _int]),
     "nt_conv1x1_nchw": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _int,

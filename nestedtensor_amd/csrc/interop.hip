@@ -499,6 +499,98 @@ __global__ __launch_bounds__(256) void transpose_u16_kernel(
   }
 }
 
+// The same transposition for output rows that do NOT begin on 128-byte lines
+// (NHWC -> NCHW of images whose H x W is no multiple of 64: output row c begins R
+// elements after row c - 1).  A 64-element piece of such a row covers two half
+// lines, and half lines are stored at about half the rate of whole ones (the L2
+// has to merge them with the neighbouring tile's).  So a tile here is not a
+// rectangle: tile k of a 64-column block is, for every output row c of the block,
+// the 64 elements of that row's k-th LINE.  The rows' lines begin up to 63 elements
+// before element 64 k, so the workgroup loads the 128 input rows [64 k - 64, 64 k +
+// 64) (each input row is read by two tiles; the second read hits the L2) and every
+// output row takes its own aligned window out of LDS.  Eight lanes write one
+// whole line, a store instruction eight of them; only a row's first and last
+// line are partial.  A constituent has (ceil(R / 64) + 1) * ceil(C / 64) tiles.
+__global__ __launch_bounds__(256) void transpose_u16_lines_kernel(
+    const uint16_t* __restrict__ in, uint16_t* __restrict__ out, const int64_t* __restrict__ offsets,
+    const int64_t* __restrict__ rows, const int64_t* __restrict__ cols,
+    const int64_t* __restrict__ tile_offsets, int64_t B) {
+  constexpr int S = 33;                       // dwords per LDS row: 64 columns and one of padding
+  __shared__ uint32_t tile[128 * S];
+  int64_t id = blockIdx.x;
+  {
+    const int64_t per_xcd = gridDim.x / 8;
+    if (id < per_xcd * 8) id = (id % 8) * per_xcd + id / 8;
+  }
+  const int64_t b = find_segment(tile_offsets, B, id);
+  const int64_t R = rows[b], C = cols[b];
+  const int64_t tiles_c = (C + 63) / 64;
+  const int64_t local = id - tile_offsets[b];
+  const int64_t k64 = (local / tiles_c) * 64;      // 64 k
+  const int64_t c0 = (local % tiles_c) * 64;
+  const uint16_t* src = in + offsets[b];
+  uint16_t* dst = out + offsets[b];
+  {
+    const int piece = threadIdx.x & 7, lr = threadIdx.x >> 3;
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+      const int r = lr + 32 * pass;
+      const int64_t row = k64 - 64 + r;            // input row, may lie outside [0, R)
+      u32x4 bits = {0u, 0u, 0u, 0u};
+      if (row >= 0 && row < R) {
+        const uint16_t* p = src + row * C + c0 + 8 * piece;
+        if (c0 + 8 * piece + 8 <= C) {
+          bits = load16_unaligned(reinterpret_cast<const char*>(p));
+        } else {
+          uint16_t e[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) e[j] = c0 + 8 * piece + j < C ? p[j] : (uint16_t)0;
+          __builtin_memcpy(&bits, e, 16);
+        }
+      }
+      uint32_t* t = &tile[r * S + 4 * piece];
+      t[0] = bits.x;
+      t[1] = bits.y;
+      t[2] = bits.z;
+      t[3] = bits.w;
+    }
+  }
+  __syncthreads();
+  // lane = (output row c of the block, 16-byte piece j of its line)
+  const int j = threadIdx.x & 7;
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int cl = (threadIdx.x >> 3) + 32 * pass;
+    const int64_t c = c0 + cl;
+    if (c >= C) continue;
+    const int64_t row_start = offsets[b] + c * R;          // element index of the output row in `out`
+    const int ph = (int)(((reinterpret_cast<uintptr_t>(out) >> 1) + (uint64_t)row_start) & 63);
+    const int first = 64 - ph + 8 * j;                     // first of this piece's eight rows of the tile
+    const uint32_t sel = (cl & 1) ? 0x07060302u : 0x05040100u;
+    const uint32_t* col = &tile[first * S + (cl >> 1)];
+    uint32_t x[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = col[i * S];
+    u32x4 v;
+    v.x = __builtin_amdgcn_perm(x[1], x[0], sel);
+    v.y = __builtin_amdgcn_perm(x[3], x[2], sel);
+    v.z = __builtin_amdgcn_perm(x[5], x[4], sel);
+    v.w = __builtin_amdgcn_perm(x[7], x[6], sel);
+    const int64_t r = k64 - ph + 8 * j;                    // first output element of the piece in its row
+    uint16_t* q = out + row_start + r;
+    if (r >= 0 && r + 8 <= R) {
+      __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(q));       // 16-byte aligned by construction
+    } else if (r + 8 > 0 && r < R) {
+      uint16_t e[8];
+      __builtin_memcpy(e, &v, 16);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (r + i >= 0 && r + i < R) q[i] = e[i];
+    }
+  }
+  (void)dst;
+}
+
 // Matrices with at most kTrNarrow rows (or columns): images of a few channels.  A
 // 64-wide tile would leave most of its lanes idle, so a workgroup takes a strip
 // of 256 * V columns (rows) of the long side instead, with V = 8 / sizeof(U), and
@@ -626,6 +718,22 @@ static int launch_transpose(const void* in, void* out, const int64_t* offsets, c
 }
 
 }  // namespace nt
+
+extern "C" int nt_transpose_ragged_lines(const void* in, void* out, const int64_t* offsets, const int64_t* rows,
+                                         const int64_t* cols, const int64_t* tile_offsets, int64_t B,
+                                         int64_t total_tiles, int elem_bytes, void* stream) {
+  if (B < 0 || total_tiles < 0) return nt::fail(NT_ERR_INVALID_ARGUMENT, "transpose_ragged_lines: negative extent");
+  if (elem_bytes != 2) return nt::fail(NT_ERR_UNSUPPORTED, "transpose_ragged_lines: 2-byte elements only");
+  if (B == 0 || total_tiles == 0) return NT_OK;
+  if (!in || !out || !offsets || !rows || !cols || !tile_offsets) {
+    return nt::fail(NT_ERR_INVALID_ARGUMENT, "transpose_ragged_lines: NULL pointer");
+  }
+  if (total_tiles > 0x7fffffffLL) return nt::fail(NT_ERR_UNSUPPORTED, "transpose_ragged_lines: too many tiles");
+  hipLaunchKernelGGL(nt::transpose_u16_lines_kernel, dim3((unsigned)total_tiles), dim3(256), 0, (hipStream_t)stream,
+                     static_cast<const uint16_t*>(in), static_cast<uint16_t*>(out), offsets, rows, cols,
+                     tile_offsets, B);
+  return nt::check_launch("transpose_u16_lines_kernel");
+}
 
 extern "C" int nt_transpose_ragged(const void* in, void* out, const int64_t* offsets,
                                    const int64_t* rows, const int64_t* cols,

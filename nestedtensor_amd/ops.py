@@ -987,7 +987,14 @@ def _transpose_constituents(impl, rows, cols, new_sizes, which):
         meta_dev, total_tiles, tr, tc = cached
     else:
         tr, tc = _transpose_tile(int(rows.max()) if B else 0, int(cols.max()) if B else 0, buf.element_size())
-        tiles = ((rows + tr - 1) // tr) * ((cols + tc - 1) // tc)
+        if (tr, tc) == (64, 64) and buf.element_size() == 2 and bool((rows % 64 != 0).any()):
+            # output rows that do not begin on 128-byte lines: the kernel that gives every
+            # output row its own line-aligned window (tile shape recorded as 0 x 0)
+            tr = tc = 0
+            tiles = torch.where((rows > 0) & (cols > 0), ((rows + 63) // 64 + 1) * ((cols + 63) // 64),
+                                torch.zeros_like(rows))
+        else:
+            tiles = ((rows + tr - 1) // tr) * ((cols + tc - 1) // tc)
         meta = torch.zeros((3, B + 1), dtype=torch.int64)
         meta[0, :B], meta[1, :B] = rows, cols
         meta[2, 1:] = torch.cumsum(tiles, 0)
@@ -997,10 +1004,16 @@ def _transpose_constituents(impl, rows, cols, new_sizes, which):
     out = torch.empty_like(buf)
     if total_tiles:
         with _C.on_device(buf.device):
-            _C.check(_C.lib.nt_transpose_ragged(
-                _C.ptr(buf), _C.ptr(out), _C.ptr(impl.offsets_dev()), _C.ptr(meta_dev[0]),
-                _C.ptr(meta_dev[1]), _C.ptr(meta_dev[2]), B, total_tiles, tr, tc, buf.element_size(),
-                _C.current_stream(buf.device)))
+            if tr == 0:
+                _C.check(_C.lib.nt_transpose_ragged_lines(
+                    _C.ptr(buf), _C.ptr(out), _C.ptr(impl.offsets_dev()), _C.ptr(meta_dev[0]),
+                    _C.ptr(meta_dev[1]), _C.ptr(meta_dev[2]), B, total_tiles, buf.element_size(),
+                    _C.current_stream(buf.device)))
+            else:
+                _C.check(_C.lib.nt_transpose_ragged(
+                    _C.ptr(buf), _C.ptr(out), _C.ptr(impl.offsets_dev()), _C.ptr(meta_dev[0]),
+                    _C.ptr(meta_dev[1]), _C.ptr(meta_dev[2]), B, total_tiles, tr, tc, buf.element_size(),
+                    _C.current_stream(buf.device)))
     res = NestedTensorImpl(out, new_sizes)
     res._offsets_dev = impl._offsets_dev      # the constituents keep their extents
     return res

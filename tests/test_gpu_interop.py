@@ -304,6 +304,42 @@ def test_transpose_two_byte_elements_with_whole_line_rows(dtype, first):
         assert torch.equal(a2._impl.buffer.view(torch.int16), a._impl.buffer.view(torch.int16)), ch
 
 
+@pytest.mark.parametrize("shift", [0, 1, 37])
+def test_transpose_ragged_lines_through_the_c_abi(shift):
+    """nt_transpose_ragged_lines (every output row written as whole 128-byte lines
+    from its own window) on matrices whose extents are multiples of nothing, one
+    with a single row and one with a single column, with the output buffer starting
+    `shift` elements into an allocation so that the lines' phase moves."""
+    from nestedtensor_amd import _C
+    from nestedtensor_amd.impl import device_offsets
+    shapes = [(1, 300), (300, 1), (64, 257), (130, 67), (255, 129), (7, 5), (1000, 64), (513, 100)]
+    g = torch.Generator().manual_seed(23)
+    mats = [torch.randint(-300, 300, s, generator=g).to(torch.int16) for s in shapes]
+    buf = torch.cat([m.reshape(-1) for m in mats]).to(DEV)
+    exp = torch.cat([m.t().contiguous().reshape(-1) for m in mats])
+    B = len(shapes)
+    rows = torch.tensor([s[0] for s in shapes], dtype=torch.int64)
+    cols = torch.tensor([s[1] for s in shapes], dtype=torch.int64)
+    offsets = device_offsets(torch.stack([rows, cols], 1).contiguous().to(DEV), B, 2)
+    tiles = ((rows + 63) // 64 + 1) * ((cols + 63) // 64)
+    toff = torch.zeros(B + 1, dtype=torch.int64)
+    toff[1:] = torch.cumsum(tiles, 0)
+    store = torch.full((buf.numel() + shift + 64,), 777, dtype=torch.int16, device=DEV)
+    out = store[shift:shift + buf.numel()]
+    rows_d, cols_d, toff_d = rows.to(DEV), cols.to(DEV), toff.to(DEV)      # alive until the kernels have run
+    rc = _C.lib.nt_transpose_ragged_lines(_C.ptr(buf), _C.ptr(out), _C.ptr(offsets), _C.ptr(rows_d),
+                                          _C.ptr(cols_d), _C.ptr(toff_d), B, int(toff[B]), 2,
+                                          _C.current_stream(DEV))
+    assert rc == 0, _C.lib.nt_last_error()
+    assert torch.equal(out.cpu(), exp)
+    # nothing outside the output was touched
+    assert bool((store[:shift] == 777).all()) and bool((store[shift + buf.numel():] == 777).all())
+    rc = _C.lib.nt_transpose_ragged_lines(_C.ptr(buf), _C.ptr(out), _C.ptr(offsets), _C.ptr(rows_d),
+                                          _C.ptr(cols_d), _C.ptr(toff_d), B, int(toff[B]), 4,
+                                          _C.current_stream(DEV))
+    assert rc != 0 and b"2-byte" in _C.lib.nt_last_error()
+
+
 @pytest.mark.parametrize("dtype", [torch.uint8, torch.float16, torch.float32, torch.int64])
 @pytest.mark.parametrize("narrow", [1, 3, 4, 7, 16])
 def test_transpose_ragged_strips(dtype, narrow):
