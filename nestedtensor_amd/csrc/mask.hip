@@ -246,10 +246,12 @@ __global__ __launch_bounds__(kWave * kRowsPerBlock) void compact_rows_kernel(
 struct BoxDims {
   int64_t d[kBoxMaxDims];
 };
-__global__ __launch_bounds__(256) void leading_box_kernel(const int32_t* __restrict__ counts,
-                                                          const uint8_t* __restrict__ prefix, int64_t rows_per,
-                                                          BoxDims dims, int nd, int32_t* __restrict__ out,
-                                                          uint32_t* done, uint32_t done_value, uint32_t* arrivals) {
+constexpr int kBoxThreads = 1024;
+__global__ __launch_bounds__(kBoxThreads) void leading_box_kernel(const int32_t* __restrict__ counts,
+                                                                  const uint8_t* __restrict__ prefix,
+                                                                  int64_t rows_per, BoxDims dims, int nd,
+                                                                  int32_t* __restrict__ out, uint32_t* done,
+                                                                  uint32_t done_value, uint32_t* arrivals) {
   __shared__ int s_ext[kBoxMaxDims];
   __shared__ int s_bad;
   const int64_t b = blockIdx.x;
@@ -260,22 +262,37 @@ __global__ __launch_bounds__(256) void leading_box_kernel(const int32_t* __restr
   if (t == 0) s_bad = 0;
   __syncthreads();
   const int32_t w = c[0];
-  int64_t stride = rows_per;
-  for (int k = 0; k < nd; ++k) {
-    stride /= dims.d[k];                 // rows per step along dim k
-    int n = 0;
-    for (int64_t j = t; j < dims.d[k]; j += 256) n += c[j * stride] != 0;
-    if (n) atomicAdd(&s_ext[k], n);
+  // 32-bit index arithmetic (the host bounds rows_per): a 64-bit division per row and
+  // dim made this kernel as long as the row counts themselves
+  const int n_rows = (int)rows_per;
+  int d[kBoxMaxDims];
+#pragma unroll
+  for (int k = 0; k < kBoxMaxDims; ++k) d[k] = (int)dims.d[k];
+  int stride = n_rows;
+#pragma unroll
+  for (int k = 0; k < kBoxMaxDims; ++k) {
+    if (k < nd) {
+      stride /= d[k];                 // rows per step along dim k
+      int n = 0;
+      for (int j = t; j < d[k]; j += kBoxThreads) n += c[(int64_t)j * stride] != 0;
+      if (n) atomicAdd(&s_ext[k], n);
+    }
   }
   __syncthreads();
+  int ext[kBoxMaxDims];
+#pragma unroll
+  for (int k = 0; k < kBoxMaxDims; ++k) ext[k] = s_ext[k];
   int bad = 0;
-  for (int64_t r = t; r < rows_per; r += 256) {
-    int64_t rest = r;
+  for (int r = t; r < n_rows; r += kBoxThreads) {
+    int rest = r;
     bool inside = true;
-    for (int k = nd - 1; k >= 0; --k) {
-      const int64_t i = rest % dims.d[k];
-      rest /= dims.d[k];
-      inside = inside && i < s_ext[k];
+#pragma unroll
+    for (int k = kBoxMaxDims - 1; k >= 0; --k) {
+      if (k < nd) {
+        const int q = rest / d[k];
+        inside = inside && (rest - q * d[k]) < ext[k];
+        rest = q;
+      }
     }
     bad |= (c[r] != (inside ? w : 0)) | (pf[r] != 1);
   }
@@ -336,7 +353,9 @@ extern "C" int nt_leading_boxes(const int32_t* counts, const uint8_t* prefix, in
                 (long long)rows_per, (long long)nd);
   }
   if (B == 0) return NT_OK;
-  if (B > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "leading_boxes: too many constituents");
+  if (B > 0x7fffffffLL || rows_per > 0x7fffffffLL) {
+    return fail(NT_ERR_UNSUPPORTED, "leading_boxes: too many constituents or rows");
+  }
   if (!counts || !prefix || !boxes || (done && !arrivals)) {
     return fail(NT_ERR_INVALID_ARGUMENT, "leading_boxes: NULL pointer");
   }
@@ -348,7 +367,7 @@ extern "C" int nt_leading_boxes(const int32_t* counts, const uint8_t* prefix, in
     prod *= dims.d[k];
   }
   if (prod != rows_per) return fail(NT_ERR_INVALID_ARGUMENT, "leading_boxes: row dims do not multiply to the rows");
-  hipLaunchKernelGGL(leading_box_kernel, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, counts, prefix,
+  hipLaunchKernelGGL(leading_box_kernel, dim3((unsigned)B), dim3(kBoxThreads), 0, (hipStream_t)stream, counts, prefix,
                      rows_per, dims, (int)nd, boxes, done, done_value, arrivals);
   return check_launch("leading_box_kernel");
 }
