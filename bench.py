@@ -417,7 +417,15 @@ def instruction_rates():
                                   ctypes.POINTER(ctypes.c_int)]
     names = ["v_fma_f32", "v_exp_f32", "v_exp_f16", "v_cvt_pk_f16_f32", "v_dot2_f32_f16", "v_max3_f32 (2 x v_max)",
              "v_mfma_f32_32x32x16_f16", "ds_read_b128", "16 mfma + 128 fma (per iteration)",
-             "16 mfma + 32 exp (per iteration)", "16 mfma + 128 fma + 32 exp (per iteration)"]
+             "16 mfma + 32 exp (per iteration)", "16 mfma + 128 fma + 32 exp (per iteration)",
+             "v_mfma_f32_32x32x16_f16, accumulators in VGPRs",
+             "16 mfma + 128 fma + 32 exp (per iteration), accumulators in VGPRs",
+             "attention key tile: 8 mfma -> max, 32 exp, pack, sum -> 8 mfma (per tile)",
+             "the same with the 16 operand fragments read from LDS (per tile)",
+             "the same, and 4 LDS stores and a workgroup barrier per tile",
+             "the same, the stored data loaded from global memory during the tile",
+             "the same, LDS tiles as rows of 144 bytes read 16 bytes per lane and row",
+             "the same, the exponentials behind a wavefront-uniform test of the tile maximum"]
     iters = 2000
     res = {}
     for kind, name in enumerate(names):
@@ -432,6 +440,22 @@ def instruction_rates():
             row["%d_waves_per_simd" % waves] = round(ms.value * 1e6 / (iters * per.value * waves), 3)
         res[name] = row
     res["unit"] = "ns per instruction (mixed rows: per iteration) and SIMD"
+    # the full tile stream on regular operands and on operands with random signs and
+    # mantissas: same instructions, different switching activity, and the shader clock
+    # the chip held meanwhile (shader-clock counter against the constant 100 MHz one)
+    lib.nt_probe_tile_clock.restype = ctypes.c_int
+    lib.nt_probe_tile_clock.argtypes = [ctypes.c_uint, ctypes.c_int, ctypes.c_int] + [ctypes.POINTER(ctypes.c_float)] * 3
+    clock_iters = 20000   # ~30 ms per launch: long enough for the power management to settle
+    tile = {}
+    for tag, noise in (("regular_operands", 0), ("random_operands", 12345), ("regular_operands_again", 0)):
+        ms, cyc, ticks = ctypes.c_float(), ctypes.c_float(), ctypes.c_float()
+        rc = lib.nt_probe_tile_clock(noise, 3, clock_iters, ctypes.byref(ms), ctypes.byref(cyc), ctypes.byref(ticks))
+        if rc != 0:
+            tile[tag] = "probe failed (%d)" % rc
+            continue
+        tile[tag] = dict(ns_per_tile_and_simd=round(ms.value * 1e6 / (clock_iters * 3), 1),
+                         shader_cycles_per_100mhz_tick=round(cyc.value / max(ticks.value, 1.0), 3))
+    res["attention key tile, 3 wavefronts per SIMD, by operand data"] = tile
     return res
 
 

@@ -15,11 +15,16 @@
 // banks; any other K takes a register-staged loop with padded LDS rows and
 // element-wise tails.
 //
-// Three tile shapes are compiled (256x128, 256x192, 256x256, eight wavefronts
-// each); the launcher picks per problem the one with the least rounds x tile
-// cost over the CUs.  The bigger tiles read less LDS per MFMA and win once the
-// grid is several rounds deep; the smaller ones quantise better on the
-// projection shapes of one attention layer.
+// Three tile shapes are compiled for problems that fill the chip (256x128,
+// 256x192, 256x256, eight wavefronts each); the launcher picks per problem the
+// one with the least rounds x tile cost over the CUs.  The bigger tiles read less
+// LDS per MFMA and win once the grid is several rounds deep; the smaller ones
+// quantise better on the projection shapes of one attention layer.  A problem
+// with fewer 256x128 tiles than half the CUs (the query and output projections
+// of cross-attention, a few thousand rows) takes 128x64 tiles of four
+// wavefronts, or 128x128 when those would not fit in one round: its duration is
+// one tile's life, and a quarter of a tile on four times as many CUs ends sooner
+// (3200 x 512 x 512: 10.6 -> 6.3 us).
 //
 // Epilogues:
 //   plain  - C row-major + bias;
@@ -584,6 +589,8 @@ static int launch_cfg(const GemmArgs<T>& a, hipStream_t stream) {
 typedef GemmCfg<4, 2, 2, 2, 128> Cfg128;   // 256 x 128
 typedef GemmCfg<4, 2, 2, 3, 128> Cfg192;   // 256 x 192
 typedef GemmCfg<4, 2, 2, 4, 128> Cfg256;   // 256 x 256
+typedef GemmCfg<2, 2, 2, 1, 128> CfgSmall; // 128 x 64, four wavefronts: problems of fewer 256-row tiles than CUs
+typedef GemmCfg<2, 2, 2, 2, 128> CfgMid;   // 128 x 128, four wavefronts
 
 // Tile shape with the least estimated time.  A tile costs its area divided by the
 // measured steady-state rate of its shape relative to 256x128 (wider wavefront
@@ -622,6 +629,11 @@ static int pick_cfg(int64_t M, int64_t N, int64_t n_split, int* which) {
     return fail(NT_ERR_UNSUPPORTED, "linear: QKV split %lld is not a multiple of a column tile",
                 (long long)n_split);
   }
+  // Fewer 256 x 128 tiles than half the CUs: the launch is one tile's life on a
+  // fraction of the chip, and a quarter-size tile on four times as many CUs is shorter.
+  if (n_split == 0 && ((M + 255) / 256) * ((N + 127) / 128) * 2 <= num_cus) {
+    best = ((M + 127) / 128) * ((N + 63) / 64) <= num_cus ? 3 : 4;
+  }
   *which = best;
   return NT_OK;
 }
@@ -639,6 +651,10 @@ static int launch_epi(const GemmArgs<T>& a, hipStream_t stream) {
   } else {
     const int rc = pick_cfg(a.M, a.N, EPI == kEpiQkv ? a.n_split : 0, &which);
     if (rc != NT_OK) return rc;
+    if constexpr (EPI != kEpiQkv) {
+      if (which == 3) return launch_cfg<T, CfgSmall, EPI>(a, stream);
+      if (which == 4) return launch_cfg<T, CfgMid, EPI>(a, stream);
+    }
     if (which == 1) return launch_cfg<T, Cfg192, EPI>(a, stream);
     if (which == 2) return launch_cfg<T, Cfg256, EPI>(a, stream);
     return launch_cfg<T, Cfg128, EPI>(a, stream);

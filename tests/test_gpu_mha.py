@@ -383,15 +383,19 @@ def test_linear_packed_fast_path():
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K", [
-    (300, 200, 64),        # one round: 256 x 128 tiles, whole K tiles
+    (300, 200, 64),        # far fewer 256-row tiles than CUs: 128 x 64 tiles, whole K tiles
     (300, 200, 72),        # K tail: element-wise loads
+    (1000, 500, 200),      # 128 x 64 tiles, ragged in every dimension
+    (3200, 768, 128),      # more 128 x 64 tiles than CUs: 128 x 128 tiles
+    (3210, 760, 104),
+    (8200, 1000, 64),      # one partly filled round of 256 x 128 tiles
     (9813, 2304, 64),      # two rounds of 256 x 192 tiles beat three of 256 x 128
     (9813, 2304, 40),
     (4096, 4096, 64),      # one round of 256 x 256 tiles
     (4100, 4090, 24),
 ])
 def test_linear_tile_shapes(M, N, K, dtype):
-    # the launcher picks one of three tile shapes per problem; every shape, with
+    # the launcher picks one of five tile shapes per problem; every shape, with
     # and without a K tail, against an fp32 reference of the same product
     from nestedtensor_amd import ops
     g = torch.Generator().manual_seed(M + N + K)
