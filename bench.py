@@ -383,6 +383,21 @@ def mha_probe(args, torch, dev):
                                   us_planned=round(_event_us(torch, planned), 2)))
             out["attention_length_sweep"] = sweep
     out["instruction_rates"] = instruction_rates()
+    # the vendor's GEMM at a size that fills the chip, on operands that do not toggle
+    # and on N(0, 1) operands: how far the matrix rate of this part depends on the data
+    by_data = {}
+    n_big = 8192
+    for tag in ("zeros", "normal", "zeros_again"):
+        if tag == "normal":
+            a = torch.randn(n_big, n_big, device=dev).half()
+            b = torch.randn(n_big, n_big, device=dev).half()
+        else:
+            a = torch.zeros(n_big, n_big, device=dev, dtype=torch.float16)
+            b = torch.zeros(n_big, n_big, device=dev, dtype=torch.float16)
+        us = _event_us(torch, lambda: torch.mm(a, b), iters=20, warmup=5)
+        by_data[tag] = dict(us=round(us, 1), TFLOPs=round(2 * n_big ** 3 / us / 1e6, 1))
+        del a, b
+    out["vendor_gemm_8192_fp16_by_operand_data"] = by_data
     print(json.dumps(out))
 
 

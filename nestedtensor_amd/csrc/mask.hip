@@ -35,7 +35,7 @@ struct NotEqual {
 template <typename P, int VEC>
 __device__ __forceinline__ uint32_t lane_flags(const u32x4& raw, const P& pred) {
   typename P::type v[VEC];
-  __builtin_memcpy(v, &raw, 16);
+  __builtin_memcpy(v, &raw, sizeof(v));   // 16 bytes wherever the vector path is taken
   uint32_t flags = 0;
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
