@@ -127,7 +127,10 @@ def test_softmax_last_dim(dtype, log):
     # a regular last dim, 1-D constituents, rows longer than a wavefront, a single element
     import torch.nn.functional as F
     cases = [[(4, 5, 5), (4, 130, 130), (4, 1, 1)], [(3, 40), (7, 40)], [(9,), (300,), (1,)],
-             [(2, 1100), (3, 513)], [(2, 3, 1023), (2, 3, 1025)], [(2, 511), (1, 4097), (1, 9001)]]   # around the register-cached row limits
+             [(2, 1100), (3, 513)], [(2, 3, 1023), (2, 3, 1025)], [(2, 511), (1, 4097), (1, 9001)],   # around the register-cached row limits
+             # a wavefront takes four consecutive rows: groups that straddle constituents of other
+             # row lengths, with a constituent without rows between them, and a ragged last group
+             [(3, 5), (0, 5), (2, 9), (5, 1024), (1, 1025), (6, 2)], [(1, 7)] * 9 + [(2, 33)]]
     for k, shapes in enumerate(cases):
         ts = [t * 3 for t in _tensors(shapes, dtype, 20 + k)]
         a = nt.nested_tensor(ts, device=DEV, dtype=dtype)
