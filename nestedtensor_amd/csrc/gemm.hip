@@ -24,7 +24,8 @@
 // of cross-attention, a few thousand rows) takes 128x64 tiles of four
 // wavefronts, or 128x128 when those would not fit in one round: its duration is
 // one tile's life, and a quarter of a tile on four times as many CUs ends sooner
-// (3200 x 512 x 512: 10.6 -> 6.3 us).
+// (3200 x 512 x 512: 10.6 -> 6.3 us; the fused in-projection of a layer of a few
+// hundred tokens: 16.0 -> 11.6 us).
 //
 // Epilogues:
 //   plain  - C row-major + bias;
@@ -631,8 +632,10 @@ static int pick_cfg(int64_t M, int64_t N, int64_t n_split, int* which) {
   }
   // Fewer 256 x 128 tiles than half the CUs: the launch is one tile's life on a
   // fraction of the chip, and a quarter-size tile on four times as many CUs is shorter.
-  if (n_split == 0 && ((M + 255) / 256) * ((N + 127) / 128) * 2 <= num_cus) {
-    best = ((M + 127) / 128) * ((N + 63) / 64) <= num_cus ? 3 : 4;
+  if (((M + 255) / 256) * ((N + 127) / 128) * 2 <= num_cus) {
+    const int small = ((M + 127) / 128) * ((N + 63) / 64) <= num_cus ? 3 : 4;
+    const int64_t small_bn = small == 3 ? CfgSmall::kBN : CfgMid::kBN;
+    if (n_split % small_bn == 0) best = small;   // (a tile must not straddle the K | V boundary)
   }
   *which = best;
   return NT_OK;
@@ -651,10 +654,8 @@ static int launch_epi(const GemmArgs<T>& a, hipStream_t stream) {
   } else {
     const int rc = pick_cfg(a.M, a.N, EPI == kEpiQkv ? a.n_split : 0, &which);
     if (rc != NT_OK) return rc;
-    if constexpr (EPI != kEpiQkv) {
-      if (which == 3) return launch_cfg<T, CfgSmall, EPI>(a, stream);
-      if (which == 4) return launch_cfg<T, CfgMid, EPI>(a, stream);
-    }
+    if (which == 3) return launch_cfg<T, CfgSmall, EPI>(a, stream);
+    if (which == 4) return launch_cfg<T, CfgMid, EPI>(a, stream);
     if (which == 1) return launch_cfg<T, Cfg192, EPI>(a, stream);
     if (which == 2) return launch_cfg<T, Cfg256, EPI>(a, stream);
     return launch_cfg<T, Cfg128, EPI>(a, stream);

@@ -410,9 +410,10 @@ def test_linear_tile_shapes(M, N, K, dtype):
 
 def test_linear_qkv_tile_shapes():
     # fused in-projection: Q | K row-major, V transposed, on the shape that takes
-    # the 256 x 192 tiles (2E = 1536 is a multiple of 192) and on a small one
+    # the 256 x 192 tiles (2E = 1536 is a multiple of 192) and on small ones (128 x 64
+    # tiles; 128 x 128 where those would be more than the CUs)
     from nestedtensor_amd import _C
-    for (T, E) in ((9813, 768), (70, 64)):
+    for (T, E) in ((9813, 768), (70, 64), (471, 768), (645, 1024)):
         g = torch.Generator().manual_seed(T)
         x = torch.randn(T, E, generator=g).half()
         w = (torch.randn(3 * E, E, generator=g) * 0.05).half()
