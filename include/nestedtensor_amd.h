@@ -176,9 +176,11 @@ int nt_mask_row_counts(const uint8_t* mask, int64_t R, int64_t M, int32_t* count
  * done (may be NULL): a word in device-visible host memory that receives
  * done_value, with system-wide release, once every line of boxes is written, so
  * that a host thread polling it (acquire) can read boxes from host memory without
- * a stream synchronisation.  arrivals (needed with done): a device word that is
- * zero when the launch starts and is left zero; launches that share it must not
- * overlap. */
+ * a stream synchronisation.  arrivals: a device word that is zero when the launch
+ * starts and is left zero; launches that share it must not overlap.  With done
+ * and WITHOUT arrivals (NULL), done is an array of B words and word b receives
+ * done_value as soon as line b is written (nothing is counted, nobody waits for
+ * the last line: the host polls the B words). */
 int64_t nt_leading_boxes_max_dims(void);
 int nt_leading_boxes(const int32_t* counts, const uint8_t* prefix, int64_t B, int64_t rows_per,
                      const int64_t* row_dims_host, int64_t nd, int32_t* boxes, uint32_t* done,

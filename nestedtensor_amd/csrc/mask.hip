@@ -308,6 +308,14 @@ __global__ __launch_bounds__(kBoxThreads) void leading_box_kernel(const int32_t*
   }
   if (t < kBoxMaxDims) out[b * (kBoxMaxDims + 2) + 2 + t] = t < nd ? s_ext[t] : 1;
   if (done == nullptr) return;
+  if (arrivals == nullptr) {
+    // one completion word per constituent: every workgroup publishes its own line
+    // (visible system-wide before the word) and nobody waits for anybody
+    __threadfence_system();
+    __syncthreads();
+    if (t == 0) __hip_atomic_store(done + b, done_value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    return;
+  }
   // The workgroup that arrives last tells the host (which polls `done`) that every
   // constituent's line is written: each workgroup makes its line visible system-wide
   // before it counts itself in, and the last one publishes after it has seen the
@@ -358,9 +366,7 @@ extern "C" int nt_leading_boxes(const int32_t* counts, const uint8_t* prefix, in
   if (B > 0x7fffffffLL || rows_per > 0x7fffffffLL) {
     return fail(NT_ERR_UNSUPPORTED, "leading_boxes: too many constituents or rows");
   }
-  if (!counts || !prefix || !boxes || (done && !arrivals)) {
-    return fail(NT_ERR_INVALID_ARGUMENT, "leading_boxes: NULL pointer");
-  }
+  if (!counts || !prefix || !boxes) return fail(NT_ERR_INVALID_ARGUMENT, "leading_boxes: NULL pointer");
   BoxDims dims;
   int64_t prod = 1;
   for (int64_t k = 0; k < kBoxMaxDims; ++k) {

@@ -395,21 +395,27 @@ void wait_for_stream(hipStream_t stream) {
 // staging buffer rules out already).
 struct BoxSignal {
   uint32_t* done;
-  uint32_t* arrivals;
+  uint32_t* arrivals;   // nullptr: one completion word per constituent (`words` of them)
   uint32_t value;
+  int64_t words;
 };
-BoxSignal box_signal(const c10::Device& device) {
+constexpr int64_t kBoxWordsMax = 64;   // constituents up to which every one has a completion word of its own
+BoxSignal box_signal(const c10::Device& device, int64_t B) {
   static thread_local Tensor flag_t;
   static thread_local std::vector<Tensor> arrivals;
   static thread_local uint32_t seq = 0;
-  if (!flag_t.defined()) flag_t = at::zeros({16}, at::TensorOptions().dtype(at::kInt).pinned_memory(true));
+  if (!flag_t.defined()) flag_t = at::zeros({kBoxWordsMax}, at::TensorOptions().dtype(at::kInt).pinned_memory(true));
+  // Few constituents: a word each, written by the workgroup that finishes the
+  // constituent's line; the arrival counter, the last workgroup's second fence and
+  // its store (three serial round trips at the end of the launch) are not needed.
+  if (B <= kBoxWordsMax) return {reinterpret_cast<uint32_t*>(flag_t.data_ptr()), nullptr, ++seq, B};
   const size_t idx = static_cast<size_t>(device.index());
   if (arrivals.size() <= idx) arrivals.resize(idx + 1);
   if (!arrivals[idx].defined()) {
     arrivals[idx] = at::zeros({16}, at::TensorOptions().dtype(at::kInt).device(device));
     C10_HIP_CHECK(hipStreamSynchronize(c10::hip::getCurrentHIPStream(device.index()).stream()));
   }
-  return {reinterpret_cast<uint32_t*>(flag_t.data_ptr()), reinterpret_cast<uint32_t*>(arrivals[idx].data_ptr()), ++seq};
+  return {reinterpret_cast<uint32_t*>(flag_t.data_ptr()), reinterpret_cast<uint32_t*>(arrivals[idx].data_ptr()), ++seq, 1};
 }
 
 // Polls the completion word for at most 200 microseconds (acquire: the lines the
@@ -418,7 +424,9 @@ BoxSignal box_signal(const c10::Device& device) {
 void wait_for_signal(const BoxSignal& sig, hipStream_t stream) {
   const auto t0 = std::chrono::steady_clock::now();
   for (int spin = 0;; ++spin) {
-    if (__atomic_load_n(sig.done, __ATOMIC_ACQUIRE) == sig.value) return;
+    int64_t seen = 0;
+    while (seen < sig.words && __atomic_load_n(sig.done + seen, __ATOMIC_ACQUIRE) == sig.value) ++seen;
+    if (seen == sig.words) return;
     __builtin_ia32_pause();
     if ((spin & 255) == 255 && std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(200)) break;
   }
@@ -573,7 +581,7 @@ Lowered from_rows(const Tensor& tensor, int64_t mask_dims, CountRows count_rows,
     uint8_t* prefix_dev = static_cast<uint8_t*>(stats_dev.data_ptr()) + 4 * R;
     count_rows(R, M, counts_dev, prefix_dev);
     int32_t* boxes = reinterpret_cast<int32_t*>(stage.data_ptr());
-    const BoxSignal sig = box_signal(tensor.device());
+    const BoxSignal sig = box_signal(tensor.device(), B);
     check(nt_leading_boxes(counts_dev, prefix_dev, B, rows_per, shape.data() + 1, levels - 1, boxes, sig.done, sig.value,
                            sig.arrivals, stream));
     wait_for_signal(sig, stream);

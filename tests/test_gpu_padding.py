@@ -611,6 +611,13 @@ def test_leading_boxes_against_every_candidate_box(dims):
         torch.cuda.synchronize()
         assert int(done[0]) == value and int(arrivals.cpu()[0]) == 0
     got = boxes.cpu()
+    # without an arrival counter: a completion word per constituent, same lines
+    words = torch.zeros(B, dtype=torch.int32).pin_memory()
+    boxes.fill_(-7)
+    _C.check(_C.lib.nt_leading_boxes(_C.ptr(counts), _C.ptr(prefix), B, rows_per, _C.i64_array(dims or [1]),
+                                     len(dims), _C.ptr(boxes), _C.ptr(words), 43, None, _C.current_stream(DEV)))
+    torch.cuda.synchronize()
+    assert bool((words == 43).all()) and torch.equal(boxes.cpu(), got)
     n_ok = 0
     for b, (c, pf) in enumerate(cases):
         ok, w, ext = _box_by_brute_force(c, pf, dims)
