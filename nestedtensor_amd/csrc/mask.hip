@@ -64,8 +64,8 @@ __device__ __forceinline__ uint32_t lane_flags<NonZeroByte, 16>(const u32x4& raw
 // counts[r] = kept entries of row r; prefix[r] = 1 iff the kept entries are
 // exactly the first counts[r] entries of the row.  A wavefront takes NR
 // consecutive rows and walks them together, so that NR loads per lane are in
-// flight at a time (one row per wavefront left the memory system mostly idle: a
-// 16-byte load, then a long chain of ballots and shuffles); a lane looks at VEC
+// flight at a time (NR = 4 for many rows of under 384 bytes, where one row per
+// wavefront leaves the memory system idle; otherwise 1); a lane looks at VEC
 // consecutive entries per step (16 bytes; one entry for short rows); ballots over
 // the lanes' "full / non-empty / is a prefix" flags decide prefix-ness without
 // any serial scan.  The results of a workgroup's 4 * NR rows leave through LDS as
@@ -164,9 +164,12 @@ static int launch_row_counts(const void* data, int64_t R, int64_t M, P pred, int
   // very short rows: one entry per lane keeps more lanes busy than 16 bytes per lane
   // (measured on 400 000 mask rows: 250 bytes 167 -> 64 us with 16-byte loads, 100
   // bytes 88 -> 61 us, 64 bytes 48 -> 57 us);
-  // few rows: one row per wavefront spreads them over more CUs
   const bool vec = M * (int64_t)sizeof(T) >= 96;
-  const int nr = R >= 8192 ? 4 : 1;
+  // many short rows: four per wavefront, all of their loads in flight (400 000 rows
+  // of 250 bytes: 64 against 72 us).  From a few hundred bytes per row one row per
+  // wavefront is faster, the more the longer the rows: more wavefronts, each a short
+  // chain (48 384 x 1015 bytes: 11.6 against 13.8 us; 8192 x 4096: 6.5 against 10.5).
+  const int nr = (R >= 8192 && M * (int64_t)sizeof(T) < 384) ? 4 : 1;
   const int64_t blocks = (R + kRowsPerBlock * nr - 1) / (kRowsPerBlock * nr);
   if (blocks > 0x7fffffffLL) return fail(NT_ERR_UNSUPPORTED, "row_counts: too many rows");
   dim3 grid((unsigned)blocks), block(kWave * kRowsPerBlock);
