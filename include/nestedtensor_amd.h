@@ -186,6 +186,17 @@ int nt_leading_boxes(const int32_t* counts, const uint8_t* prefix, int64_t B, in
                      const int64_t* row_dims_host, int64_t nd, int32_t* boxes, uint32_t* done,
                      uint32_t done_value, uint32_t* arrivals, void* stream);
 
+/* nt_leading_boxes for a host that polls: lines (device-visible host memory, 8-byte
+ * aligned) receives max_dims + 2 uint64 per constituent, entry i of a line =
+ * (uint32) entry i of nt_leading_boxes' line in the low half and `stamp` (not 0)
+ * in the high half, each written with one 8-byte store.  An entry is valid for the
+ * host the moment its high half reads `stamp` (use a stamp the buffer has not held
+ * before, e.g. a call counter); no fence and no completion word are involved, so
+ * the launch ends without a round trip to host memory. */
+int nt_leading_boxes_stamped(const int32_t* counts, const uint8_t* prefix, int64_t B, int64_t rows_per,
+                             const int64_t* row_dims_host, int64_t nd, uint64_t* lines, uint32_t stamp,
+                             void* stream);
+
 /* The same statistics for the mask `data != padding` of a dense tensor viewed as
  * [R, M] elements of type elem_type, without materialising the mask; the
  * comparison is the one of the element type (NaN != x is true, -0.0 != 0.0 is

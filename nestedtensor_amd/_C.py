@@ -50,6 +50,8 @@ SIGNATURES = {
     "nt_leading_boxes_max_dims": (_i64, []),
     "nt_leading_boxes": (_int, [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _i64, _c_void_p, _c_void_p, ctypes.c_uint32,
                                 _c_void_p, _c_void_p]),
+    "nt_leading_boxes_stamped": (_int, [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _i64, _c_void_p, ctypes.c_uint32,
+                                        _c_void_p]),
     "nt_value_row_counts": (_int, [_c_void_p, _int, ctypes.c_double, _i64, _i64, _c_void_p, _c_void_p,
                                    _c_void_p]),
     "nt_compact_rows": (_int, [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _c_void_p, _c_void_p]),

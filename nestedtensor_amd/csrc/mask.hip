@@ -256,7 +256,8 @@ __global__ __launch_bounds__(kBoxThreads) void leading_box_kernel(const int32_t*
                                                                   const uint8_t* __restrict__ prefix,
                                                                   int64_t rows_per, BoxDims dims, int nd,
                                                                   int32_t* __restrict__ out, uint32_t* done,
-                                                                  uint32_t done_value, uint32_t* arrivals) {
+                                                                  uint32_t done_value, uint32_t* arrivals,
+                                                                  uint32_t stamp) {
   __shared__ int s_ext[kBoxMaxDims];
   __shared__ int s_bad;
   const int64_t b = blockIdx.x;
@@ -303,6 +304,20 @@ __global__ __launch_bounds__(kBoxThreads) void leading_box_kernel(const int32_t*
   }
   if (bad) s_bad = 1;
   __syncthreads();
+  if (stamp != 0) {
+    // Every entry of the line travels with the call's stamp in the upper half of
+    // one 8-byte word (a single store, atomic for whoever reads it): the host takes
+    // an entry as soon as it carries the stamp, in any order, and the launch needs
+    // no fence and no completion word, i.e. no round trip to host memory before it
+    // can end.
+    if (t < kBoxMaxDims + 2) {
+      const int32_t v = t == 0 ? (s_bad ? 0 : 1) : (t == 1 ? w : (t - 2 < nd ? s_ext[t - 2] : 1));
+      const uint64_t word = (uint64_t)(uint32_t)v | ((uint64_t)stamp << 32);
+      __hip_atomic_store(reinterpret_cast<uint64_t*>(out) + b * (kBoxMaxDims + 2) + t, word, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+    return;
+  }
   if (t == 0) {
     // an empty box is described as all zeros (the rows' extents along the axes are
     // zero already when w is)
@@ -358,9 +373,9 @@ extern "C" int nt_mask_row_counts(const uint8_t* mask, int64_t R, int64_t M, int
 
 extern "C" int64_t nt_leading_boxes_max_dims(void) { return kBoxMaxDims; }
 
-extern "C" int nt_leading_boxes(const int32_t* counts, const uint8_t* prefix, int64_t B, int64_t rows_per,
-                                const int64_t* row_dims_host, int64_t nd, int32_t* boxes, uint32_t* done,
-                                uint32_t done_value, uint32_t* arrivals, void* stream) {
+static int leading_boxes(const int32_t* counts, const uint8_t* prefix, int64_t B, int64_t rows_per,
+                         const int64_t* row_dims_host, int64_t nd, int32_t* boxes, uint32_t* done,
+                         uint32_t done_value, uint32_t* arrivals, uint32_t stamp, void* stream) {
   if (B < 0 || rows_per < 1 || nd < 0 || nd > kBoxMaxDims || (nd > 0 && !row_dims_host)) {
     return fail(NT_ERR_INVALID_ARGUMENT, "leading_boxes: bad shape (B=%lld rows=%lld dims=%lld)", (long long)B,
                 (long long)rows_per, (long long)nd);
@@ -379,8 +394,23 @@ extern "C" int nt_leading_boxes(const int32_t* counts, const uint8_t* prefix, in
   }
   if (prod != rows_per) return fail(NT_ERR_INVALID_ARGUMENT, "leading_boxes: row dims do not multiply to the rows");
   hipLaunchKernelGGL(leading_box_kernel, dim3((unsigned)B), dim3(kBoxThreads), 0, (hipStream_t)stream, counts, prefix,
-                     rows_per, dims, (int)nd, boxes, done, done_value, arrivals);
+                     rows_per, dims, (int)nd, boxes, done, done_value, arrivals, stamp);
   return check_launch("leading_box_kernel");
+}
+
+extern "C" int nt_leading_boxes(const int32_t* counts, const uint8_t* prefix, int64_t B, int64_t rows_per,
+                                const int64_t* row_dims_host, int64_t nd, int32_t* boxes, uint32_t* done,
+                                uint32_t done_value, uint32_t* arrivals, void* stream) {
+  return leading_boxes(counts, prefix, B, rows_per, row_dims_host, nd, boxes, done, done_value, arrivals, 0, stream);
+}
+
+extern "C" int nt_leading_boxes_stamped(const int32_t* counts, const uint8_t* prefix, int64_t B, int64_t rows_per,
+                                        const int64_t* row_dims_host, int64_t nd, uint64_t* lines, uint32_t stamp,
+                                        void* stream) {
+  if (stamp == 0) return fail(NT_ERR_INVALID_ARGUMENT, "leading_boxes_stamped: the stamp must not be 0");
+  if ((uintptr_t)lines % 8 != 0) return fail(NT_ERR_INVALID_ARGUMENT, "leading_boxes_stamped: lines must be 8-byte aligned");
+  return leading_boxes(counts, prefix, B, rows_per, row_dims_host, nd, reinterpret_cast<int32_t*>(lines), nullptr, 0,
+                       nullptr, stamp, stream);
 }
 
 extern "C" int nt_value_row_counts(const void* data, int elem_type, double padding, int64_t R,

@@ -399,16 +399,19 @@ struct BoxSignal {
   uint32_t value;
   int64_t words;
 };
-constexpr int64_t kBoxWordsMax = 64;   // constituents up to which every one has a completion word of its own
+constexpr int64_t kBoxWordsMax = 64;       // completion words in the pinned block
+constexpr int64_t kBoxStampedMax = 1024;   // constituents up to which the host polls stamped lines
 BoxSignal box_signal(const c10::Device& device, int64_t B) {
   static thread_local Tensor flag_t;
   static thread_local std::vector<Tensor> arrivals;
   static thread_local uint32_t seq = 0;
   if (!flag_t.defined()) flag_t = at::zeros({kBoxWordsMax}, at::TensorOptions().dtype(at::kInt).pinned_memory(true));
-  // Few constituents: a word each, written by the workgroup that finishes the
-  // constituent's line; the arrival counter, the last workgroup's second fence and
-  // its store (three serial round trips at the end of the launch) are not needed.
-  if (B <= kBoxWordsMax) return {reinterpret_cast<uint32_t*>(flag_t.data_ptr()), nullptr, ++seq, B};
+  // Up to kBoxStampedMax constituents the lines carry the call's stamp themselves
+  // (nt_leading_boxes_stamped): no completion word, no counter (stamp 0 is never used).
+  if (B <= kBoxStampedMax) {
+    if (++seq == 0) ++seq;
+    return {nullptr, nullptr, seq, 0};
+  }
   const size_t idx = static_cast<size_t>(device.index());
   if (arrivals.size() <= idx) arrivals.resize(idx + 1);
   if (!arrivals[idx].defined()) {
@@ -572,7 +575,7 @@ Lowered from_rows(const Tensor& tensor, int64_t mask_dims, CountRows count_rows,
   bool boxes_ok = false;
   Tensor stats_dev;
   const bool try_boxes = R > 0 && rows_per > 0 && levels - 1 <= kBoxDims;
-  Tensor& stage = pinned_staging(std::max<int64_t>(5 * R, try_boxes ? 4 * box_ints * B : 0) + 16);
+  Tensor& stage = pinned_staging(std::max<int64_t>(5 * R, try_boxes ? 8 * box_ints * B : 0) + 16);
   int32_t* counts = reinterpret_cast<int32_t*>(stage.data_ptr());
   uint8_t* prefix = static_cast<uint8_t*>(stage.data_ptr()) + 4 * R;
   if (try_boxes) {
@@ -582,9 +585,41 @@ Lowered from_rows(const Tensor& tensor, int64_t mask_dims, CountRows count_rows,
     count_rows(R, M, counts_dev, prefix_dev);
     int32_t* boxes = reinterpret_cast<int32_t*>(stage.data_ptr());
     const BoxSignal sig = box_signal(tensor.device(), B);
-    check(nt_leading_boxes(counts_dev, prefix_dev, B, rows_per, shape.data() + 1, levels - 1, boxes, sig.done, sig.value,
-                           sig.arrivals, stream));
-    wait_for_signal(sig, stream);
+    std::vector<int32_t> unstamped;
+    if (sig.done == nullptr) {
+      // every entry arrives as {value, stamp} in one 8-byte word; poll until all carry
+      // this call's stamp (bounded: then the stream is synchronised, after which they do)
+      uint64_t* lines = reinterpret_cast<uint64_t*>(stage.data_ptr());
+      check(nt_leading_boxes_stamped(counts_dev, prefix_dev, B, rows_per, shape.data() + 1, levels - 1, lines, sig.value,
+                                     stream));
+      const int64_t n_words = B * box_ints;
+      const auto t0 = std::chrono::steady_clock::now();
+      int64_t seen = 0;
+      for (int spin = 0; seen < n_words; ++spin) {
+        while (seen < n_words &&
+               static_cast<uint32_t>(__atomic_load_n(lines + seen, __ATOMIC_ACQUIRE) >> 32) == sig.value) {
+          ++seen;
+        }
+        if (seen == n_words) break;
+        __builtin_ia32_pause();
+        if ((spin & 255) == 255 && std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(200)) {
+          C10_HIP_CHECK(hipStreamSynchronize(stream));
+          break;
+        }
+      }
+      unstamped.resize(static_cast<size_t>(n_words));
+      for (int64_t i = 0; i < n_words; ++i) {
+        const uint64_t word = __atomic_load_n(lines + i, __ATOMIC_ACQUIRE);
+        TORCH_CHECK(static_cast<uint32_t>(word >> 32) == sig.value,
+                    "nested_tensor_from_tensor_mask: the device did not deliver the nested size");
+        unstamped[static_cast<size_t>(i)] = static_cast<int32_t>(static_cast<uint32_t>(word));
+      }
+      boxes = unstamped.data();
+    } else {
+      check(nt_leading_boxes(counts_dev, prefix_dev, B, rows_per, shape.data() + 1, levels - 1, boxes, sig.done, sig.value,
+                             sig.arrivals, stream));
+      wait_for_signal(sig, stream);
+    }
     boxes_ok = true;
     for (int64_t b = 0; b < B && boxes_ok; ++b) boxes_ok = boxes[b * box_ints] == 1;
     if (boxes_ok) {

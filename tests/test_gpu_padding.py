@@ -618,6 +618,13 @@ def test_leading_boxes_against_every_candidate_box(dims):
                                      len(dims), _C.ptr(boxes), _C.ptr(words), 43, None, _C.current_stream(DEV)))
     torch.cuda.synchronize()
     assert bool((words == 43).all()) and torch.equal(boxes.cpu(), got)
+    # stamped lines: every entry {value, stamp} in one 8-byte word, nothing else to wait for
+    lines = torch.zeros(B, K + 2, dtype=torch.int64).pin_memory()
+    _C.check(_C.lib.nt_leading_boxes_stamped(_C.ptr(counts), _C.ptr(prefix), B, rows_per, _C.i64_array(dims or [1]),
+                                             len(dims), _C.ptr(lines), 44, _C.current_stream(DEV)))
+    torch.cuda.synchronize()
+    assert bool(((lines >> 32) == 44).all())
+    assert torch.equal((lines & 0xffffffff).to(torch.int32), got)
     n_ok = 0
     for b, (c, pf) in enumerate(cases):
         ok, w, ext = _box_by_brute_force(c, pf, dims)
