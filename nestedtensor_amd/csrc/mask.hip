@@ -246,8 +246,9 @@ __global__ __launch_bounds__(kWave * kRowsPerBlock) void compact_rows_kernel(
 // rows whose index is below an extent in every row dim)?  That is what the mask
 // of a padded tensor looks like, and then the nested size is (extents, w) and
 // nothing else of the statistics has to leave the device.  One workgroup per
-// constituent: the extents are counted along the axes through the origin, then
-// every row is compared with what the box predicts.
+// constituent, one pass over its rows (the kernel is a chain of memory round
+// trips; counting the extents along the axes first and comparing every row with
+// the box in a second pass were three of them).
 struct BoxDims {
   int64_t d[kBoxMaxDims];
 };
@@ -260,50 +261,91 @@ __global__ __launch_bounds__(kBoxThreads) void leading_box_kernel(const int32_t*
                                                                   uint32_t stamp) {
   __shared__ int s_ext[kBoxMaxDims];
   __shared__ int s_bad;
+  __shared__ unsigned s_kept, s_max_w, s_inv_min_w;
   const int64_t b = blockIdx.x;
   const int32_t* c = counts + b * rows_per;
   const uint8_t* pf = prefix + b * rows_per;
   const int t = threadIdx.x;
   if (t < kBoxMaxDims) s_ext[t] = 0;
-  if (t == 0) s_bad = 0;
+  if (t == 0) {
+    s_bad = 0;
+    s_kept = 0;
+    s_max_w = 0;
+    s_inv_min_w = 0;
+  }
   __syncthreads();
-  const int32_t w = c[0];
+  // One pass over the rows (one memory round trip): the constituent keeps a leading
+  // box iff no row fails the prefix test, every row that keeps anything keeps the
+  // same number, and those rows are as many as their bounding box from the origin
+  // holds (they all lie inside it, so then they fill it).
   // 32-bit index arithmetic (the host bounds rows_per): a 64-bit division per row and
   // dim made this kernel as long as the row counts themselves
   const int n_rows = (int)rows_per;
   int d[kBoxMaxDims];
 #pragma unroll
   for (int k = 0; k < kBoxMaxDims; ++k) d[k] = (int)dims.d[k];
-  int stride = n_rows;
+  int bad = 0, top[kBoxMaxDims];
+  unsigned kept = 0, max_w = 0, inv_min_w = 0;
 #pragma unroll
-  for (int k = 0; k < kBoxMaxDims; ++k) {
-    if (k < nd) {
-      stride /= d[k];                 // rows per step along dim k
-      int n = 0;
-      for (int j = t; j < d[k]; j += kBoxThreads) n += c[(int64_t)j * stride] != 0;
-      if (n) atomicAdd(&s_ext[k], n);
-    }
-  }
-  __syncthreads();
-  int ext[kBoxMaxDims];
-#pragma unroll
-  for (int k = 0; k < kBoxMaxDims; ++k) ext[k] = s_ext[k];
-  int bad = 0;
+  for (int k = 0; k < kBoxMaxDims; ++k) top[k] = 0;
   for (int r = t; r < n_rows; r += kBoxThreads) {
+    const int32_t count = c[r];
+    bad |= pf[r] != 1;
+    if (count == 0) continue;
+    ++kept;
+    max_w = (unsigned)count > max_w ? (unsigned)count : max_w;
+    inv_min_w = ~(unsigned)count > inv_min_w ? ~(unsigned)count : inv_min_w;
     int rest = r;
-    bool inside = true;
 #pragma unroll
     for (int k = kBoxMaxDims - 1; k >= 0; --k) {
       if (k < nd) {
         const int q = rest / d[k];
-        inside = inside && (rest - q * d[k]) < ext[k];
+        const int i1 = rest - q * d[k] + 1;
+        top[k] = i1 > top[k] ? i1 : top[k];
         rest = q;
       }
     }
-    bad |= (c[r] != (inside ? w : 0)) | (pf[r] != 1);
   }
   if (bad) s_bad = 1;
+  // folded over the wavefront first: a thousand lanes updating five LDS words one
+  // after the other took longer than the rest of the kernel
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    kept += (unsigned)__shfl_xor((int)kept, off, kWave);
+    const unsigned m1 = (unsigned)__shfl_xor((int)max_w, off, kWave);
+    const unsigned m2 = (unsigned)__shfl_xor((int)inv_min_w, off, kWave);
+    max_w = m1 > max_w ? m1 : max_w;
+    inv_min_w = m2 > inv_min_w ? m2 : inv_min_w;
+#pragma unroll
+    for (int k = 0; k < kBoxMaxDims; ++k) {
+      if (k < nd) {
+        const int o = __shfl_xor(top[k], off, kWave);
+        top[k] = o > top[k] ? o : top[k];
+      }
+    }
+  }
+  if ((t & (kWave - 1)) == 0 && kept) {
+    atomicAdd(&s_kept, kept);
+    atomicMax(&s_max_w, max_w);
+    atomicMax(&s_inv_min_w, inv_min_w);
+#pragma unroll
+    for (int k = 0; k < kBoxMaxDims; ++k) {
+      if (k < nd) atomicMax(&s_ext[k], top[k]);
+    }
+  }
   __syncthreads();
+  if (t == 0) {
+    unsigned long long volume = 1;
+#pragma unroll
+    for (int k = 0; k < kBoxMaxDims; ++k) {
+      if (k < nd) volume *= (unsigned)s_ext[k];
+    }
+    if (s_kept != 0 && (s_max_w != ~s_inv_min_w || volume != s_kept)) s_bad = 1;
+  }
+  __syncthreads();
+  // an empty box is described as all zeros (the extents are zero already when
+  // nothing is kept)
+  const int32_t w = (int32_t)s_max_w;
   if (stamp != 0) {
     // Every entry of the line travels with the call's stamp in the upper half of
     // one 8-byte word (a single store, atomic for whoever reads it): the host takes
