@@ -139,9 +139,7 @@ __global__ __launch_bounds__(kWave * kRowsPerBlock) void row_counts_kernel(
   }
 #pragma unroll
   for (int r = 0; r < NR; ++r) {
-    int c = count[r];
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) c += __shfl_xor(c, off, kWave);
+    const int c = wave_reduce_sum(count[r]);
     if (lane == 0) {
       s_count[wave * NR + r] = c;
       s_prefix[wave * NR + r] = is_prefix[r] ? 1 : 0;

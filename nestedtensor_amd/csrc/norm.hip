@@ -24,9 +24,7 @@ constexpr int kNormRowsPerBlock = 4;   // one wavefront each
 
 template <typename T>
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
-  return v;
+  return wave_reduce_sum(v);
 }
 
 // x (+ residual) of one 16-byte piece as floats
@@ -259,8 +257,7 @@ __device__ __forceinline__ void softmax_row(const T* __restrict__ src, T* __rest
 #pragma unroll
       for (int j = 0; j < V; ++j) m = fmaxf(m, v[k][j]);
     }
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, kWave));
+    m = wave_reduce_max(m);
     float s = 0.0f;
 #pragma unroll
     for (int k = 0; k < kCache; ++k) {
@@ -272,7 +269,7 @@ __device__ __forceinline__ void softmax_row(const T* __restrict__ src, T* __rest
         if (!LOG) v[k][j] = e;
       }
     }
-    s = wave_sum<T>(s);
+    s = wave_reduce_sum(s);
     const float inv = 1.0f / s, ls = logf(s);
 #pragma unroll
     for (int k = 0; k < kCache; ++k) {
@@ -301,8 +298,7 @@ __device__ __forceinline__ void softmax_row(const T* __restrict__ src, T* __rest
     for (int j = 0; j < V; ++j) m = fmaxf(m, (float)t[j]);
   }
   for (int64_t i = whole * V + lane; i < n; i += kWave) m = fmaxf(m, (float)src[i]);
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, kWave));
+  m = wave_reduce_max(m);
   float s = 0.0f;
   for (int64_t p = lane; p < whole; p += kWave) {
     T t[V];

@@ -79,4 +79,44 @@ __device__ __forceinline__ int64_t find_segment(const int64_t* offsets, int64_t 
   return lo;
 }
 
+// Reductions over the 64 lanes of a wavefront on the vector ALU's data-parallel
+// primitives: four shifted adds within each row of 16 lanes, then the row totals
+// are passed on to rows 1 and 3 and to rows 2 and 3 (row_bcast:15, row_bcast:31);
+// lane 63 holds the total and is read back as a scalar, so the result is uniform.
+// Seven vector instructions, against six LDS-crossbar permutes and their address
+// arithmetic for the same reduction written with __shfl_xor.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float old, float src) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, src),
+                                                               CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float wave_reduce_sum(float v) {
+  v += dpp_move<0x111, 0xf>(0.0f, v);   // row_shr:1
+  v += dpp_move<0x112, 0xf>(0.0f, v);   // row_shr:2
+  v += dpp_move<0x114, 0xf>(0.0f, v);   // row_shr:4
+  v += dpp_move<0x118, 0xf>(0.0f, v);   // row_shr:8
+  v += dpp_move<0x142, 0xa>(0.0f, v);   // row_bcast:15 into rows 1 and 3
+  v += dpp_move<0x143, 0xc>(0.0f, v);   // row_bcast:31 into rows 2 and 3
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+__device__ __forceinline__ int wave_reduce_sum(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);
+  return __builtin_amdgcn_readlane(v, 63);
+}
+__device__ __forceinline__ float wave_reduce_max(float v) {
+  const float lowest = -__builtin_inff();
+  v = fmaxf(v, dpp_move<0x111, 0xf>(lowest, v));
+  v = fmaxf(v, dpp_move<0x112, 0xf>(lowest, v));
+  v = fmaxf(v, dpp_move<0x114, 0xf>(lowest, v));
+  v = fmaxf(v, dpp_move<0x118, 0xf>(lowest, v));
+  v = fmaxf(v, dpp_move<0x142, 0xa>(lowest, v));
+  v = fmaxf(v, dpp_move<0x143, 0xc>(lowest, v));
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
 }  // namespace nt
